@@ -1,0 +1,131 @@
+/*
+ * geo_sc.h - C ABI of the MI355X (gfx950) stochastic-computing convolution library
+ * (libgeo_sc.so).
+ *
+ * The library implements, with hand-written HIP kernels, the one data-parallel path of
+ * nanocad-lab/geo: LFSR/comparator bit-stream generation, the SC convolution / grouped
+ * matmul forward with partial binary accumulation (OR inside a group, integer add across
+ * groups) and the surrogate-gradient backward.  No torch types cross this boundary: plain
+ * device pointers, sizes, a stream handle, int status codes.
+ *
+ * Tensor conventions are the reference's: weight (Cout, Cin, W, H) with W = dim 2 and
+ * H = dim 3, H being the dimension that is accumulated with binary adders; activation
+ * (N, Cin, Wx, Hx) dense NCHW fp32; output (N, Cout, Wo, Ho) int32 with
+ * Wo = Wx + 2*pad_w - W + 1 and Ho = Hx + 2*pad_h - H + 1.  Stride is 1 (the reference's
+ * native code accepts a stride and ignores it, sc.cpp:292, sc_cuda.cpp:47).
+ *
+ * All pointers are DEVICE pointers unless stated otherwise.  Every call enqueues work on
+ * `stream` and returns without synchronising; the caller owns all buffers.
+ */
+#ifndef GEO_SC_H
+#define GEO_SC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GEO_SC_VERSION 1
+
+/* A hipStream_t, passed as an opaque pointer so that C consumers need no HIP headers.
+ * NULL is the default stream. */
+typedef void* geo_sc_stream_t;
+
+enum geo_sc_status {
+    GEO_SC_OK = 0,
+    GEO_SC_ERR_INVALID_ARGUMENT = 1,   /* null pointer, non-positive size, kernel larger than input */
+    GEO_SC_ERR_BIT_LENGTH = 2,         /* stream length not in {8,16,32,64,128,256} */
+    GEO_SC_ERR_WORKSPACE = 3,          /* workspace pointer null / too small / misaligned */
+    GEO_SC_ERR_LAUNCH = 4,             /* a HIP call or kernel launch failed */
+    GEO_SC_ERR_UNSUPPORTED = 5         /* valid request the library does not implement */
+};
+
+/*
+ * Problem description shared by all entry points.
+ *
+ * Progressive loading (sc_cuda_kernel.cu:155-165, :681-688): at stream cycle b = 1..L the
+ * generators compare (code >> s) << s with s = total_width - min(total_width,
+ * (b / load_wait + 1) * load_width - 1).  load_width >= total_width + 1 disables it, which
+ * is what the reference CPU kernel computes; the reference's Python always passes
+ * total_width = 7 (utils_functional.py:28, :497).
+ */
+typedef struct geo_sc_conv_desc {
+    int32_t n;            /* batch */
+    int32_t c_in;
+    int32_t w_in;         /* activation dim 2, unpadded */
+    int32_t h_in;         /* activation dim 3, unpadded */
+    int32_t c_out;
+    int32_t w_k;          /* kernel dim 2: OR-accumulated together with c_in */
+    int32_t h_k;          /* kernel dim 3: binary-added */
+    int32_t pad_w;        /* zero padding of dim 2, both sides */
+    int32_t pad_h;        /* zero padding of dim 3, both sides */
+    int32_t bit_length;   /* stream length L: 8,16,32,64,128,256 */
+    int32_t total_width;  /* progressive loading, see above */
+    int32_t load_width;
+    int32_t load_wait_w;  /* load_wait of the weight generator */
+    int32_t load_wait_a;  /* load_wait of the activation generator */
+} geo_sc_conv_desc;
+
+/* Library version (GEO_SC_VERSION of the build). */
+int geo_sc_version(void);
+
+/* Static, human-readable text of a status code. */
+const char* geo_sc_status_string(int status);
+
+/*
+ * Bytes of device scratch the forward needs for `desc` (tables + bit-packed weight streams
+ * + bit-packed activation streams).  The reference allocates the same buffers itself with
+ * cudaMallocManaged on every call (sc_cuda_kernel.cu:1747-1796); here the caller brings
+ * them so that a framework allocator can be used.
+ */
+int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
+
+/*
+ * SC convolution forward with y-dimension (H) partial binary accumulation and LFSR stream
+ * generators:  float codes -> weight streams -> activation streams -> AND / OR / popcount.
+ *
+ * Replaces, behind one call:
+ *   sc_extension.conv2d_add_partial_new                       (sc.cpp:292-472)
+ *   sc_extension_cuda.conv2d_add_partial_variable_acc, dim!=0 (sc_cuda.cpp:47-63)
+ *     -> conv2d_add_partial_direct_variable_cuda               (sc_cuda_kernel.cu:1732-1834)
+ *     -> stream_generation_transpose_add_variable              (sc_cuda_kernel.cu:91-170)
+ *     -> stream_compute_add_direct_variable                    (sc_cuda_kernel.cu:590-1004)
+ *
+ * x: (n, c_in, w_in, h_in) fp32;  w: (c_out, c_in, w_k, h_k) fp32;
+ * y: (n, c_out, Wo, Ho) int32, fully overwritten.
+ * workspace: at least the size reported above, 256-byte aligned.
+ */
+int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
+                                      void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
+
+/*
+ * The two stream generators on their own (the forward runs exactly these kernels).
+ *
+ * Activation streams: uint32 [n][P][c_in][Wi][Hi] over the PADDED item, P = ceil(L/32);
+ * element i (flat index in the padded item) starts its LFSR at i % (L-1) + 1; the register
+ * advances before each comparison; bits enter MSB-first; for L < 32 a word holds L bits
+ * (sc.cpp:405-438, sc_cuda_kernel.cu:662-692).
+ *
+ * Weight streams: uint32 [P][h_k][c_in*w_k][ceil(c_out/16)][2][16]: for each pack, kernel
+ * row, OR-group member k = c_in_index*w_k + w_index and tile of 16 output channels, the 16
+ * positive-rail words followed by the 16 negative-rail words (zero for c_out padding).
+ * Seeds (67+k) % (L-1) + 1 / (37+k) % (L-1) + 1, one sequence per k shared by every h and
+ * c_out (sc.cpp:336-388, sc_cuda_kernel.cu:91-170).
+ *
+ * `tables` is scratch of geo_sc_stream_tables_size(L) bytes.
+ */
+int geo_sc_stream_tables_size(int bit_length, size_t* bytes);
+int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* streams, void* tables,
+                       geo_sc_stream_t stream);
+int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
+                          geo_sc_stream_t stream);
+/* Word counts of the two stream buffers above. */
+int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
+int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GEO_SC_H */
