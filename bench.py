@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the SC convolution hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--length 128]
+                    [--no-cpu-baseline]
+
+One step = one pass of the hot path over one batch of synthetic input that is already
+resident in HBM: float->code conversion, LFSR stream generation for weights and
+activations, the AND/OR/popcount convolution (and the surrogate backward once
+``--pass fwdbwd`` is supported by the build).  Prints ONE JSON line.
+
+The default workload is the configuration the headline metric is quoted on: SC conv2d
+128->128 3x3 at 16x16, batch 256, pad 1, stream length 128, activations U[0,1), weights
+U[-1,1) (with these distributions every OR rail saturates, so this input is for timing
+only; the kernels have no data-dependent early exit).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X nominal peaks used for the roofline fractions
+PEAK_VALU_WORD_OPS = 256 * 64 * 2.4e9   # CUs x lanes x clock: 32-bit VALU ops per second
+PEAK_HBM_BYTES = 8.0e12
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C3", choices=["C1", "C3", "C4", "C5"])
+    ap.add_argument("--length", type=int, default=0, help="stream length (default: the workload's)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def time_events(fn, steps, warmup, torch):
+    """Per-call durations (ms) measured with events on the stream fn launches on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in evs]
+
+
+def cpu_baseline(x, w, L, pad):
+    """The reference's own CPU kernel (compiled from its source into oracle/_ref) when it is
+    loadable here, else this repository's C restatement of it; timed on the host cores."""
+    import torch
+    from oracle import sc_oracle as so
+
+    threads = torch.get_num_threads()
+    ref = so.load_ref()
+    if ref is not None:
+        kind = "reference"
+
+        def run():
+            return ref.conv2d_add_partial_new(x, w, L, (pad, pad), (1, 1))
+        variant = so.ref_variants_usable()[0]
+        try:
+            threads = len(os.sched_getaffinity(0))
+        except AttributeError:
+            pass
+        threads = min(threads, so.max_threads())
+        note = f"sc.cpp compiled -O3 -fopenmp ({variant} path), OpenMP over batch"
+    else:
+        kind = "port"
+        threads = so.max_threads()
+        xn, wn = x.numpy(), w.numpy()
+
+        def run():
+            return so.conv2d_add_partial(xn, wn, L, (pad, pad), fast=True)
+        note = "C restatement (oracle/sc_oracle.c, fast loop order), OpenMP over batch"
+    run()  # warm-up
+    times = []
+    budget_start = time.time()
+    for _ in range(5):
+        t = time.time()
+        run()
+        times.append(time.time() - t)
+        if time.time() - budget_start > 25:
+            break
+    return kind, threads, statistics.median(times), note
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(the path shards over the batch with no communication in forward; nothing here uses a second GPU)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    from geo_amd import capi
+    from geo_amd import workloads as wl
+
+    sx, sw, pad, L0, vx, vw = wl.SHAPES[args.workload]
+    L = args.length or L0
+    x, w = wl.make_inputs(sx, sw, "prescribed", 0, vx, vw)
+    xd, wd = x.cuda(), w.cuda()
+    desc = capi.make_desc(xd.shape, wd.shape, L, (pad, pad))
+    ws = torch.empty(capi.workspace_size(desc), dtype=torch.uint8, device="cuda")
+    out = torch.empty(capi.output_shape(desc), dtype=torch.int32, device="cuda")
+
+    def step():
+        capi.conv2d_add_partial_forward(xd, wd, L, (pad, pad), out=out, workspace=ws, desc=desc)
+
+    # whole step: barrier-free on one GPU, synchronise both sides of the timed region
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    B = wl.bit_macs(xd.shape, wd.shape, pad, L)
+    value = B / (ms_per_step * 1e-3)
+
+    # dominant kernel alone (AND/OR/popcount on pre-generated streams), HIP events on its stream
+    act = capi.act_streams(xd, desc)
+    wgt = capi.weight_streams(wd, desc)
+    k_ms = time_events(lambda: capi.conv2d_add_partial_from_streams(act, wgt, desc, out=out), args.steps,
+                       args.warmup, torch)
+    k_avg = sum(k_ms) / len(k_ms)
+    word_ops = 2 * B / 32
+    achieved = word_ops / (k_avg * 1e-3)
+    gen_ms = time_events(lambda: (capi.act_streams(xd, desc), capi.weight_streams(wd, desc)), min(args.steps, 10),
+                         2, torch)
+    N, Cin, Wx, Hx = xd.shape
+    Cout, _, W, H = wd.shape
+    alg_bytes = 4 * (xd.numel() + wd.numel() + out.numel())
+    stream_bytes = 4 * (act.numel() + wgt.numel())
+
+    result = {
+        "metric": "SC bit-MACs/sec (whole forward op: codes + LFSR streams + AND/OR/popcount conv) at stream len "
+                  f"{L}",
+        "value": value,
+        "unit": "bit-MAC/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32 bit-packed streams, int32 accumulate",
+        "data": "synthetic (torch.manual_seed(0); activations U[0,1), weights U[-1,1))",
+        "config": {"workload": f"{args.workload}: SC conv2d {tuple(x.shape)} * {tuple(w.shape)} pad {pad}, "
+                               f"stream length {L}, y-dimension partial binary accumulation, LFSR generators",
+                   "pass": "fwd", "bit_macs_per_step": B},
+        "roofline": {
+            "bound": "valu",
+            "kernel": "k_conv_fwd (v_and_or_b32 / v_bcnt_u32_b32)",
+            "achieved": achieved / 1e12,
+            "peak": PEAK_VALU_WORD_OPS / 1e12,
+            "unit": "T word-op/s",
+            "frac": achieved / PEAK_VALU_WORD_OPS,
+            "kernel_ms_avg": k_avg,
+            "kernel_ms_min": min(k_ms),
+            "algorithmic_word_ops": word_ops,
+            "hbm_algorithmic_bytes": alg_bytes,
+            "hbm_stream_bytes_read_by_kernel": stream_bytes,
+            "hbm_frac_of_peak": (stream_bytes + 4 * out.numel()) / (k_avg * 1e-3) / PEAK_HBM_BYTES,
+            "traffic": None,
+        },
+        "stages_ms": {"stream_generation": sum(gen_ms) / len(gen_ms), "conv_kernel": k_avg},
+    }
+    if not args.no_cpu_baseline:
+        kind, cores, sec, note = cpu_baseline(x, w, L, pad)
+        result["cpu_baseline"] = {
+            "value": B / sec, "unit": "bit-MAC/s", "cores": cores, "kind": kind,
+            "sample": f"same workload, full batch, median of up to 5 runs after 1 warm-up ({sec:.3f} s/run); {note}",
+            "gpu_over_cpu": value / (B / sec),
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

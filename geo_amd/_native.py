@@ -1,0 +1,86 @@
+"""Loader of the native code built by ``python -m geo_amd.build``.
+
+Nothing here falls back to Python or CPU code: if a library is missing the import fails
+with the command that builds it.
+"""
+from __future__ import annotations
+
+import ctypes
+import importlib.util
+import os
+import sys
+import sysconfig
+
+import torch  # noqa: F401  loads the HIP runtime the libraries bind to
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIBDIR = os.path.join(HERE, "lib")
+_BUILD_HINT = "build the native code first: python -m geo_amd.build"
+
+
+class ConvDesc(ctypes.Structure):
+    """geo_sc_conv_desc of include/geo_sc.h"""
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "n", "c_in", "w_in", "h_in", "c_out", "w_k", "h_k", "pad_w", "pad_h", "bit_length",
+        "total_width", "load_width", "load_wait_w", "load_wait_a")]
+
+
+# every symbol include/geo_sc.h declares: name -> (restype, argtypes)
+_P = ctypes.c_void_p
+_SZ = ctypes.POINTER(ctypes.c_size_t)
+_D = ctypes.POINTER(ConvDesc)
+C_API = {
+    "geo_sc_version": (ctypes.c_int, []),
+    "geo_sc_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "geo_sc_conv2d_add_partial_workspace_size": (ctypes.c_int, [_D, _SZ]),
+    "geo_sc_conv2d_add_partial_forward": (ctypes.c_int, [_D, _P, _P, _P, _P, ctypes.c_size_t, _P]),
+    "geo_sc_conv2d_add_partial_from_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
+    "geo_sc_stream_tables_size": (ctypes.c_int, [ctypes.c_int, _SZ]),
+    "geo_sc_act_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
+    "geo_sc_weight_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
+    "geo_sc_act_stream_words": (ctypes.c_int, [_D, _SZ]),
+    "geo_sc_weight_stream_words": (ctypes.c_int, [_D, _SZ]),
+}
+
+_lib = None
+_modules = {}
+
+
+def lib_path() -> str:
+    return os.path.join(LIBDIR, "libgeo_sc.so")
+
+
+def lib() -> ctypes.CDLL:
+    """libgeo_sc.so with argument types set."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.isfile(path):
+            raise ImportError(f"{path} not found; {_BUILD_HINT}")
+        L = ctypes.CDLL(path)
+        for name, (res, args) in C_API.items():
+            fn = getattr(L, name)  # AttributeError if the library lacks a declared symbol
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def module(name: str):
+    """The PyTorch extension module ``sc_extension_cuda`` or ``sc_extension``."""
+    if name not in _modules:
+        path = os.path.join(LIBDIR, name + sysconfig.get_config_var("EXT_SUFFIX"))
+        if not os.path.isfile(path):
+            raise ImportError(f"{path} not found; {_BUILD_HINT}")
+        spec = importlib.util.spec_from_file_location(name, path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _modules[name] = mod
+    return _modules[name]
+
+
+def register_reference_module_names():
+    """Make ``import sc_extension`` / ``import sc_extension_cuda`` resolve to this build, the
+    way the reference's utils_functional.py imports them (utils_functional.py:11-12)."""
+    for name in ("sc_extension", "sc_extension_cuda"):
+        sys.modules[name] = module(name)

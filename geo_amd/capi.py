@@ -1,0 +1,131 @@
+"""Python callers of the C ABI in ``include/geo_sc.h`` (ctypes, raw device pointers).
+
+torch is used for device memory and the current stream only; every function below is one
+C call.  These are what the GPU parity tests and the benchmark drive.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _native
+from ._native import ConvDesc
+
+NEUTRAL_LOADING = dict(total_width=7, load_width=8, load_wait_w=1, load_wait_a=1)
+
+
+class GeoScError(RuntimeError):
+    def __init__(self, status: int, what: str):
+        self.status = status
+        text = _native.lib().geo_sc_status_string(status).decode()
+        super().__init__(f"{what}: {text} (status {status})")
+
+
+def _check(status: int, what: str):
+    if status != 0:
+        raise GeoScError(status, what)
+
+
+def make_desc(x_shape, w_shape, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
+              load_wait_a=1) -> ConvDesc:
+    """``padding=(p0, p1)`` follows the reference: p0 pads the last dim, p1 the one before."""
+    n, c_in, w_in, h_in = (int(v) for v in x_shape)
+    c_out, c_in2, w_k, h_k = (int(v) for v in w_shape)
+    if c_in != c_in2:
+        raise ValueError(f"channel mismatch: {c_in} vs {c_in2}")
+    return ConvDesc(n, c_in, w_in, h_in, c_out, w_k, h_k, int(padding[1]), int(padding[0]), int(bit_length),
+                    int(total_width), int(load_width), int(load_wait_w), int(load_wait_a))
+
+
+def _stream_ptr(stream=None):
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def version() -> int:
+    return _native.lib().geo_sc_version()
+
+
+def workspace_size(desc: ConvDesc) -> int:
+    out = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_conv2d_add_partial_workspace_size(ctypes.byref(desc), ctypes.byref(out)),
+           "workspace query")
+    return out.value
+
+
+def output_shape(desc: ConvDesc):
+    return (desc.n, desc.c_out, desc.w_in + 2 * desc.pad_w - desc.w_k + 1, desc.h_in + 2 * desc.pad_h - desc.h_k + 1)
+
+
+def _require_gpu_f32(t, name):
+    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+        raise ValueError(f"{name} must be a contiguous float32 GPU tensor")
+
+
+def conv2d_add_partial_forward(x, w, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
+                               load_wait_a=1, out=None, workspace=None, stream=None, desc=None):
+    """int32 (N, Cout, Wo, Ho) GPU tensor via geo_sc_conv2d_add_partial_forward."""
+    _require_gpu_f32(x, "x")
+    _require_gpu_f32(w, "w")
+    if desc is None:
+        desc = make_desc(x.shape, w.shape, bit_length, padding, total_width, load_width, load_wait_w, load_wait_a)
+    ws_bytes = workspace_size(desc)
+    if workspace is None:
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty(output_shape(desc), dtype=torch.int32, device=x.device)
+    _check(_native.lib().geo_sc_conv2d_add_partial_forward(ctypes.byref(desc), _ptr(x), _ptr(w), _ptr(out),
+                                                           _ptr(workspace), workspace.numel(), _stream_ptr(stream)),
+           "geo_sc_conv2d_add_partial_forward")
+    return out
+
+
+def _tables(bit_length, device):
+    n = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_stream_tables_size(int(bit_length), ctypes.byref(n)), "tables size")
+    return torch.empty(n.value, dtype=torch.uint8, device=device)
+
+
+def act_streams(x, desc: ConvDesc, stream=None):
+    """int32-typed tensor of stream words [N][P][Cin][Wi][Hi] (reinterpret as uint32)."""
+    _require_gpu_f32(x, "x")
+    n = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_act_stream_words(ctypes.byref(desc), ctypes.byref(n)), "act words")
+    packs = (desc.bit_length + 31) // 32
+    wi, hi = desc.w_in + 2 * desc.pad_w, desc.h_in + 2 * desc.pad_h
+    out = torch.empty((desc.n, packs, desc.c_in, wi, hi), dtype=torch.int32, device=x.device)
+    assert out.numel() == n.value
+    tables = _tables(desc.bit_length, x.device)
+    _check(_native.lib().geo_sc_act_streams(ctypes.byref(desc), _ptr(x), _ptr(out), _ptr(tables),
+                                            _stream_ptr(stream)), "geo_sc_act_streams")
+    return out
+
+
+def weight_streams(w, desc: ConvDesc, stream=None):
+    """int32-typed tensor of stream words [P][H][Cin*W][ceil(Cout/16)][2][16]."""
+    _require_gpu_f32(w, "w")
+    n = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
+    packs = (desc.bit_length + 31) // 32
+    out = torch.empty((packs, desc.h_k, desc.c_in * desc.w_k, (desc.c_out + 15) // 16, 2, 16), dtype=torch.int32,
+                      device=w.device)
+    assert out.numel() == n.value
+    tables = _tables(desc.bit_length, w.device)
+    _check(_native.lib().geo_sc_weight_streams(ctypes.byref(desc), _ptr(w), _ptr(out), _ptr(tables),
+                                               _stream_ptr(stream)), "geo_sc_weight_streams")
+    return out
+
+
+def conv2d_add_partial_from_streams(act, wgt, desc: ConvDesc, out=None, stream=None):
+    """The AND/OR/popcount kernel alone on pre-generated streams (int32-typed words)."""
+    if out is None:
+        out = torch.empty(output_shape(desc), dtype=torch.int32, device=act.device)
+    _check(_native.lib().geo_sc_conv2d_add_partial_from_streams(ctypes.byref(desc), _ptr(act), _ptr(wgt), _ptr(out),
+                                                                _stream_ptr(stream)),
+           "geo_sc_conv2d_add_partial_from_streams")
+    return out

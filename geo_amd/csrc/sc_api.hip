@@ -1,0 +1,187 @@
+// C ABI of libgeo_sc.so: argument validation, workspace carve-up, kernel sequencing.
+#include "sc_common.h"
+
+namespace geo_sc {
+
+namespace {
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+}  // namespace
+
+int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
+{
+    if (!d || !g) return GEO_SC_ERR_INVALID_ARGUMENT;
+    int n_bits;
+    switch (d->bit_length) {
+    case 8: n_bits = 3; break;
+    case 16: n_bits = 4; break;
+    case 32: n_bits = 5; break;
+    case 64: n_bits = 6; break;
+    case 128: n_bits = 7; break;
+    case 256: n_bits = 8; break;
+    default: return GEO_SC_ERR_BIT_LENGTH;
+    }
+    if (d->n < 1 || d->c_in < 1 || d->w_in < 1 || d->h_in < 1 || d->c_out < 1 || d->w_k < 1 || d->h_k < 1 ||
+        d->pad_w < 0 || d->pad_h < 0)
+        return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (d->total_width < 0 || d->total_width > 30 || d->load_width < 1 || d->load_wait_w < 1 || d->load_wait_a < 1)
+        return GEO_SC_ERR_INVALID_ARGUMENT;
+    g->n = d->n;
+    g->c_in = d->c_in;
+    g->w_in = d->w_in;
+    g->h_in = d->h_in;
+    g->c_out = d->c_out;
+    g->w_k = d->w_k;
+    g->h_k = d->h_k;
+    g->pad_w = d->pad_w;
+    g->pad_h = d->pad_h;
+    g->L = d->bit_length;
+    g->n_bits = n_bits;
+    g->packs = (g->L + 31) / 32;
+    g->bit_unit = g->L < 32 ? g->L : 32;
+    g->total_width = d->total_width;
+    // any load_width above total_width+1 behaves like total_width+1; clamp so that the
+    // products in the kernels cannot overflow
+    g->load_width = d->load_width > g->total_width + 1 ? g->total_width + 1 : d->load_width;
+    g->load_wait_w = d->load_wait_w;
+    g->load_wait_a = d->load_wait_a;
+    const long long wi = (long long)d->w_in + 2LL * d->pad_w, hi = (long long)d->h_in + 2LL * d->pad_h;
+    const long long wo = wi - d->w_k + 1, ho = hi - d->h_k + 1;
+    if (wo < 1 || ho < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const long long plane = (long long)d->c_in * wi * hi;
+    const long long k_or = (long long)d->c_in * d->w_k;
+    if (plane > 0x7fffffffLL || k_or > 0x7fffffffLL || (long long)d->c_out * wo * ho > 0x7fffffffLL)
+        return GEO_SC_ERR_INVALID_ARGUMENT;
+    g->wi = (int)wi;
+    g->hi = (int)hi;
+    g->wo = (int)wo;
+    g->ho = (int)ho;
+    g->k_or = (int)k_or;
+    g->n_cotile = (d->c_out + kCoTile - 1) / kCoTile;
+    g->act_plane = (size_t)plane;
+    g->act_words = (size_t)d->n * g->packs * g->act_plane;
+    g->wgt_words = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile * 2 * kCoTile;
+    g->off_tables = 0;
+    g->off_wgt = align256(table_bytes(g->L));
+    g->off_act = g->off_wgt + align256(g->wgt_words * sizeof(uint32_t));
+    g->ws_bytes = g->off_act + align256(g->act_words * sizeof(uint32_t));
+    return GEO_SC_OK;
+}
+
+}  // namespace geo_sc
+
+using namespace geo_sc;
+
+extern "C" {
+
+int geo_sc_version(void) { return GEO_SC_VERSION; }
+
+const char* geo_sc_status_string(int status)
+{
+    switch (status) {
+    case GEO_SC_OK: return "ok";
+    case GEO_SC_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case GEO_SC_ERR_BIT_LENGTH: return "stream length must be one of 8, 16, 32, 64, 128, 256";
+    case GEO_SC_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
+    case GEO_SC_ERR_LAUNCH: return "HIP launch failed";
+    case GEO_SC_ERR_UNSUPPORTED: return "not implemented";
+    default: return "unknown status";
+    }
+}
+
+int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes)
+{
+    Geometry g;
+    if (!bytes) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    *bytes = g.ws_bytes;
+    return GEO_SC_OK;
+}
+
+int geo_sc_stream_tables_size(int bit_length, size_t* bytes)
+{
+    if (!bytes) return GEO_SC_ERR_INVALID_ARGUMENT;
+    switch (bit_length) {
+    case 8: case 16: case 32: case 64: case 128: case 256: break;
+    default: return GEO_SC_ERR_BIT_LENGTH;
+    }
+    *bytes = table_bytes(bit_length);
+    return GEO_SC_OK;
+}
+
+int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words)
+{
+    Geometry g;
+    if (!words) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    *words = g.act_words;
+    return GEO_SC_OK;
+}
+
+int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words)
+{
+    Geometry g;
+    if (!words) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    *words = g.wgt_words;
+    return GEO_SC_OK;
+}
+
+int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* streams, void* tables,
+                       geo_sc_stream_t stream)
+{
+    Geometry g;
+    int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!x || !streams || !tables) return GEO_SC_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    rc = launch_build_tables(g, (uint32_t*)tables, s);
+    if (rc != GEO_SC_OK) return rc;
+    return launch_act_streams(g, x, streams, (const uint32_t*)tables, s);
+}
+
+int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
+                          geo_sc_stream_t stream)
+{
+    Geometry g;
+    int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!w || !streams || !tables) return GEO_SC_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    rc = launch_build_tables(g, (uint32_t*)tables, s);
+    if (rc != GEO_SC_OK) return rc;
+    return launch_weight_streams(g, w, streams, (const uint32_t*)tables, s);
+}
+
+int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,
+                                           const uint32_t* weight_streams, int32_t* y, geo_sc_stream_t stream)
+{
+    Geometry g;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!act_streams || !weight_streams || !y) return GEO_SC_ERR_INVALID_ARGUMENT;
+    return launch_conv_forward(g, act_streams, weight_streams, y, (hipStream_t)stream);
+}
+
+int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
+                                      void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    Geometry g;
+    int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!x || !w || !y) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (!workspace || workspace_bytes < g.ws_bytes || ((uintptr_t)workspace & 255u)) return GEO_SC_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    uint32_t* tables = (uint32_t*)(ws + g.off_tables);
+    uint32_t* wgt = (uint32_t*)(ws + g.off_wgt);
+    uint32_t* act = (uint32_t*)(ws + g.off_act);
+    if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
+    if ((rc = launch_weight_streams(g, w, wgt, tables, s)) != GEO_SC_OK) return rc;
+    if ((rc = launch_act_streams(g, x, act, tables, s)) != GEO_SC_OK) return rc;
+    return launch_conv_forward(g, act, wgt, y, s);
+}
+
+}  // extern "C"

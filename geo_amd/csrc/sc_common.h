@@ -1,0 +1,52 @@
+// Shared host/device definitions of the SC convolution kernels (gfx950).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "geo_sc.h"
+
+namespace geo_sc {
+
+// Output channels per weight tile: one tile = 16 positive-rail words + 16 negative-rail
+// words = one 128-byte line, fetched by a wave as two scalar 16-dword loads.
+constexpr int kCoTile = 16;
+
+// Derived sizes of one problem; filled by make_geometry() after validation.
+struct Geometry {
+    int n, c_in, w_in, h_in, c_out, w_k, h_k, pad_w, pad_h;
+    int L, n_bits, packs, bit_unit;
+    int total_width, load_width, load_wait_w, load_wait_a;
+    int wi, hi;          // padded activation dims 2 / 3
+    int wo, ho;          // output dims 2 / 3
+    int k_or;            // OR-group size c_in * w_k
+    int n_cotile;        // ceil(c_out / kCoTile)
+    size_t act_plane;    // c_in * wi * hi words: one pack of one item
+    size_t act_words;    // n * packs * act_plane
+    size_t wgt_words;    // packs * h_k * k_or * n_cotile * 2 * kCoTile
+    // workspace carve-up (byte offsets, 256-aligned)
+    size_t off_tables, off_wgt, off_act, ws_bytes;
+};
+
+// Stream tables (device memory, built per call):
+//   posp1[r], r < L-1 : 1 + index in the LFSR cycle of state r+1  (cycle[0] = 1)
+//   thr[code][j]      : bit string, MSB-first, of [code > cycle[j mod (L-1)]] for
+//                       j < 32 * words_per_code, long enough to read L bits from any
+//                       offset <= L-1 plus one spare word for the funnel shift.
+inline __host__ __device__ int table_words_per_code(int L) { return (2 * L + 31) / 32 + 2; }
+inline __host__ __device__ size_t table_bytes(int L)
+{
+    return sizeof(uint32_t) * ((size_t)L + (size_t)L * table_words_per_code(L));
+}
+
+int make_geometry(const geo_sc_conv_desc* d, Geometry* g);
+
+// launchers (each returns a geo_sc_status)
+int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s);
+int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s);
+int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
+                          hipStream_t s);
+int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
+
+}  // namespace geo_sc

@@ -1,0 +1,240 @@
+// LFSR / comparator stream generation for gfx950.
+//
+// A stream bit is [code > state], the register being advanced before each comparison
+// (sc.cpp:365-378, :429-432).  All six registers are maximal, so the states an element
+// sees are one fixed cycle of period L-1 entered at an offset that depends on its seed
+// only.  Instead of stepping a register L times per element, a per-call table holds, for
+// every code, the comparison results along that cycle as a bit string; an element's P
+// stream words are then P funnel shifts out of the string at its seed's offset.  The few
+// leading cycles that progressive loading alters are patched bit by bit from the same
+// table.
+#include "sc_common.h"
+
+namespace geo_sc {
+
+namespace {
+
+constexpr int kGenThreads = 256;
+
+__device__ __forceinline__ uint32_t lfsr_step(uint32_t s, uint32_t tap_mask, uint32_t state_mask)
+{
+    // Fibonacci LFSR: shift left, feed back the parity of the tapped bits.
+    // taps (bit indices): 3:{2,1} 4:{3,2} 5:{4,2} 6:{5,4} 7:{6,5} 8:{7,5,4,3}  (sc.cpp:262-290)
+    return ((s << 1) & state_mask) | (__popc(s & tap_mask) & 1u);
+}
+
+__host__ __device__ inline uint32_t tap_mask_for(int n_bits)
+{
+    switch (n_bits) {
+    case 3: return 0x06u;
+    case 4: return 0x0Cu;
+    case 5: return 0x14u;
+    case 6: return 0x30u;
+    case 7: return 0x60u;
+    default: return 0xB8u;
+    }
+}
+
+// One block.  tables = posp1[L] (entry L-1 unused) followed by thr[L][wpc].
+__global__ __launch_bounds__(kGenThreads) void k_build_tables(uint32_t* __restrict__ tables, int L, int n_bits)
+{
+    __shared__ uint16_t cyc[256];
+    const int period = L - 1;
+    if (threadIdx.x == 0) {
+        uint32_t s = 1;
+        const uint32_t tm = tap_mask_for(n_bits), sm = (uint32_t)L - 1u;
+        for (int j = 0; j < period; j++) {
+            cyc[j] = (uint16_t)s;
+            s = lfsr_step(s, tm, sm);
+        }
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < period; j += kGenThreads) tables[cyc[j] - 1] = (uint32_t)(j + 1);
+    if (threadIdx.x == 0) tables[L - 1] = 0;
+    const int wpc = table_words_per_code(L);
+    uint32_t* thr = tables + L;
+    for (int idx = threadIdx.x; idx < L * wpc; idx += kGenThreads) {
+        const int code = idx / wpc, wi = idx % wpc;
+        int j = (wi * 32) % period;
+        uint32_t word = 0;
+        for (int b = 0; b < 32; b++) {
+            word = (word << 1) | (uint32_t)(code > (int)cyc[j]);
+            j = (j + 1 == period) ? 0 : j + 1;
+        }
+        thr[idx] = word;
+    }
+}
+
+struct GenParams {
+    int L, packs, bit_unit, wpc;
+    int total_width, load_width, load_wait;
+    int ramp;  // leading cycles whose compared code is masked by progressive loading
+};
+
+__device__ __forceinline__ int loaded_code(int code, int cycle, const GenParams& gp)
+{
+    // sc_cuda_kernel.cu:156-160 / :682-685
+    int cw = (cycle / gp.load_wait + 1) * gp.load_width - 1;
+    cw = cw > gp.total_width ? gp.total_width : cw;
+    const int sh = gp.total_width - cw;
+    return (code >> sh) << sh;
+}
+
+// Stream word `p` of (code, cycle offset o); thr_lds = table in LDS.
+__device__ __forceinline__ uint32_t stream_word(const uint32_t* thr_lds, int code, int o, int p, const GenParams& gp)
+{
+    const uint32_t* row = thr_lds + code * gp.wpc;
+    const int start = o + p * gp.bit_unit;
+    const uint32_t hi = row[start >> 5], lo = row[(start >> 5) + 1];
+    const uint64_t both = ((uint64_t)hi << 32) | lo;
+    uint32_t word = (uint32_t)((both << (start & 31)) >> 32) >> (32 - gp.bit_unit);
+    int nb = gp.ramp - p * gp.bit_unit;
+    nb = nb > gp.bit_unit ? gp.bit_unit : nb;
+    for (int b = 0; b < nb; b++) {
+        const int t = p * gp.bit_unit + b;
+        const int c2 = loaded_code(code, t + 1, gp);
+        const int j = o + t;
+        const uint32_t bit = (thr_lds[c2 * gp.wpc + (j >> 5)] >> (31 - (j & 31))) & 1u;
+        const uint32_t m = 1u << (gp.bit_unit - 1 - b);
+        word = (word & ~m) | (bit ? m : 0u);
+    }
+    return word;
+}
+
+__device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, const uint32_t* __restrict__ tables, int L, int wpc)
+{
+    const int n = L + L * wpc;
+    for (int i = threadIdx.x; i < n; i += kGenThreads) lds[i] = tables[i];
+    __syncthreads();
+}
+
+// Activation streams [n][P][c_in][Wi][Hi] from the unpadded fp32 input; padding positions
+// produce zero words but keep their place in the seed numbering (sc.cpp:409-413).
+__global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __restrict__ x,
+                                                            uint32_t* __restrict__ streams,
+                                                            const uint32_t* __restrict__ tables, GenParams gp, int n,
+                                                            int c_in, int w_in, int h_in, int pad_w, int pad_h)
+{
+    extern __shared__ uint32_t lds[];
+    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    const uint32_t* posp1 = lds;
+    const uint32_t* thr = lds + gp.L;
+    const int wi = w_in + 2 * pad_w, hi = h_in + 2 * pad_h;
+    const uint32_t plane = (uint32_t)c_in * wi * hi;
+    const size_t total = (size_t)n * plane;
+    const float Lf = (float)gp.L, top = (float)(gp.L - 1);
+    for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
+        const uint32_t item = (uint32_t)(e / plane);
+        const uint32_t i = (uint32_t)(e - (size_t)item * plane);
+        const uint32_t q = i % (uint32_t)hi;
+        const uint32_t r = i / (uint32_t)hi;
+        const uint32_t p = r % (uint32_t)wi;
+        const uint32_t c = r / (uint32_t)wi;
+        const int ps = (int)p - pad_w, qs = (int)q - pad_h;
+        int code = 0;
+        if (ps >= 0 && ps < w_in && qs >= 0 && qs < h_in) {
+            const float v = x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs];
+            // ceil(clamp(x*L, 0, L-1))  (sc.cpp:301)
+            code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
+        }
+        const int o = (int)posp1[i % (uint32_t)(gp.L - 1)];
+        uint32_t* dst = streams + (size_t)item * gp.packs * plane + i;
+        for (int pk = 0; pk < gp.packs; pk++) dst[(size_t)pk * plane] = code ? stream_word(thr, code, o, pk, gp) : 0u;
+    }
+}
+
+// Weight streams, tiled layout [P][h_k][k][cotile][rail][16]; one thread per
+// (h, k, padded c_out), c_out fastest so that a wave writes whole tiles.
+__global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __restrict__ w,
+                                                               uint32_t* __restrict__ streams,
+                                                               const uint32_t* __restrict__ tables, GenParams gp,
+                                                               int c_out, int c_in, int w_k, int h_k, int n_cotile)
+{
+    extern __shared__ uint32_t lds[];
+    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    const uint32_t* posp1 = lds;
+    const uint32_t* thr = lds + gp.L;
+    const int k_or = c_in * w_k;
+    const int co_pad = n_cotile * kCoTile;
+    const size_t total = (size_t)h_k * k_or * co_pad;
+    const size_t pack_stride = (size_t)h_k * k_or * n_cotile * 2 * kCoTile;
+    const float Lf = (float)gp.L, top = (float)(gp.L - 1);
+    for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
+        const int co = (int)(e % co_pad);
+        const size_t r = e / co_pad;
+        const int k = (int)(r % k_or);
+        const int v = (int)(r / k_or);
+        const int ci = k / w_k, u = k % w_k;
+        int cp = 0, cn = 0;
+        if (co < c_out) {
+            const float wv = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v];
+            const float t = wv * Lf;
+            cp = (int)ceilf(fminf(fmaxf(t, 0.0f), top));    // sc.cpp:303
+            cn = (int)ceilf(-fminf(fmaxf(t, -top), 0.0f));  // sc.cpp:304
+        }
+        const int op = (int)posp1[(67 + k) % (gp.L - 1)];  // sc.cpp:345
+        const int on = (int)posp1[(37 + k) % (gp.L - 1)];  // sc.cpp:346
+        const size_t base = (((size_t)v * k_or + k) * n_cotile + co / kCoTile) * (2 * kCoTile) + (co % kCoTile);
+        for (int pk = 0; pk < gp.packs; pk++) {
+            streams[pk * pack_stride + base] = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
+            streams[pk * pack_stride + base + kCoTile] = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+        }
+    }
+}
+
+GenParams gen_params(const Geometry& g, int load_wait)
+{
+    GenParams gp;
+    gp.L = g.L;
+    gp.packs = g.packs;
+    gp.bit_unit = g.bit_unit;
+    gp.wpc = table_words_per_code(g.L);
+    gp.total_width = g.total_width;
+    gp.load_width = g.load_width;
+    gp.load_wait = load_wait;
+    // cycles b = 1 .. m*wait-1 compare a masked code, m = ceil((tw+1)/lw) - 1
+    const long long m = (g.total_width + 1 + g.load_width - 1) / g.load_width - 1;
+    long long ramp = m * (long long)load_wait - 1;
+    if (ramp < 0) ramp = 0;
+    if (ramp > g.L) ramp = g.L;
+    gp.ramp = (int)ramp;
+    return gp;
+}
+
+int grid_for(size_t total)
+{
+    size_t blocks = (total + kGenThreads - 1) / kGenThreads;
+    const size_t cap = 256 * 16;  // 256 CUs, a few blocks each; the kernels grid-stride
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (int)blocks;
+}
+
+}  // namespace
+
+int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s)
+{
+    hipLaunchKernelGGL(k_build_tables, dim3(1), dim3(kGenThreads), 0, s, tables, g.L, g.n_bits);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s)
+{
+    const GenParams gp = gen_params(g, g.load_wait_a);
+    const size_t total = (size_t)g.n * g.act_plane;
+    hipLaunchKernelGGL(k_act_streams, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x, streams,
+                       tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
+                          hipStream_t s)
+{
+    const GenParams gp = gen_params(g, g.load_wait_w);
+    const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
+    hipLaunchKernelGGL(k_weight_streams, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, w, streams,
+                       tables, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+}  // namespace geo_sc

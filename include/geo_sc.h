@@ -28,6 +28,7 @@ extern "C" {
 #endif
 
 #define GEO_SC_VERSION 1
+#define GEO_SC_API __attribute__((visibility("default")))
 
 /* A hipStream_t, passed as an opaque pointer so that C consumers need no HIP headers.
  * NULL is the default stream. */
@@ -69,10 +70,10 @@ typedef struct geo_sc_conv_desc {
 } geo_sc_conv_desc;
 
 /* Library version (GEO_SC_VERSION of the build). */
-int geo_sc_version(void);
+GEO_SC_API int geo_sc_version(void);
 
 /* Static, human-readable text of a status code. */
-const char* geo_sc_status_string(int status);
+GEO_SC_API const char* geo_sc_status_string(int status);
 
 /*
  * Bytes of device scratch the forward needs for `desc` (tables + bit-packed weight streams
@@ -80,7 +81,7 @@ const char* geo_sc_status_string(int status);
  * cudaMallocManaged on every call (sc_cuda_kernel.cu:1747-1796); here the caller brings
  * them so that a framework allocator can be used.
  */
-int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
+GEO_SC_API int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
 
 /*
  * SC convolution forward with y-dimension (H) partial binary accumulation and LFSR stream
@@ -97,7 +98,7 @@ int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_
  * y: (n, c_out, Wo, Ho) int32, fully overwritten.
  * workspace: at least the size reported above, 256-byte aligned.
  */
-int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
+GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
                                       void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
 
 /*
@@ -116,14 +117,22 @@ int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float*
  *
  * `tables` is scratch of geo_sc_stream_tables_size(L) bytes.
  */
-int geo_sc_stream_tables_size(int bit_length, size_t* bytes);
-int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* streams, void* tables,
+GEO_SC_API int geo_sc_stream_tables_size(int bit_length, size_t* bytes);
+GEO_SC_API int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* streams, void* tables,
                        geo_sc_stream_t stream);
-int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
+GEO_SC_API int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
                           geo_sc_stream_t stream);
+/*
+ * The AND / OR / popcount kernel alone, on streams in the two layouts above (what the
+ * forward runs after its generators; the body of stream_compute_add_direct_variable,
+ * sc_cuda_kernel.cu:693-1002, and of matmul_outer, sc.cpp:12-259).  y is fully overwritten.
+ */
+GEO_SC_API int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,
+                                                      const uint32_t* weight_streams, int32_t* y,
+                                                      geo_sc_stream_t stream);
 /* Word counts of the two stream buffers above. */
-int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
-int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);
+GEO_SC_API int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
+GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,218 @@
+"""GPU parity of the HIP forward path, driven through the C ABI (geo_amd.capi) and through
+the PyTorch modules with the reference's names.  Everything is compared bit-for-bit with
+the CPU oracle, the reference-kernel fixtures and the reference-kernel checksums."""
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+from geo_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = (8, 16, 32, 64, 128, 256)
+
+
+@pytest.fixture(scope="module")
+def capi():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from geo_amd import capi as m
+    return m
+
+
+@pytest.fixture(scope="module")
+def so():
+    from oracle import sc_oracle
+    return sc_oracle
+
+
+def gpu_forward(capi, x, w, L, pad, **kw):
+    if isinstance(pad, int):
+        pad = (pad, pad)
+    xd = torch.as_tensor(x).float().contiguous().cuda()
+    wd = torch.as_tensor(w).float().contiguous().cuda()
+    y = capi.conv2d_add_partial_forward(xd, wd, L, pad, **kw)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def u32(t):
+    return t.cpu().numpy().view(np.uint32)
+
+
+# ------------------------------------------------------------------ stream generators
+@pytest.mark.parametrize("L", LENGTHS)
+@pytest.mark.parametrize("loading", [(7, 8, 1, 1), (7, 2, 2, 2), (7, 1, 3, 5), (7, 3, 40, 7)])
+def test_activation_streams_match_oracle(capi, so, L, loading):
+    tw, lw, ww, wa = loading
+    x, _ = wl.make_inputs((3, 5, 7, 6), (2, 5, 3, 3), "prescribed", seed=L)
+    x.view(-1)[::13] = 0.0
+    x.view(-1)[5::17] = 1.0
+    d = capi.make_desc(x.shape, (2, 5, 3, 3), L, (2, 1), tw, lw, ww, wa)
+    got = u32(capi.act_streams(x.cuda(), d))
+    xp = np.pad(x.numpy(), ((0, 0), (0, 0), (1, 1), (2, 2)))
+    for n in range(x.shape[0]):
+        exp = so.act_streams(xp[n], L, tw, lw, wa)
+        assert np.array_equal(got[n], exp), (L, loading, n)
+
+
+@pytest.mark.parametrize("L", LENGTHS)
+@pytest.mark.parametrize("loading", [(7, 8, 1, 1), (7, 2, 2, 2), (7, 1, 3, 5)])
+def test_weight_streams_match_oracle(capi, so, L, loading):
+    tw, lw, ww, wa = loading
+    _, w = wl.make_inputs((1, 6, 4, 4), (19, 6, 3, 2), "prescribed", seed=100 + L)
+    w.view(-1)[::7] = 0.0
+    d = capi.make_desc((1, 6, 4, 4), w.shape, L, (0, 0), tw, lw, ww, wa)
+    got = u32(capi.weight_streams(w.cuda(), d))          # [P][H][K][cot][2][16]
+    wpos, wneg = so.weight_streams(w.numpy(), L, tw, lw, ww)  # [P][H][Cin][W][Cout]
+    P, H, Cin, W, Cout = wpos.shape
+    got = got.reshape(P, H, Cin, W, -1, 2, 16)
+    gp = got[..., 0, :].reshape(P, H, Cin, W, -1)
+    gn = got[..., 1, :].reshape(P, H, Cin, W, -1)
+    assert np.array_equal(gp[..., :Cout], wpos)
+    assert np.array_equal(gn[..., :Cout], wneg)
+    assert not gp[..., Cout:].any() and not gn[..., Cout:].any()   # c_out padding is zero
+
+
+# ------------------------------------------------------------------ forward: fixtures
+def test_forward_matches_reference_fixtures(capi, fixtures_small):
+    for name, d in fixtures_small.items():
+        y = gpu_forward(capi, d["x"], d["w"], d["L"], d["pad"])
+        assert y.dtype == np.int32 and y.shape == d["y"].shape
+        assert np.array_equal(y, d["y"]), name
+
+
+@pytest.mark.parametrize("shape_x,shape_w,pad,L,mode", [
+    ((3, 5, 9, 7), (6, 5, 3, 3), (1, 1), 64, "prescribed"),
+    ((2, 4, 8, 8), (17, 4, 5, 5), (2, 2), 32, "prescribed"),     # two c_out tiles, one partial
+    ((2, 3, 7, 9), (5, 3, 1, 1), (0, 0), 128, "kaiming"),        # 1x1
+    ((2, 6, 5, 8), (4, 6, 2, 4), (1, 0), 256, "prescribed"),     # even kernel, asymmetric pad
+    ((1, 2, 9, 9), (3, 2, 7, 7), (3, 3), 16, "prescribed"),      # run-time kernel width
+    ((5, 16, 1, 8), (33, 16, 1, 8), (0, 0), 128, "prescribed"),  # SC-linear mapping
+    ((2, 3, 11, 5), (4, 3, 3, 5), (0, 2), 8, "prescribed"),      # odd row count, L=8
+    ((70, 2, 3, 3), (3, 2, 3, 3), (0, 0), 64, "sparse"),         # waves spanning items
+])
+def test_forward_matches_oracle(capi, so, shape_x, shape_w, pad, L, mode):
+    x, w = wl.make_inputs(shape_x, shape_w, mode, seed=L + shape_x[0])
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad)
+    got = gpu_forward(capi, x, w, L, pad)
+    assert np.array_equal(got, exp)
+
+
+@pytest.mark.parametrize("loading", [(7, 2, 2, 2), (7, 1, 4, 4), (7, 4, 3, 3), (7, 2, 1, 1)])
+@pytest.mark.parametrize("L", [16, 64, 128])
+def test_forward_progressive_loading_matches_oracle(capi, so, loading, L):
+    """Pinned by the reference's GPU source text only (sc_cuda_kernel.cu:155-165): no CPU
+    code in the reference executes progressive loading."""
+    tw, lw, ww, wa = loading
+    x, w = wl.make_inputs((2, 4, 6, 6), (5, 4, 3, 3), "prescribed", seed=7)
+    kw = dict(total_width=tw, load_width=lw, load_wait_w=ww, load_wait_a=wa)
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, (1, 1), **kw)
+    got = gpu_forward(capi, x, w, L, (1, 1), **kw)
+    assert np.array_equal(got, exp)
+    neutral = gpu_forward(capi, x, w, L, (1, 1))
+    assert not np.array_equal(got, neutral) or L == 16
+
+
+# ------------------------------------------------------------------ forward: full sizes
+@pytest.mark.parametrize("name", [
+    "C1_prescribed_L64", "C3_sparse_L32", "C3_sparse_L128", "C3_sparse_L256", "C3_kaiming_L128",
+    "C3_kaiming_L256", "C3_q7_L128", "C3_q7_L256", "C3_prescribed_L128", "C4_prescribed_L128",
+    "C5_kaiming_L256", "C5_sparse_L256", "C5_prescribed_L256",
+])
+def test_forward_full_size_checksums(capi, checksums, name):
+    """SHA-256 of the int32 output against the reference CPU kernel's, inputs regenerated
+    from the seed."""
+    c = checksums[name]
+    x, w, pad, _ = wl.named(c["shape_name"], c["mode"])
+    y = gpu_forward(capi, x, w, c["L"], pad)
+    assert list(y.shape) == c["shape"]
+    assert int(y.astype(np.int64).sum()) == c["sum"]
+    assert int(np.abs(y.astype(np.int64)).sum()) == c["abs_sum"]
+    assert hashlib.sha256(np.ascontiguousarray(y).tobytes()).hexdigest() == c["sha256"]
+
+
+def test_forward_full_size_properties(capi):
+    """Size-independent properties at the headline shape: identical seeds for every batch
+    item, c_out equivariance, the |y| <= H*L bound, zero input -> zero output."""
+    x, w, pad, L = wl.named("C3", "kaiming")
+    y = gpu_forward(capi, x, w, L, pad)
+    assert np.abs(y).max() <= 3 * L
+    perm = torch.randperm(x.shape[0], generator=torch.Generator().manual_seed(1))
+    yp = gpu_forward(capi, x[perm], w, L, pad)
+    assert np.array_equal(yp, y[perm.numpy()])
+    cperm = torch.randperm(w.shape[0], generator=torch.Generator().manual_seed(2))
+    yc = gpu_forward(capi, x, w[cperm], L, pad)
+    assert np.array_equal(yc, y[:, cperm.numpy()])
+    assert not gpu_forward(capi, torch.zeros_like(x), w, L, pad).any()
+    x2 = x.clone()
+    x2[1:] = x[0]
+    y2 = gpu_forward(capi, x2, w, L, pad)
+    assert np.array_equal(y2[5], y2[0]) and np.array_equal(y2[0], y[0])
+
+
+# ------------------------------------------------------------------ boundary behaviour
+def test_c_abi_error_codes(capi):
+    x = torch.zeros((1, 2, 4, 4), device="cuda")
+    w = torch.zeros((3, 2, 3, 3), device="cuda")
+    with pytest.raises(capi.GeoScError) as e:
+        capi.conv2d_add_partial_forward(x, w, 100)
+    assert e.value.status == 2
+    with pytest.raises(capi.GeoScError) as e:
+        capi.conv2d_add_partial_forward(x, torch.zeros((3, 2, 5, 5), device="cuda"), 64)
+    assert e.value.status == 1
+    with pytest.raises(capi.GeoScError) as e:
+        capi.conv2d_add_partial_forward(x, w, 64, load_wait_w=0)
+    assert e.value.status == 1
+    with pytest.raises(capi.GeoScError) as e:
+        capi.conv2d_add_partial_forward(x, w, 64, workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+    assert e.value.status == 3
+
+
+def test_torch_modules_with_reference_names(capi, so, fixtures_small):
+    from geo_amd import _native
+    sc_cuda = _native.module("sc_extension_cuda")
+    sc_cpu_name = _native.module("sc_extension")
+    d = fixtures_small["T2"]
+    x, w = torch.from_numpy(d["x"]), torch.from_numpy(d["w"])
+    pad = d["pad"]
+    # GPU op, positional call exactly as utils_functional.py:497 makes it
+    y = sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), d["L"], (pad, pad), (1, 1), 7, 8, 1, False, 2)
+    assert y.is_cuda and y.dtype == torch.int32
+    assert np.array_equal(y.cpu().numpy(), d["y"])
+    # caller-side padding as the reference does it (utils_functional.py:496)
+    xp = torch.nn.functional.pad(x, (pad, pad, pad, pad)).cuda()
+    y2 = sc_cuda.conv2d_add_partial_variable_acc(xp, w.cuda(), d["L"], (0, 0), (1, 1), 7, 8, 1, False, 2)
+    assert np.array_equal(y2.cpu().numpy(), d["y"])
+    # non-contiguous input is made contiguous rather than mis-indexed
+    xt = x.cuda().transpose(2, 3).contiguous().transpose(2, 3)
+    y3 = sc_cuda.conv2d_add_partial_variable_acc(xt, w.cuda(), d["L"], (pad, pad), (1, 1), 7, 8, 1, False, 2)
+    assert np.array_equal(y3.cpu().numpy(), d["y"])
+    # progressive loading through the module
+    y4 = sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), d["L"], (pad, pad), (1, 1), 7, 2, 2, False, 2)
+    exp4 = so.conv2d_add_partial(d["x"], d["w"], d["L"], (pad, pad), 7, 2, 2, 2)
+    assert np.array_equal(y4.cpu().numpy(), exp4)
+    # host-tensor entry point (utils_functional.py:493): same kernels, result back on the host
+    y5 = sc_cpu_name.conv2d_add_partial_new(x, w, d["L"], (pad, pad), (1, 1))
+    assert not y5.is_cuda and np.array_equal(y5.numpy(), d["y"])
+    # errors are raised, not undefined behaviour
+    with pytest.raises(RuntimeError):
+        sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), 100, (pad, pad), (1, 1), 7, 8, 1, False, 2)
+    with pytest.raises(RuntimeError):
+        sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), 64, (pad, pad), (1, 1), 7, 8, 1, False, 0)
+    with pytest.raises(RuntimeError):
+        sc_cuda.conv2d_or_acc(x.cuda(), w.cuda(), 64, (pad, pad), (1, 1), False)
+
+
+def test_runs_on_the_current_stream_and_single_hip_runtime(capi, fixtures_small):
+    d = fixtures_small["T3"]
+    x, w = torch.from_numpy(d["x"]).cuda(), torch.from_numpy(d["w"]).cuda()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        y = capi.conv2d_add_partial_forward(x, w, d["L"], (d["pad"], d["pad"]))
+    s.synchronize()
+    assert np.array_equal(y.cpu().numpy(), d["y"])
+    with open("/proc/self/maps") as f:
+        hips = {line.split()[-1] for line in f if "libamdhip64" in line}
+    assert len(hips) == 1, hips
