@@ -39,6 +39,9 @@ def parse():
     ap.add_argument("--workload", default="C3", choices=["C1", "C3", "C4", "C5"])
     ap.add_argument("--length", type=int, default=0, help="stream length (default: the workload's)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="also launch one plain device copy of this many MiB (reads MIB, writes MIB): the known-size "
+                         "kernel that hardware traffic counters are scaled by")
     return ap.parse_args()
 
 
@@ -121,6 +124,12 @@ def main():
 
     def step():
         capi.conv2d_add_partial_forward(xd, wd, L, (pad, pad), out=out, workspace=ws, desc=desc)
+
+    if args.copy_calibration:
+        src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     # whole step: barrier-free on one GPU, synchronise both sides of the timed region
     for _ in range(args.warmup):

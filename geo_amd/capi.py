@@ -129,3 +129,32 @@ def conv2d_add_partial_from_streams(act, wgt, desc: ConvDesc, out=None, stream=N
                                                                 _stream_ptr(stream)),
            "geo_sc_conv2d_add_partial_from_streams")
     return out
+
+
+def backward_workspace_size(desc: ConvDesc) -> int:
+    out = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_conv2d_add_partial_backward_workspace_size(ctypes.byref(desc), ctypes.byref(out)),
+           "backward workspace query")
+    return out.value
+
+
+def conv2d_add_partial_backward(x, w, grad_y, bit_length=128, padding=(0, 0), need_grad_x=True, need_grad_w=True,
+                                workspace=None, stream=None, desc=None):
+    """(grad_x, grad_w) of the surrogate via geo_sc_conv2d_add_partial_backward; an output
+    that is not needed is returned as None."""
+    _require_gpu_f32(x, "x")
+    _require_gpu_f32(w, "w")
+    _require_gpu_f32(grad_y, "grad_y")
+    if desc is None:
+        desc = make_desc(x.shape, w.shape, bit_length, padding)
+    if tuple(grad_y.shape) != output_shape(desc):
+        raise ValueError(f"grad_y has shape {tuple(grad_y.shape)}, expected {output_shape(desc)}")
+    if workspace is None:
+        workspace = torch.empty(backward_workspace_size(desc), dtype=torch.uint8, device=x.device)
+    gx = torch.empty_like(x) if need_grad_x else None
+    gw = torch.empty_like(w) if need_grad_w else None
+    _check(_native.lib().geo_sc_conv2d_add_partial_backward(ctypes.byref(desc), _ptr(x), _ptr(w), _ptr(grad_y),
+                                                            _ptr(gx), _ptr(gw), _ptr(workspace), workspace.numel(),
+                                                            _stream_ptr(stream)),
+           "geo_sc_conv2d_add_partial_backward")
+    return gx, gw

@@ -184,4 +184,27 @@ int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float*
     return launch_conv_forward(g, act, wgt, y, s);
 }
 
+int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes)
+{
+    Geometry g;
+    if (!bytes) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    *bytes = backward_workspace_bytes(g);
+    return GEO_SC_OK;
+}
+
+int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float* x, const float* w,
+                                       const float* grad_y, float* grad_x, float* grad_w, void* workspace,
+                                       size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    Geometry g;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!x || !w || !grad_y || (!grad_x && !grad_w)) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (!workspace || workspace_bytes < backward_workspace_bytes(g) || ((uintptr_t)workspace & 255u))
+        return GEO_SC_ERR_WORKSPACE;
+    return launch_conv_backward(g, x, w, grad_y, grad_x, grad_w, workspace, (hipStream_t)stream);
+}
+
 }  // extern "C"

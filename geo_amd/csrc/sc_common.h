@@ -48,5 +48,8 @@ int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, con
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
+size_t backward_workspace_bytes(const Geometry& g);
+int launch_conv_backward(const Geometry& g, const float* x, const float* w, const float* gy, float* gx, float* gw,
+                         void* workspace, hipStream_t s);
 
 }  // namespace geo_sc

@@ -13,6 +13,7 @@
 // word) pair.  A kernel row's popcounts are folded into int32 sums with v_bcnt_u32_b32.
 // Consecutive workgroups take the c_out tiles of the same positions.
 #include "sc_common.h"
+#include <stdlib.h>
 
 namespace geo_sc {
 
@@ -27,6 +28,7 @@ struct FwdParams {
     int row_groups;        // ceil(wo / R)
     long long slots;       // n * row_groups * ho
     unsigned act_plane;    // c_in * wi * hi
+    int map;
 };
 
 // acc |= a & w with w wave-uniform: a single v_and_or_b32 whose first source is the SGPR.
@@ -43,8 +45,19 @@ template <int R, int WK>
 __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 {
     constexpr int C = kCoTile;
-    const int cot = blockIdx.x % q.n_cotile;
-    const long long slot0 = (long long)(blockIdx.x / q.n_cotile) * 64 + threadIdx.x;
+    int cot, mt;
+    if (q.map == 0) {
+        cot = blockIdx.x % q.n_cotile;
+        mt = blockIdx.x / q.n_cotile;
+    } else {
+        // workgroup ids are dealt round-robin to the 8 XCDs: keep all c_out tiles of one
+        // position tile on one XCD so that its L2 serves their common activation words
+        const unsigned per = 8u * q.n_cotile;
+        const unsigned grp = blockIdx.x / per, rem = blockIdx.x % per;
+        mt = grp * 8 + (rem & 7);
+        cot = rem >> 3;
+    }
+    const long long slot0 = (long long)mt * 64 + threadIdx.x;
     const bool live = slot0 < q.slots;
     const long long slot = live ? slot0 : 0;
     const int b = (int)(slot % q.ho);
@@ -85,10 +98,17 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
             const uint32_t* wp = q.wgt + ((size_t)(p * q.h_k + v) * k_or * q.n_cotile + cot) * (2 * C);
 
             if constexpr (WK > 0) {
-                for (int ci = 0; ci < q.c_in; ci++) {
-                    uint32_t aw[NROWS];
+                // activation words are fetched one channel ahead of their use
+                uint32_t aw[NROWS], an[NROWS];
 #pragma unroll
-                    for (int j = 0; j < NROWS; j++) aw[j] = ap[row_off[j]];
+                for (int j = 0; j < NROWS; j++) an[j] = ap[row_off[j]];
+#pragma unroll 2
+                for (int ci = 0; ci < q.c_in; ci++) {
+#pragma unroll
+                    for (int j = 0; j < NROWS; j++) aw[j] = an[j];
+                    ap += (ci + 1 < q.c_in) ? ch_stride : 0u;
+#pragma unroll
+                    for (int j = 0; j < NROWS; j++) an[j] = ap[row_off[j]];
 #pragma unroll
                     for (int u = 0; u < WK; u++) {
                         uint32_t wv[2 * C];
@@ -103,7 +123,6 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
                             }
                         wp += k_stride;
                     }
-                    ap += ch_stride;
                 }
             } else {
                 for (int ci = 0; ci < q.c_in; ci++) {
@@ -154,7 +173,10 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     q.row_groups = (g.wo + R - 1) / R;
     q.slots = (long long)g.n * q.row_groups * g.ho;
     const long long tiles = (q.slots + 63) / 64;
-    const long long blocks = tiles * g.n_cotile;
+    long long blocks = tiles * g.n_cotile;
+    const char* e = getenv("GEO_SC_MAP");
+    q.map = e ? atoi(e) : 0;
+    if (q.map) blocks = (tiles + 7) / 8 * 8 * g.n_cotile;
     if (blocks <= 0 || blocks > 0x7fffffffLL) return GEO_SC_ERR_INVALID_ARGUMENT;
     hipLaunchKernelGGL((k_conv_fwd<R, WK>), dim3((unsigned)blocks), dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;

@@ -1,0 +1,143 @@
+"""Functional SC layer with the reference's interface (utils_functional.py), for the one
+configuration this build accelerates: ``forward='1d_bin'`` (OR over input channels and
+kernel dim 2, binary add over kernel dim 3), ``generator='lfsr'``, ``legacy=False``.
+
+Forward values come from the HIP SC kernels (integer counts / stream length); gradients
+are those of the reference's floating-point surrogate ``conv2d_or_bin_1d``
+(utils_functional.py:235-252), computed by the HIP backward kernels instead of autograd
+over 2*H dense convolutions.  The surrogate's own forward is never evaluated: the
+reference overwrites its value with the SC result anyway (utils_functional.py:631-634).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from . import capi
+
+# Default precision is 8-bit integer, one bit is the sign (utils_functional.py:28)
+prec_default = 7
+
+
+def quantize(input, prec=8):
+    """round(x * 2^prec) clamped to +-(2^prec - 1), scaled back (utils_functional.py:33-39)."""
+    prec_2 = 2 ** prec
+    return (input * prec_2).round().clamp(-prec_2 + 1, prec_2 - 1) / prec_2
+
+
+def quantize_shift(tensor, scale=None, scale_only=False):
+    """Power-of-two scale, then 8-bit quantisation of tensor/scale (utils_functional.py:41-57)."""
+    if scale_only:
+        scale = 2 ** torch.ceil(torch.log2(torch.mean(tensor) * 2))
+        return torch.ones_like(tensor) * scale, scale
+    if scale is None:
+        scale = 2 ** torch.ceil(torch.log2(torch.mean(tensor) * 3))
+    q = ((tensor / scale) * 128).round().clamp(-127, 127) / 128
+    return q * scale, scale
+
+
+def conv2d_or_bin_1d(activation, w_pos, w_neg, padding, stride):
+    """The surrogate itself, in plain torch (utils_functional.py:235-252): one W x 1
+    convolution per kernel row and rail, 1 - exp(-z), summed over rows.  Kept as the
+    executable definition of what the HIP backward differentiates; the layer does not
+    call it."""
+    i_y = activation.size(3)
+    f_y = w_pos.size(3)
+    pos, neg = [], []
+    for j in range(f_y):
+        a_sec = activation[..., j:i_y - f_y + j + 1]
+        pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[..., j:j + 1], stride=stride)))
+        neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[..., j:j + 1], stride=stride)))
+    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
+
+
+class _SCConv2dAddPartial(torch.autograd.Function):
+    """value: SC count / L  (HIP forward);  gradient: surrogate (HIP backward)."""
+
+    @staticmethod
+    def forward(ctx, activation, weight, bit_length, padding, load_unit, load_wait):
+        origin = activation.device
+        dev = origin if activation.is_cuda else torch.device("cuda", torch.cuda.current_device())
+        x = activation.detach().to(dev, torch.float32).contiguous()
+        w = weight.detach().to(dev, torch.float32).contiguous()
+        pad = (int(padding[0]), int(padding[1]))
+        if activation.is_cuda:
+            # sc_extension_cuda.conv2d_add_partial_variable_acc(..., prec_default, load_unit,
+            # load_wait_w, False, 2): one wait for both generators (utils_functional.py:497)
+            loading = dict(total_width=prec_default, load_width=int(load_unit), load_wait_w=int(load_wait),
+                           load_wait_a=int(load_wait))
+        else:
+            # host tensors take the reference's CPU entry point, which has no progressive
+            # loading (utils_functional.py:493)
+            loading = dict(capi.NEUTRAL_LOADING)
+        counts = capi.conv2d_add_partial_forward(x, w, int(bit_length), pad, **loading)
+        ctx.save_for_backward(x, w)
+        ctx.pad = pad
+        ctx.origin = origin
+        ctx.bit_length = int(bit_length)
+        ctx.act_dtype = activation.dtype
+        ctx.w_dtype = weight.dtype
+        ctx.w_device = weight.device
+        return (counts.float() / bit_length).to(origin)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w = ctx.saved_tensors
+        g = grad_out.detach().to(x.device, torch.float32).contiguous()
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        gx = gw = None
+        if need_x or need_w:
+            gx, gw = capi.conv2d_add_partial_backward(x, w, g, ctx.bit_length, ctx.pad, need_x, need_w)
+        if gx is not None:
+            gx = gx.to(ctx.origin, ctx.act_dtype)
+        if gw is not None:
+            gw = gw.to(ctx.w_device, ctx.w_dtype)
+        return gx, gw, None, None, None, None
+
+
+def conv2d_generic(activation, weight, padding, stride, **kwargs):
+    """Generic SC conv2d layer, same call as the reference's (utils_functional.py:406-634).
+
+    Keyword arguments read: bit_length (128), generator (None), forward ('full_or'), legacy
+    (False), load_unit (8), load_wait_w (1), load_wait_a (1); prec/acc/share/z_unit are
+    accepted and unused on this path.  Only forward='1d_bin', generator='lfsr',
+    legacy=False is implemented; anything else raises NotImplementedError.
+    """
+    bit_length = kwargs.get("bit_length", 128)
+    generator = kwargs.get("generator", None)
+    forward = kwargs.get("forward", "full_or")
+    legacy = kwargs.get("legacy", False)
+    load_unit = kwargs.get("load_unit", 8)
+    load_wait_w = kwargs.get("load_wait_w", 1)
+    if forward != "1d_bin" or generator != "lfsr" or legacy:
+        raise NotImplementedError(
+            f"conv2d_generic(forward={forward!r}, generator={generator!r}, legacy={legacy}): this build implements "
+            "forward='1d_bin', generator='lfsr', legacy=False only")
+    if isinstance(stride, int):
+        stride = (stride, stride)
+    if tuple(stride) != (1, 1):
+        raise NotImplementedError("the SC kernels compute stride 1 only (the reference's native code ignores stride)")
+    if isinstance(padding, int):
+        padding = (padding, padding)
+    return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), load_unit, load_wait_w)
+
+
+def smoke_layer_step():
+    """One SC layer forward + backward on cuda:0 against the torch surrogate (used by the
+    smoke check)."""
+    from . import workloads as wl
+
+    x, w = wl.make_inputs((2, 4, 8, 8), (6, 4, 3, 3), "q7", seed=3)
+    x = x.cuda().requires_grad_(True)
+    w = (w * 4).cuda().requires_grad_(True)
+    y = conv2d_generic(x, w, (1, 1), (1, 1), bit_length=64, forward="1d_bin", generator="lfsr")
+    g = torch.linspace(-1, 1, y.numel(), device="cuda").reshape(y.shape)
+    y.backward(g)
+    xr = x.detach().double().requires_grad_(True)
+    wr = w.detach().double().requires_grad_(True)
+    xp = F.pad(xr, (1, 1, 1, 1))
+    p, n = conv2d_or_bin_1d(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)), (0, 0), (1, 1))
+    (p - n).backward(g.double())
+    for got, ref in ((x.grad, xr.grad), (w.grad, wr.grad)):
+        err = (got.double() - ref).abs().max().item()
+        assert err <= 1e-5 * ref.abs().max().item(), err

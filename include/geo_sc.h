@@ -134,6 +134,24 @@ GEO_SC_API int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* de
 GEO_SC_API int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
 GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);
 
+/*
+ * Backward of the layer through the reference's floating-point surrogate
+ * (utils_functional.py:611-634 with conv2d_or_bin_1d, :235-252; differentiated there by
+ * torch autograd, there is no native counterpart in the reference):
+ *     wp = clamp(w, 0, 100), wn = -clamp(w, -100, 0), x~ = zero-padded x
+ *     z+-_v = corr2d(x~[..., v : v+Ho], w+-[..., v:v+1]),   v < h_k
+ *     y^    = sum_v (1 - exp(-z+_v)) - sum_v (1 - exp(-z-_v))
+ * grad_x (n, c_in, w_in, h_in) = d y^ / d x contracted with grad_y (padding sliced off);
+ * grad_w (c_out, c_in, w_k, h_k) = d y^ / d w contracted with grad_y, clamp passing its
+ * gradient on the closed interval.  fp32 throughout, fp32 accumulation.  Either output may
+ * be NULL to skip it.  bit_length and the loading fields of `desc` are validated but do not
+ * enter the result.
+ */
+GEO_SC_API int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
+GEO_SC_API int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float* x, const float* w,
+                                                  const float* grad_y, float* grad_x, float* grad_w,
+                                                  void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,91 @@
+"""Gradient oracle of the SC convolution layer: TEST INFRASTRUCTURE, never on the product
+path.
+
+The reference has no native backward.  It builds a floating-point surrogate of the layer
+with ordinary torch ops and lets autograd differentiate it (utils_functional.py:611-634
+with conv2d_or_bin_1d, utils_functional.py:235-252).  ``surrogate_autograd`` restates
+exactly that composition (pad -> clamp -> per-row W x 1 convolutions -> 1 - exp(-z) ->
+stack/sum -> value overwrite -> pos - neg) in double precision; ``surrogate_closed_form``
+is an independent numpy evaluation of the derivative formulas, used to pin the first on
+small shapes together with finite differences (tests/test_oracle_surrogate.py).
+
+Pinning status: pinned by closed form + central finite differences; the reference's Python
+modules are not imported.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+
+def surrogate_autograd(x, w, grad_out, padding=(0, 0), sc_value=None, dtype=torch.float64):
+    """(grad_x, grad_w, surrogate_value) as torch tensors of ``dtype``.
+
+    ``padding=(p0,p1)``: p0 pads the last dim, p1 the one before (utils_functional.py:496).
+    ``sc_value`` (optional) is written over the surrogate's value the way the reference does
+    (utils_functional.py:632-633) to show that the overwrite does not reach the gradients.
+    """
+    x = torch.as_tensor(x).detach().to(dtype).requires_grad_(True)
+    w = torch.as_tensor(w).detach().to(dtype).requires_grad_(True)
+    g = torch.as_tensor(grad_out).detach().to(dtype)
+    act = F.pad(x, (padding[0], padding[0], padding[1], padding[1]))
+    w_pos = w.clamp(0, 100)
+    w_neg = -(w.clamp(-100, 0))
+    i_y, f_y = act.size(3), w.size(3)
+    pos, neg = [], []
+    for j in range(f_y):
+        a_sec = act[..., j:i_y - f_y + j + 1].clone()
+        pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[..., j:j + 1].clone())))
+        neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[..., j:j + 1].clone())))
+    pos_v = torch.stack(pos, 0).sum(0)
+    neg_v = torch.stack(neg, 0).sum(0)
+    value = (pos_v - neg_v).detach().clone()
+    if sc_value is not None:
+        pos_v.data = torch.as_tensor(sc_value).to(dtype)
+        neg_v.data = torch.zeros_like(neg_v)
+    out = pos_v - neg_v
+    out.backward(g)
+    return x.grad.detach(), w.grad.detach(), value
+
+
+def surrogate_closed_form(x, w, grad_out, padding=(0, 0)):
+    """(grad_x, grad_w, value) in float64 numpy from the written-out derivative:
+        z+-_v[n,co,a,b] = sum_{ci,u} xp[n,ci,a+u,b+v] * w+-[co,ci,u,v]
+        value           = sum_v (1-exp(-z+_v)) - (1-exp(-z-_v))
+        dL/dz+_v = g exp(-z+_v),  dL/dz-_v = -g exp(-z-_v)
+        dL/dw    = [0<=w<=100] dL/dw+  -  [-100<=w<=0] dL/dw-
+    """
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    g = np.asarray(grad_out, dtype=np.float64)
+    p0, p1 = int(padding[0]), int(padding[1])
+    xp = np.pad(x, ((0, 0), (0, 0), (p1, p1), (p0, p0)))
+    N, Cin, Wi, Hi = xp.shape
+    Cout, _, W, H = w.shape
+    Wo, Ho = Wi - W + 1, Hi - H + 1
+    wp = np.clip(w, 0, 100)
+    wn = -np.clip(w, -100, 0)
+    value = np.zeros((N, Cout, Wo, Ho))
+    gxp = np.zeros_like(xp)
+    gwp = np.zeros_like(w)
+    gwn = np.zeros_like(w)
+    for v in range(H):
+        zp = np.zeros((N, Cout, Wo, Ho))
+        zn = np.zeros((N, Cout, Wo, Ho))
+        for u in range(W):
+            patch = xp[:, :, u:u + Wo, v:v + Ho]
+            zp += np.einsum("ncab,oc->noab", patch, wp[:, :, u, v])
+            zn += np.einsum("ncab,oc->noab", patch, wn[:, :, u, v])
+        value += (1 - np.exp(-zp)) - (1 - np.exp(-zn))
+        dzp = g * np.exp(-zp)
+        dzn = -g * np.exp(-zn)
+        for u in range(W):
+            patch = xp[:, :, u:u + Wo, v:v + Ho]
+            gwp[:, :, u, v] = np.einsum("noab,ncab->oc", dzp, patch)
+            gwn[:, :, u, v] = np.einsum("noab,ncab->oc", dzn, patch)
+            gxp[:, :, u:u + Wo, v:v + Ho] += np.einsum("noab,oc->ncab", dzp, wp[:, :, u, v])
+            gxp[:, :, u:u + Wo, v:v + Ho] += np.einsum("noab,oc->ncab", dzn, wn[:, :, u, v])
+    gw = gwp * ((w >= 0) & (w <= 100)) - gwn * ((w >= -100) & (w <= 0))
+    gx = gxp[:, :, p1:Wi - p1, p0:Hi - p0]
+    return gx, gw, value
