@@ -1,0 +1,102 @@
+"""The 4-layer SC CNN of the reference's training script (network.py:126-190,
+``CONV_tiny_add_partial``), restated on this build's layer modules, and the bookkeeping of
+one training step (utils_own.py:81-114).  Only what the 4-layer training-step workload
+needs; datasets, checkpointing and the CLI are not part of this build.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import utils_class
+
+# loss scale of the reference's training loop (utils_own.py:18, :81)
+SCALE_FACTOR = 128
+
+
+class CONV_tiny_add_partial(nn.Module):
+    """conv 3->32 k5 p2 @32x32, BN, AvgPool2, Hardtanh(0,1); 32->32 k5 p2 @16x16; 32->64 k5 p2
+    @8x8; conv 64->classes k4 p0 @4x4 as the classifier; BN1d.  Per-layer stream length is
+    2**err[i]; load_unit / load_wait are the progressive-loading settings per layer."""
+
+    def __init__(self, num_classes=10, c_ins=3, uniform=False, generator="lfsr", sc_compute="1d_bin", legacy=False,
+                 relu=False):
+        super().__init__()
+        self.bn1 = utils_class.BatchNorm2d_fixed(32)
+        self.bn2 = utils_class.BatchNorm2d_fixed(32)
+        self.bn3 = utils_class.BatchNorm2d_fixed(64)
+        self.bn4 = utils_class.BatchNorm1d_fixed(num_classes)
+        self.conv1 = utils_class.Conv2d_Add_Partial(c_ins, 32, kernel_size=5, padding=2, bias=False)
+        self.conv2 = utils_class.Conv2d_Add_Partial(32, 32, kernel_size=5, padding=2, bias=False)
+        self.conv3 = utils_class.Conv2d_Add_Partial(32, 64, kernel_size=5, padding=2, bias=False)
+        self.fc1 = utils_class.Conv2d_Add_Partial(64, num_classes, kernel_size=4, padding=0, bias=False)
+        self.tanh = nn.Hardtanh(0, 1)
+        self.pool = nn.AvgPool2d(2)
+        self.err = [7, 7, 7, 7]
+        self.z_unit = [3, 3, 4, 4]
+        self.load_unit = [2, 2, 2, 2]
+        self.load_wait_w = [2, 2, 2, 2]
+        # the reference's forward reads `load_wait`, which its training script sets from the
+        # command line (main_conv.py:182); the default there is 2 per layer
+        self.load_wait = [2, 2, 2, 2]
+        self.num_classes = num_classes
+        self.generator = generator
+        self.compute = sc_compute
+        self.legacy = legacy
+        self.relu = relu
+        if uniform:
+            self.conv1.weight_org *= 2
+            self.conv2.weight_org *= 2
+            self.conv1.weight.data *= 2
+            self.conv2.weight.data *= 2
+
+    def _sc(self, conv, x, i, wait_w_index=None):
+        j = i if wait_w_index is None else wait_w_index
+        return conv(x, err=self.err[i], forward=self.compute, generator=self.generator, z_unit=2 ** self.z_unit[i],
+                    legacy=self.legacy, load_unit=self.load_unit[i], load_wait_w=self.load_wait[j],
+                    load_wait_a=self.load_wait[i])
+
+    def _block(self, conv, bn, x, i):
+        x = bn(self._sc(conv, x, i))
+        if self.relu:
+            x = F.relu(x)
+        return self.tanh(self.pool(x))
+
+    def forward(self, x_in, target=None):
+        x = self._block(self.conv1, self.bn1, x_in, 0)
+        x = self._block(self.conv2, self.bn2, x, 1)
+        x = self._block(self.conv3, self.bn3, x, 2)
+        # the classifier layer takes the third layer's weight wait (network.py:186)
+        x = self._sc(self.fc1, x, 3, wait_w_index=2)
+        return self.bn4(x.view(-1, self.num_classes))
+
+
+def make_param_copies(model):
+    """Full-precision master copies the optimiser updates (main_conv.py:203-213)."""
+    return [p.detach().clone().float().requires_grad_(True) for p in model.parameters()]
+
+
+def train_step(model, inputs, target, criterion, optimizer, param_copy):
+    """One step of the reference's loop (utils_own.py:79-114): scaled loss, backward, restore
+    full-precision weights, hand gradients to the master copies, un-scale, optimiser step,
+    copy back, refresh ``weight_org`` clamped to [-1, 0.999].  Returns the unscaled loss."""
+    output = model(inputs)
+    loss = criterion(output, target) * SCALE_FACTOR
+    for p in model.parameters():
+        p.grad = None
+    loss.backward()
+    for m in model.modules():
+        if hasattr(m, "weight_org"):
+            m.weight.data.copy_(m.weight_org)
+    params = list(model.parameters())
+    for master, p in zip(param_copy, params):
+        master.grad = None if p.grad is None else (p.grad.data.float() / SCALE_FACTOR)
+    optimizer.step()
+    for master, p in zip(param_copy, params):
+        p.data.copy_(master.data)
+    for m in model.modules():
+        if hasattr(m, "weight_org"):
+            m.weight_org.copy_(m.weight.data.clamp(-1, 0.999))
+    optimizer.zero_grad()
+    return loss.detach() / SCALE_FACTOR
