@@ -6,8 +6,10 @@
 
 One step = one pass of the hot path over one batch of synthetic input that is already
 resident in HBM: float->code conversion, LFSR stream generation for weights and
-activations, the AND/OR/popcount convolution (and the surrogate backward once
-``--pass fwdbwd`` is supported by the build).  Prints ONE JSON line.
+activations, the AND/OR/popcount convolution, then the surrogate backward (both gradients)
+for an upstream gradient of the output's shape.  ``--pass fwd`` times the forward alone.
+Prints ONE JSON line; ``value`` is SC bit-MACs of the step divided by the step's whole
+duration (the backward does no bit-MACs, so the forward-only rate is reported next to it).
 
 The default workload is the configuration the headline metric is quoted on: SC conv2d
 128->128 3x3 at 16x16, batch 256, pad 1, stream length 128, activations U[0,1), weights
@@ -38,6 +40,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C3", choices=["C1", "C3", "C4", "C5"])
     ap.add_argument("--length", type=int, default=0, help="stream length (default: the workload's)")
+    ap.add_argument("--pass", dest="passes", default="fwdbwd", choices=["fwd", "fwdbwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="also launch one plain device copy of this many MiB (reads MIB, writes MIB): the known-size "
@@ -122,8 +125,20 @@ def main():
     ws = torch.empty(capi.workspace_size(desc), dtype=torch.uint8, device="cuda")
     out = torch.empty(capi.output_shape(desc), dtype=torch.int32, device="cuda")
 
-    def step():
+    with_bwd = args.passes == "fwdbwd"
+    gy = torch.randn(out.shape, generator=torch.Generator().manual_seed(1)).cuda()
+    ws_b = torch.empty(capi.backward_workspace_size(desc), dtype=torch.uint8, device="cuda") if with_bwd else None
+
+    def fwd():
         capi.conv2d_add_partial_forward(xd, wd, L, (pad, pad), out=out, workspace=ws, desc=desc)
+
+    def bwd():
+        capi.conv2d_add_partial_backward(xd, wd, gy, L, (pad, pad), workspace=ws_b, desc=desc)
+
+    def step():
+        fwd()
+        if with_bwd:
+            bwd()
 
     if args.copy_calibration:
         src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device="cuda").fill_(1)
@@ -145,6 +160,13 @@ def main():
     B = wl.bit_macs(xd.shape, wd.shape, pad, L)
     value = B / (ms_per_step * 1e-3)
 
+    fwd_ms = time_events(fwd, args.steps, 2, torch)
+    fwd_avg = sum(fwd_ms) / len(fwd_ms)
+    bwd_avg = None
+    if with_bwd:
+        bwd_ms = time_events(bwd, args.steps, 2, torch)
+        bwd_avg = sum(bwd_ms) / len(bwd_ms)
+
     # dominant kernel alone (AND/OR/popcount on pre-generated streams), HIP events on its stream
     act = capi.act_streams(xd, desc)
     wgt = capi.weight_streams(wd, desc)
@@ -161,8 +183,8 @@ def main():
     stream_bytes = 4 * (act.numel() + wgt.numel())
 
     result = {
-        "metric": "SC bit-MACs/sec (whole forward op: codes + LFSR streams + AND/OR/popcount conv) at stream len "
-                  f"{L}",
+        "metric": "SC bit-MACs/sec over one layer step ("
+                  + ("forward + surrogate backward" if with_bwd else "forward") + f") at stream len {L}",
         "value": value,
         "unit": "bit-MAC/s",
         "n_gpus": 1,
@@ -176,7 +198,8 @@ def main():
         "data": "synthetic (torch.manual_seed(0); activations U[0,1), weights U[-1,1))",
         "config": {"workload": f"{args.workload}: SC conv2d {tuple(x.shape)} * {tuple(w.shape)} pad {pad}, "
                                f"stream length {L}, y-dimension partial binary accumulation, LFSR generators",
-                   "pass": "fwd", "bit_macs_per_step": B},
+                   "pass": args.passes, "bit_macs_per_step": B},
+        "layer_ms": {"fwd": fwd_avg, "bwd": bwd_avg, "fwd_bit_macs_per_s": B / (fwd_avg * 1e-3)},
         "roofline": {
             "bound": "valu",
             "kernel": "k_conv_fwd (v_and_or_b32 / v_bcnt_u32_b32)",
@@ -192,7 +215,11 @@ def main():
             "hbm_frac_of_peak": (stream_bytes + 4 * out.numel()) / (k_avg * 1e-3) / PEAK_HBM_BYTES,
             "traffic": None,
         },
-        "stages_ms": {"stream_generation": sum(gen_ms) / len(gen_ms), "conv_kernel": k_avg},
+        "stages_ms": {"stream_generation": sum(gen_ms) / len(gen_ms), "conv_kernel": k_avg, "backward": bwd_avg},
+        "backward_flops": {"algorithmic": 12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H,
+                           "achieved_tflops": (12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H
+                                               / (bwd_avg * 1e-3) / 1e12) if bwd_avg else None,
+                           "peak_tflops_fp32_mfma": 157.3},
     }
     if not args.no_cpu_baseline:
         kind, cores, sec, note = cpu_baseline(x, w, L, pad)
