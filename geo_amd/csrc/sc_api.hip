@@ -59,6 +59,8 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     g->n_cotile = (d->c_out + kCoTile - 1) / kCoTile;
     g->act_plane = (size_t)plane;
     g->act_words = (size_t)d->n * g->packs * g->act_plane;
+    g->act_item_inner = wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
+                        (unsigned long long)g->act_words < 0xffffffffull;
     g->wgt_words = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile * 2 * kCoTile;
     g->off_tables = 0;
     g->off_wgt = align256(table_bytes(g->L));

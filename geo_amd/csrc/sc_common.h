@@ -23,6 +23,10 @@ struct Geometry {
     int k_or;            // OR-group size c_in * w_k
     int n_cotile;        // ceil(c_out / kCoTile)
     size_t act_plane;    // c_in * wi * hi words: one pack of one item
+    // Activation stream layout.  false: [n][P][c_in][wi][hi].  true: [P][c_in][wi][hi][n] (batch item
+    // innermost), used when the output has a single row so that the convolution kernel's lanes,
+    // which then run over batch items, read consecutive words.
+    bool act_item_inner;
     size_t act_words;    // n * packs * act_plane
     size_t wgt_words;    // packs * h_k * k_or * n_cotile * 2 * kCoTile
     // workspace carve-up (byte offsets, 256-aligned)

@@ -13,22 +13,20 @@
 // word) pair.  A kernel row's popcounts are folded into int32 sums with v_bcnt_u32_b32.
 // Consecutive workgroups take the c_out tiles of the same positions.
 #include "sc_common.h"
-#include <stdlib.h>
 
 namespace geo_sc {
 
 namespace {
 
 struct FwdParams {
-    const uint32_t* __restrict__ act;  // [n][P][c_in][wi][hi]
+    const uint32_t* __restrict__ act;  // [n][P][c_in][wi][hi], or [P][c_in][wi][hi][n] with ROWS_IN_N
     const uint32_t* __restrict__ wgt;  // [P][h_k][k_or][n_cotile][2][16]
     int32_t* __restrict__ y;           // [n][c_out][wo][ho]
-    int c_in, wi, hi, c_out, w_k, h_k, packs;
+    int n, c_in, wi, hi, c_out, w_k, h_k, packs;
     int wo, ho, n_cotile;
-    int row_groups;        // ceil(wo / R)
-    long long slots;       // n * row_groups * ho
+    int row_groups;        // ceil(wo / R), or ceil(n / R) when the rows of a lane are batch items
+    long long slots;       // lane slots: n * row_groups * ho, or row_groups * ho
     unsigned act_plane;    // c_in * wi * hi
-    int map;
 };
 
 // acc |= a & w with w wave-uniform: a single v_and_or_b32 whose first source is the SGPR.
@@ -39,44 +37,89 @@ __device__ __forceinline__ void and_or(uint32_t& acc, uint32_t a, uint32_t w_uni
     asm("v_and_or_b32 %0, %1, %2, %0" : "+v"(acc) : "s"(w_uniform), "v"(a));
 }
 
-// R rows per lane, WK = kernel extent in dim 2 known at compile time (0: run-time extent,
-// rows handled one at a time).
-template <int R, int WK>
+// OR-accumulate CU consecutive input channels: per channel NW activation words per lane and
+// WK weight lines per wave.  word(r, u) is the activation word row r meets at kernel tap u.
+template <int R, int WK, int CU, int NW, bool ROWS_IN_N>
+__device__ __forceinline__ void or_channels(uint32_t (&orp)[R][kCoTile], uint32_t (&orn)[R][kCoTile],
+                                            const uint32_t*& ap, const uint32_t*& wp, const unsigned (&off)[NW],
+                                            unsigned ch_stride, unsigned k_stride)
+{
+    constexpr int C = kCoTile;
+    uint32_t aw[CU][NW];
+#pragma unroll
+    for (int cu = 0; cu < CU; cu++)
+#pragma unroll
+        for (int j = 0; j < NW; j++) aw[cu][j] = ap[cu * ch_stride + off[j]];
+#pragma unroll
+    for (int cu = 0; cu < CU; cu++)
+#pragma unroll
+        for (int u = 0; u < WK; u++) {
+            uint32_t wv[2 * C];
+#pragma unroll
+            for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const uint32_t a = aw[cu][ROWS_IN_N ? r * WK + u : r + u];
+#pragma unroll
+                for (int c = 0; c < C; c++) {
+                    and_or(orp[r][c], a, wv[c]);
+                    and_or(orn[r][c], a, wv[C + c]);
+                }
+            }
+            wp += k_stride;
+        }
+    ap += CU * ch_stride;
+}
+
+// Template parameters:
+//   R   rows of accumulators per lane.  ROWS_IN_N == false: R consecutive output rows a
+//       (dim 2) of one item; the WK kernel taps slide over R+WK-1 activation words, so each
+//       word is loaded once per channel.  ROWS_IN_N == true (outputs with a single row, e.g.
+//       the SC-linear mapping): R consecutive batch items.
+//   WK  kernel extent in dim 2 (0: run-time extent, R == 1).
+//   CU  input channels per loop trip, chosen so that a trip holds ~192 and-or instructions.
+template <int R, int WK, int CU, bool ROWS_IN_N>
 __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 {
     constexpr int C = kCoTile;
-    int cot, mt;
-    if (q.map == 0) {
-        cot = blockIdx.x % q.n_cotile;
-        mt = blockIdx.x / q.n_cotile;
-    } else {
-        // workgroup ids are dealt round-robin to the 8 XCDs: keep all c_out tiles of one
-        // position tile on one XCD so that its L2 serves their common activation words
-        const unsigned per = 8u * q.n_cotile;
-        const unsigned grp = blockIdx.x / per, rem = blockIdx.x % per;
-        mt = grp * 8 + (rem & 7);
-        cot = rem >> 3;
-    }
-    const long long slot0 = (long long)mt * 64 + threadIdx.x;
+    static_assert(WK > 0 || (R == 1 && !ROWS_IN_N), "run-time kernel extent handles one row per lane");
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long slot0 = (long long)(blockIdx.x / q.n_cotile) * 64 + threadIdx.x;
     const bool live = slot0 < q.slots;
     const long long slot = live ? slot0 : 0;
-    const int b = (int)(slot % q.ho);
+    // lane slot -> (first item n, first output row a0, output column b).  With ROWS_IN_N the
+    // R rows of a lane are items n and n + row_groups, consecutive lanes are consecutive
+    // items, and the activation streams are stored item-innermost.
+    const int b = ROWS_IN_N ? (int)(slot / q.row_groups) : (int)(slot % q.ho);
     const long long t = slot / q.ho;
-    const int a0 = (int)(t % q.row_groups) * R;
-    const long long n = t / q.row_groups;
+    const int a0 = ROWS_IN_N ? 0 : (int)(t % q.row_groups) * R;
+    const long long n = ROWS_IN_N ? slot % q.row_groups : t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
 
-    constexpr int NROWS = WK > 0 ? R + WK - 1 : 1;
-    // rows a0 .. a0+NROWS-1 of the padded item; rows past the end (partial last group) are
-    // clamped: they only feed outputs that are never stored
-    unsigned row_off[NROWS];
+    constexpr int NW = WK == 0 ? 1 : (ROWS_IN_N ? R * WK : R + WK - 1);
+    // word offsets inside one channel plane.  Rows past the end (partial last group) are
+    // clamped to valid ones: they only feed outputs that are never stored.
+    unsigned off[NW];
+    if constexpr (WK > 0) {
 #pragma unroll
-    for (int j = 0; j < NROWS; j++) {
-        int row = a0 + j;
-        row = row < q.wi ? row : q.wi - 1;
-        row_off[j] = (unsigned)row * q.hi;
+        for (int j = 0; j < NW; j++) {
+            if (ROWS_IN_N) {
+                const int r = j / WK, u = j % WK;
+                off[j] = (n + (long long)r * q.row_groups < q.n ? (unsigned)r * q.row_groups : 0u) +
+                         (unsigned)u * q.hi * q.n;
+            } else {
+                const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+                off[j] = (unsigned)row * q.hi;
+            }
+        }
+    } else {
+        off[0] = 0;
     }
-    const uint32_t* act_n = q.act + (size_t)n * q.packs * q.act_plane + b;
-    const unsigned ch_stride = (unsigned)q.wi * q.hi;
+    // strides (words) of one pack, one kernel row step, one channel
+    const size_t pack_stride = ROWS_IN_N ? (size_t)q.act_plane * q.n : (size_t)q.act_plane;
+    const unsigned v_stride = ROWS_IN_N ? (unsigned)q.n : 1u;
+    const unsigned ch_stride = ROWS_IN_N ? (unsigned)q.wi * q.hi * q.n : (unsigned)q.wi * q.hi;
+    const uint32_t* act_n = ROWS_IN_N ? q.act + (size_t)b * q.n + n : q.act + (size_t)n * item_stride + b;
     const int k_or = q.c_in * q.w_k;
     const unsigned k_stride = (unsigned)q.n_cotile * 2 * C;
 
@@ -94,52 +137,29 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 #pragma unroll
                 for (int c = 0; c < C; c++) orp[r][c] = orn[r][c] = 0u;
 
-            const uint32_t* ap = act_n + (size_t)p * q.act_plane + v;
+            const uint32_t* ap = act_n + (size_t)p * pack_stride + (size_t)v * v_stride;
             const uint32_t* wp = q.wgt + ((size_t)(p * q.h_k + v) * k_or * q.n_cotile + cot) * (2 * C);
 
             if constexpr (WK > 0) {
-                // activation words are fetched one channel ahead of their use
-                uint32_t aw[NROWS], an[NROWS];
-#pragma unroll
-                for (int j = 0; j < NROWS; j++) an[j] = ap[row_off[j]];
-#pragma unroll 2
-                for (int ci = 0; ci < q.c_in; ci++) {
-#pragma unroll
-                    for (int j = 0; j < NROWS; j++) aw[j] = an[j];
-                    ap += (ci + 1 < q.c_in) ? ch_stride : 0u;
-#pragma unroll
-                    for (int j = 0; j < NROWS; j++) an[j] = ap[row_off[j]];
-#pragma unroll
-                    for (int u = 0; u < WK; u++) {
-                        uint32_t wv[2 * C];
-#pragma unroll
-                        for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
-#pragma unroll
-                        for (int r = 0; r < R; r++)
-#pragma unroll
-                            for (int c = 0; c < C; c++) {
-                                and_or(orp[r][c], aw[r + u], wv[c]);
-                                and_or(orn[r][c], aw[r + u], wv[C + c]);
-                            }
-                        wp += k_stride;
-                    }
-                }
+                int ci = 0;
+                for (; ci + CU <= q.c_in; ci += CU)
+                    or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, ch_stride, k_stride);
+                if constexpr (CU > 1)
+                    for (; ci < q.c_in; ci++)
+                        or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, ch_stride, k_stride);
             } else {
                 for (int ci = 0; ci < q.c_in; ci++) {
                     for (int u = 0; u < q.w_k; u++) {
                         uint32_t wv[2 * C];
 #pragma unroll
                         for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
+                        int row = a0 + u;
+                        row = row < q.wi ? row : q.wi - 1;
+                        const uint32_t aw = ap[(unsigned)row * q.hi];
 #pragma unroll
-                        for (int r = 0; r < R; r++) {
-                            int row = a0 + r + u;
-                            row = row < q.wi ? row : q.wi - 1;
-                            const uint32_t aw = ap[(unsigned)row * q.hi];
-#pragma unroll
-                            for (int c = 0; c < C; c++) {
-                                and_or(orp[r][c], aw, wv[c]);
-                                and_or(orn[r][c], aw, wv[C + c]);
-                            }
+                        for (int c = 0; c < C; c++) {
+                            and_or(orp[0][c], aw, wv[c]);
+                            and_or(orn[0][c], aw, wv[C + c]);
                         }
                         wp += k_stride;
                     }
@@ -162,23 +182,29 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
         if (co >= q.c_out) break;
         int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
 #pragma unroll
-        for (int r = 0; r < R; r++)
-            if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[r][c];
+        for (int r = 0; r < R; r++) {
+            if (ROWS_IN_N) {
+                if (n + (long long)r * q.row_groups < q.n)
+                    yo[(size_t)r * q.row_groups * q.c_out * out_plane] = sum[r][c];
+            } else {
+                if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[r][c];
+            }
+        }
     }
 }
 
-template <int R, int WK>
+template <int R, int WK, int CU, bool ROWS_IN_N>
 int launch(const Geometry& g, FwdParams q, hipStream_t s)
 {
-    q.row_groups = (g.wo + R - 1) / R;
-    q.slots = (long long)g.n * q.row_groups * g.ho;
+    q.row_groups = ROWS_IN_N ? (g.n + R - 1) / R : (g.wo + R - 1) / R;
+    q.slots = ROWS_IN_N ? (long long)q.row_groups * g.ho : (long long)g.n * q.row_groups * g.ho;
     const long long tiles = (q.slots + 63) / 64;
-    long long blocks = tiles * g.n_cotile;
-    const char* e = getenv("GEO_SC_MAP");
-    q.map = e ? atoi(e) : 0;
-    if (q.map) blocks = (tiles + 7) / 8 * 8 * g.n_cotile;
+    const long long blocks = tiles * g.n_cotile;
     if (blocks <= 0 || blocks > 0x7fffffffLL) return GEO_SC_ERR_INVALID_ARGUMENT;
-    hipLaunchKernelGGL((k_conv_fwd<R, WK>), dim3((unsigned)blocks), dim3(64), 0, s, q);
+    // per-lane word offsets are 32-bit
+    if ((unsigned long long)R * g.packs * g.act_plane >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
+    if (ROWS_IN_N != g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
+    hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks), dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
@@ -203,14 +229,30 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     q.act_plane = (unsigned)g.act_plane;
     q.row_groups = 0;
     q.slots = 0;
-    // rows per lane: more rows reuse each weight word more often, but need enough lane
-    // slots to fill 256 CUs
-    const bool two_rows = g.wo >= 2;
+    q.n = g.n;
+    // Two accumulator rows per lane halve the weight traffic per instruction.  Outputs with
+    // several rows take them along dim 2 (sliding-window reuse of activation words); outputs
+    // with a single row (the SC-linear mapping, classifier layers) take two batch items.
+    if (g.wo >= 2) {
+        switch (g.w_k) {
+        case 1: return launch<2, 1, 3, false>(g, q, s);
+        case 3: return launch<2, 3, 1, false>(g, q, s);
+        case 5: return launch<2, 5, 1, false>(g, q, s);
+        default: return launch<1, 0, 1, false>(g, q, s);
+        }
+    }
+    if (g.act_item_inner) {
+        switch (g.w_k) {
+        case 1: return launch<2, 1, 3, true>(g, q, s);
+        case 3: return launch<2, 3, 1, true>(g, q, s);
+        default: return launch<2, 5, 1, true>(g, q, s);
+        }
+    }
     switch (g.w_k) {
-    case 1: return two_rows ? launch<2, 1>(g, q, s) : launch<1, 1>(g, q, s);
-    case 3: return two_rows ? launch<2, 3>(g, q, s) : launch<1, 3>(g, q, s);
-    case 5: return two_rows ? launch<2, 5>(g, q, s) : launch<1, 5>(g, q, s);
-    default: return launch<1, 0>(g, q, s);
+    case 1: return launch<1, 1, 3, false>(g, q, s);
+    case 3: return launch<1, 3, 1, false>(g, q, s);
+    case 5: return launch<1, 5, 1, false>(g, q, s);
+    default: return launch<1, 0, 1, false>(g, q, s);
     }
 }
 

@@ -108,8 +108,10 @@ __device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, const uint32_t
     __syncthreads();
 }
 
-// Activation streams [n][P][c_in][Wi][Hi] from the unpadded fp32 input; padding positions
-// produce zero words but keep their place in the seed numbering (sc.cpp:409-413).
+// Activation streams from the unpadded fp32 input; padding positions produce zero words but
+// keep their place in the seed numbering (sc.cpp:409-413).  Layout [n][P][c_in][Wi][Hi], or
+// with ITEM_INNER [P][c_in][Wi][Hi][n]; threads run along the innermost axis of the output.
+template <bool ITEM_INNER>
 __global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __restrict__ x,
                                                             uint32_t* __restrict__ streams,
                                                             const uint32_t* __restrict__ tables, GenParams gp, int n,
@@ -124,8 +126,14 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __rest
     const size_t total = (size_t)n * plane;
     const float Lf = (float)gp.L, top = (float)(gp.L - 1);
     for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
-        const uint32_t item = (uint32_t)(e / plane);
-        const uint32_t i = (uint32_t)(e - (size_t)item * plane);
+        uint32_t item, i;
+        if (ITEM_INNER) {
+            i = (uint32_t)(e / (uint32_t)n);
+            item = (uint32_t)(e - (size_t)i * n);
+        } else {
+            item = (uint32_t)(e / plane);
+            i = (uint32_t)(e - (size_t)item * plane);
+        }
         const uint32_t q = i % (uint32_t)hi;
         const uint32_t r = i / (uint32_t)hi;
         const uint32_t p = r % (uint32_t)wi;
@@ -138,8 +146,15 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __rest
             code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
         }
         const int o = (int)posp1[i % (uint32_t)(gp.L - 1)];
-        uint32_t* dst = streams + (size_t)item * gp.packs * plane + i;
-        for (int pk = 0; pk < gp.packs; pk++) dst[(size_t)pk * plane] = code ? stream_word(thr, code, o, pk, gp) : 0u;
+        if (ITEM_INNER) {
+            uint32_t* dst = streams + (size_t)i * n + item;
+            for (int pk = 0; pk < gp.packs; pk++)
+                dst[(size_t)pk * plane * n] = code ? stream_word(thr, code, o, pk, gp) : 0u;
+        } else {
+            uint32_t* dst = streams + (size_t)item * gp.packs * plane + i;
+            for (int pk = 0; pk < gp.packs; pk++)
+                dst[(size_t)pk * plane] = code ? stream_word(thr, code, o, pk, gp) : 0u;
+        }
     }
 }
 
@@ -222,8 +237,12 @@ int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, con
 {
     const GenParams gp = gen_params(g, g.load_wait_a);
     const size_t total = (size_t)g.n * g.act_plane;
-    hipLaunchKernelGGL(k_act_streams, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x, streams,
-                       tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+    if (g.act_item_inner)
+        hipLaunchKernelGGL(k_act_streams<true>, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
+                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+    else
+        hipLaunchKernelGGL(k_act_streams<false>, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
+                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

@@ -104,7 +104,9 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, c
 /*
  * The two stream generators on their own (the forward runs exactly these kernels).
  *
- * Activation streams: uint32 [n][P][c_in][Wi][Hi] over the PADDED item, P = ceil(L/32);
+ * Activation streams: uint32 [n][P][c_in][Wi][Hi] over the PADDED item, P = ceil(L/32)
+ * (when the output has a single row, Wo == 1, with n >= 2 and w_k in {1,3,5}, the same words are
+ * stored batch-item-innermost, [P][c_in][Wi][Hi][n], which is what the convolution kernel reads then);
  * element i (flat index in the padded item) starts its LFSR at i % (L-1) + 1; the register
  * advances before each comparison; bits enter MSB-first; for L < 32 a word holds L bits
  * (sc.cpp:405-438, sc_cuda_kernel.cu:662-692).

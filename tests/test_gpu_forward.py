@@ -57,6 +57,17 @@ def test_activation_streams_match_oracle(capi, so, L, loading):
         assert np.array_equal(got[n], exp), (L, loading, n)
 
 
+def test_activation_streams_item_innermost_layout(capi, so):
+    """Outputs with a single row (here 3-wide input, 3-wide kernel, no padding) get their
+    streams as [P][Cin][Wi][Hi][N]: same words, batch item innermost."""
+    L = 64
+    x, _ = wl.make_inputs((5, 4, 3, 6), (2, 4, 3, 3), "prescribed", seed=77)
+    d = capi.make_desc(x.shape, (2, 4, 3, 3), L, (0, 0))
+    got = u32(capi.act_streams(x.cuda(), d)).reshape(2, 4, 3, 6, 5)
+    for n in range(5):
+        assert np.array_equal(got[..., n], so.act_streams(x[n].numpy(), L))
+
+
 @pytest.mark.parametrize("L", LENGTHS)
 @pytest.mark.parametrize("loading", [(7, 8, 1, 1), (7, 2, 2, 2), (7, 1, 3, 5)])
 def test_weight_streams_match_oracle(capi, so, L, loading):
@@ -73,6 +84,27 @@ def test_weight_streams_match_oracle(capi, so, L, loading):
     assert np.array_equal(gp[..., :Cout], wpos)
     assert np.array_equal(gn[..., :Cout], wneg)
     assert not gp[..., Cout:].any() and not gn[..., Cout:].any()   # c_out padding is zero
+
+
+def test_conv_kernel_alone_on_oracle_streams(capi, so):
+    """The AND/OR/popcount kernel fed with streams produced by the CPU oracle; the last wave
+    is partly empty and starts in the third item."""
+    L = 64
+    x, w = wl.make_inputs((3, 5, 8, 7), (18, 5, 3, 3), "prescribed", seed=31)
+    d = capi.make_desc(x.shape, w.shape, L, (1, 1))
+    xp = np.pad(x.numpy(), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    act = np.stack([so.act_streams(xp[n], L) for n in range(x.shape[0])])           # [N][P][Cin][Wi][Hi]
+    wpos, wneg = so.weight_streams(w.numpy(), L)                                     # [P][H][Cin][W][Cout]
+    P, H, Cin, W, Cout = wpos.shape
+    K, ncot = Cin * W, (Cout + 15) // 16
+    pad_c = ncot * 16 - Cout
+    tiled = np.zeros((P, H, K, ncot, 2, 16), dtype=np.uint32)
+    tiled[..., 0, :] = np.pad(wpos.reshape(P, H, K, Cout), ((0, 0),) * 3 + ((0, pad_c),)).reshape(P, H, K, ncot, 16)
+    tiled[..., 1, :] = np.pad(wneg.reshape(P, H, K, Cout), ((0, 0),) * 3 + ((0, pad_c),)).reshape(P, H, K, ncot, 16)
+    y = capi.conv2d_add_partial_from_streams(torch.from_numpy(act.view(np.int32)).cuda(),
+                                             torch.from_numpy(tiled.view(np.int32)).cuda(), d)
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, (1, 1))
+    assert np.array_equal(y.cpu().numpy(), exp)
 
 
 # ------------------------------------------------------------------ forward: fixtures
@@ -92,6 +124,12 @@ def test_forward_matches_reference_fixtures(capi, fixtures_small):
     ((5, 16, 1, 8), (33, 16, 1, 8), (0, 0), 128, "prescribed"),  # SC-linear mapping
     ((2, 3, 11, 5), (4, 3, 3, 5), (0, 2), 8, "prescribed"),      # odd row count, L=8
     ((70, 2, 3, 3), (3, 2, 3, 3), (0, 0), 64, "sparse"),         # waves spanning items
+    ((7, 5, 3, 9), (4, 5, 3, 3), (0, 0), 64, "prescribed"),      # single output row: lanes pair up batch items (odd N)
+    ((3, 5, 5, 9), (4, 5, 5, 3), (0, 0), 32, "prescribed"),      # same with a 5-wide kernel
+    ((9, 8, 1, 6), (3, 8, 1, 2), (0, 0), 128, "prescribed"),     # 1-wide kernel, channels in trips of 3 + tail
+    ((5, 4, 4, 4), (3, 4, 4, 4), (0, 0), 32, "prescribed"),      # classifier-style layer, run-time width
+    ((1, 1, 1, 1), (1, 1, 1, 1), (0, 0), 8, "prescribed"),       # smallest possible
+    ((2, 10, 6, 6), (5, 10, 1, 1), (0, 0), 64, "kaiming"),       # 1x1 conv, 10 channels = 3 trips + 1
 ])
 def test_forward_matches_oracle(capi, so, shape_x, shape_w, pad, L, mode):
     x, w = wl.make_inputs(shape_x, shape_w, mode, seed=L + shape_x[0])
