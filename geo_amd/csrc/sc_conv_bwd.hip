@@ -28,7 +28,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kTile = 128;   // block tile in I and J
 constexpr int kChunk = 16;   // K per LDS stage
-constexpr int kLd = 130;     // LDS row stride: 8*kLd = 16 (mod 32) keeps I-major staging conflict-free
+constexpr int kLd = 132;     // LDS row stride in floats: rows stay 16-byte aligned for float4 stores
 
 enum Epilogue { EPI_STORE = 0, EPI_EXP_TIMES_G = 1 };
 
@@ -40,40 +40,91 @@ struct GemmParams {
     long long lda, ldb, ldc;  // leading dimensions (elements)
     int k_per_split;          // K range of one blockIdx.z; c advances by c_split_stride per split
     long long c_split_stride;
-    // EPI_EXP_TIMES_G: c[i][j] = g[(n*c_out + j%c_out)*npos + pos] * exp(-acc), i = n*npos + pos
+    // EPI_EXP_TIMES_G: c[i][j] = g[goff[i] + (j % c_out) * npos] * exp(-acc)
     const float* __restrict__ g;
+    const int* __restrict__ goff;
     int c_out, npos;
 };
 
-// Stage a kChunk x kTile tile of an operand into LDS as s[k][i].
-//   K-major operand: element (k, i) at p[k*ld + i]  -> rows of the tile are contiguous
-//   I-major operand: element (k, i) at p[i*ld + k]  -> each thread walks 8 consecutive k
-template <bool KMAJOR>
-__device__ __forceinline__ void stage_tile(float (*s)[kLd], const float* __restrict__ p, long long ld, int i0,
-                                           int k0, int I, int k_end)
-{
-    const int t = threadIdx.x;
-    if (KMAJOR) {
-#pragma unroll
-        for (int rep = 0; rep < 8; rep++) {
-            const int kk = rep * 2 + (t >> 7), ii = t & 127;
-            const int k = k0 + kk, i = i0 + ii;
-            s[kk][ii] = (k < k_end && i < I) ? p[(long long)k * ld + i] : 0.0f;
-        }
-    } else {
-        const int ii = t >> 1, kb = (t & 1) * 8;
-        const int i = i0 + ii;
-        const float* row = p + (long long)i * ld + k0 + kb;
-#pragma unroll
-        for (int c = 0; c < 8; c++) s[kb + c][ii] = (i < I && k0 + kb + c < k_end) ? row[c] : 0.0f;
-    }
-}
+// Staging of one kChunk x kTile operand tile, split in two so that the global loads of chunk
+// c+1 are in flight while the MFMAs of chunk c run: fetch() reads 8 elements per thread into
+// registers, commit() writes them to LDS as s[k][i].
+//   K-major operand: element (k, i) at p[k*ld + i]
+//   I-major operand: element (k, i) at p[i*ld + k]
+// VEC: the operand's leading dimension and extent along its contiguous axis are multiples of
+// 4 floats, so full chunks move as two float4 per thread; the last partial chunk and the
+// general case use guarded scalar loads (out-of-range lanes read a valid dummy address and
+// are zeroed by a select, no divergent branches).
+template <bool KMAJOR, bool VEC>
+struct Stager {
+    const float* p;      // this thread's first element of the current chunk
+    const float* dummy;  // any valid address of the operand
+    long long ld;
+    int kk0, ii;         // first k (inside the chunk) and first i (inside the tile) of this thread
+    bool i_ok;
 
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+    // element c (0..7) of this thread sits at (k, i) = (kk0 + kdelta(c), ii + idelta(c))
+    static __device__ __forceinline__ int kdelta(int c) { return KMAJOR ? (VEC ? (c >> 2) * 8 : c * 2) : c; }
+    static __device__ __forceinline__ int idelta(int c) { return KMAJOR && VEC ? (c & 3) : 0; }
+
+    __device__ __forceinline__ void init(const float* base, long long ld_, int i0, int k_begin, int I)
+    {
+        const int t = threadIdx.x;
+        ld = ld_;
+        dummy = base;
+        if (KMAJOR) {
+            if (VEC) {
+                kk0 = t >> 5;  // rows kk0 and kk0 + 8, four consecutive i
+                ii = (t & 31) * 4;
+            } else {
+                kk0 = t >> 7;  // rows kk0, kk0 + 2, ..., kk0 + 14, one i
+                ii = t & 127;
+            }
+            p = base + (long long)(k_begin + kk0) * ld + i0 + ii;
+        } else {
+            ii = t >> 1;
+            kk0 = (t & 1) * 8;  // eight consecutive k of one i
+            p = base + (long long)(i0 + ii) * ld + k_begin + kk0;
+        }
+        i_ok = i0 + ii < I;
+    }
+    // k_left = k_end - k0 of the chunk being fetched
+    __device__ __forceinline__ void fetch(float (&r)[8], int k_left)
+    {
+        if (VEC && k_left >= kChunk) {
+            const float* q0 = i_ok ? p : dummy;
+            const float* q1 = i_ok ? p + (KMAJOR ? 8 * ld : 4) : dummy;
+            const float4 v0 = *(const float4*)q0, v1 = *(const float4*)q1;
+            r[0] = i_ok ? v0.x : 0.0f; r[1] = i_ok ? v0.y : 0.0f; r[2] = i_ok ? v0.z : 0.0f; r[3] = i_ok ? v0.w : 0.0f;
+            r[4] = i_ok ? v1.x : 0.0f; r[5] = i_ok ? v1.y : 0.0f; r[6] = i_ok ? v1.z : 0.0f; r[7] = i_ok ? v1.w : 0.0f;
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const bool ok = i_ok && kk0 + kdelta(c) < k_left;
+                const float* qq = ok ? p + (KMAJOR ? (long long)kdelta(c) * ld + idelta(c) : (long long)c) : dummy;
+                const float v = *qq;
+                r[c] = ok ? v : 0.0f;
+            }
+        }
+        p += KMAJOR ? (long long)kChunk * ld : (long long)kChunk;
+    }
+    __device__ __forceinline__ void commit(float (*s)[kLd], const float (&r)[8]) const
+    {
+        if (KMAJOR && VEC) {
+            *(float4*)&s[kk0][ii] = make_float4(r[0], r[1], r[2], r[3]);
+            *(float4*)&s[kk0 + 8][ii] = make_float4(r[4], r[5], r[6], r[7]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) s[kk0 + kdelta(c)][ii] = r[c];
+        }
+    }
+};
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC>
 __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
 {
-    __shared__ float as[2][kChunk][kLd];
-    __shared__ float bs[2][kChunk][kLd];
+    __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
+    __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
     const int i0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile;
     const int k_begin = blockIdx.z * q.k_per_split;
     const int k_end = min(q.K, k_begin + q.k_per_split);
@@ -89,16 +140,24 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
 
-    int buf = 0;
+    Stager<A_KMAJOR, VEC> sa;
+    Stager<B_KMAJOR, VEC> sb;
+    sa.init(q.a, q.lda, i0, k_begin, q.I);
+    sb.init(q.b, q.ldb, j0, k_begin, q.J);
+    float ra[8], rb[8];
     if (k_begin < k_end) {
-        stage_tile<A_KMAJOR>(as[0], q.a, q.lda, i0, k_begin, q.I, k_end);
-        stage_tile<B_KMAJOR>(bs[0], q.b, q.ldb, j0, k_begin, q.J, k_end);
+        sa.fetch(ra, k_end - k_begin);
+        sb.fetch(rb, k_end - k_begin);
+        sa.commit(as[0], ra);
+        sb.commit(bs[0], rb);
     }
     __syncthreads();
+    int buf = 0;
     for (int k0 = k_begin; k0 < k_end; k0 += kChunk) {
-        if (k0 + kChunk < k_end) {
-            stage_tile<A_KMAJOR>(as[buf ^ 1], q.a, q.lda, i0, k0 + kChunk, q.I, k_end);
-            stage_tile<B_KMAJOR>(bs[buf ^ 1], q.b, q.ldb, j0, k0 + kChunk, q.J, k_end);
+        const bool more = k0 + kChunk < k_end;
+        if (more) {
+            sa.fetch(ra, k_end - k0 - kChunk);
+            sb.fetch(rb, k_end - k0 - kChunk);
         }
 #pragma unroll
         for (int kk = 0; kk < kChunk; kk += 2) {
@@ -109,6 +168,11 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
             acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
             acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (more) {
+            // the other buffer was last read one trip ago, before that trip's barrier
+            sa.commit(as[buf ^ 1], ra);
+            sb.commit(bs[buf ^ 1], rb);
         }
         __syncthreads();
         buf ^= 1;
@@ -128,34 +192,60 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
                 if (i >= q.I) continue;
                 float v = acc[x][y][r];
                 if (EPI == EPI_EXP_TIMES_G) {
-                    const int n = i / q.npos, pos = i - n * q.npos;
                     const int co = j >= q.c_out ? j - q.c_out : j;
-                    v = q.g[((long long)n * q.c_out + co) * q.npos + pos] * expf(-v);
+                    v = q.g[q.goff[i] + co * q.npos] * expf(-v);
                 }
                 c[(long long)i * q.ldc + j] = v;
             }
         }
 }
 
-// col[m][k] = x~[n, ci, a+u, b+v] for kernel row v; m = (n, a, b), k = ci*W + u; x~ is the
-// zero-padded activation, read straight from the unpadded tensor.
-__global__ __launch_bounds__(256) void k_im2col_row(const float* __restrict__ x, float* __restrict__ col, int v,
-                                                    long long total, int c_in, int w_in, int h_in, int pad_w,
-                                                    int pad_h, int w_k, int wo, int ho)
+// Per output position m = (n, a, b): where its receptive field starts in the unpadded input.
+//   base[m] = ((n*c_in)*w_in + (a - pad_w))*h_in + (b - pad_h),  arow[m] = a - pad_w,  bcol[m] = b - pad_h
+//   goff[m] = (n*c_out)*npos + (a*ho + b): index of grad_y[n][0][a][b]
+// Built once per call; it keeps integer divisions out of the per-element kernels.
+__global__ __launch_bounds__(256) void k_position_table(int* __restrict__ base, int* __restrict__ arow,
+                                                        int* __restrict__ bcol, int* __restrict__ goff, int m_total,
+                                                        int c_in, int c_out, int w_in, int h_in, int pad_w, int pad_h,
+                                                        int wo, int ho)
 {
-    const int k_or = c_in * w_k;
-    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)gridDim.x * 256) {
-        const int k = (int)(e % k_or);
-        const long long m = e / k_or;
-        const int b = (int)(m % ho);
-        const long long t = m / ho;
-        const int a = (int)(t % wo);
-        const long long n = t / wo;
-        const int ci = k / w_k, u = k - ci * w_k;
-        const int p = a + u - pad_w, qq = b + v - pad_h;
-        float val = 0.0f;
-        if (p >= 0 && p < w_in && qq >= 0 && qq < h_in) val = x[((n * c_in + ci) * w_in + p) * h_in + qq];
-        col[e] = val;
+    for (int m = blockIdx.x * 256 + threadIdx.x; m < m_total; m += gridDim.x * 256) {
+        const int b = m % ho;
+        const int t = m / ho;
+        const int a = t % wo;
+        const int n = t / wo;
+        base[m] = ((n * c_in) * w_in + (a - pad_w)) * h_in + (b - pad_h);
+        arow[m] = a - pad_w;
+        bcol[m] = b - pad_h;
+        goff[m] = n * c_out * wo * ho + (m - n * wo * ho);
+    }
+}
+
+// col[k][m] = x~[n, ci, a+u, b+v] for kernel row v; k = ci*W + u, m = (n, a, b); x~ is the
+// zero-padded activation, read straight from the unpadded tensor.  blockIdx.y selects a group
+// of kIm2colChannels input channels; a thread reads its position's table entry once and moves
+// all kernel taps of those channels.  Reads and writes run along m.
+constexpr int kIm2colChannels = 4;
+__global__ __launch_bounds__(256) void k_im2col_row(const float* __restrict__ x, float* __restrict__ col,
+                                                    const int* __restrict__ base, const int* __restrict__ arow,
+                                                    const int* __restrict__ bcol, int v, int m_total, int c_in,
+                                                    int w_in, int h_in, int w_k)
+{
+    const int ci0 = blockIdx.y * kIm2colChannels;
+    const int ci1 = min(c_in, ci0 + kIm2colChannels);
+    for (int m = blockIdx.x * 256 + threadIdx.x; m < m_total; m += gridDim.x * 256) {
+        const int r0 = arow[m], c = bcol[m] + v;
+        const bool c_ok = c >= 0 && c < h_in;
+        const float* src = x + base[m] + v;
+        for (int ci = ci0; ci < ci1; ci++) {
+            float* dst = col + (size_t)ci * w_k * m_total + m;
+            for (int u = 0; u < w_k; u++) {
+                const int r = r0 + u;
+                float val = 0.0f;
+                if (c_ok && r >= 0 && r < w_in) val = src[(ci * w_in + u) * h_in];
+                dst[(size_t)u * m_total] = val;
+            }
+        }
     }
 }
 
@@ -180,19 +270,35 @@ __global__ __launch_bounds__(256) void k_weight_operands(const float* __restrict
     }
 }
 
-// dL/dw[co][ci][u][v] from the split partial sums part[s][k][j] (fixed summation order).
+// dL/dw[co][ci][u][v] from the split partial sums part[s][k][j].  A block takes 32
+// consecutive (k, co) entries; 8 groups of threads each sum every 8th split, the groups are
+// then added in a fixed order, so the result does not depend on scheduling.
 __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ part, const float* __restrict__ w,
                                                       float* __restrict__ gw, int v, int splits, int c_out, int k_or,
                                                       int h_k)
 {
+    __shared__ float red[2][8][32];
     const int total = k_or * c_out;
     const long long stride = (long long)k_or * 2 * c_out;
-    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
-        const int co = e % c_out, k = e / c_out;
-        float sp = 0.0f, sn = 0.0f;
-        for (int s = 0; s < splits; s++) {
+    const int lane = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const int e = blockIdx.x * 32 + lane;
+    const bool ok = e < total;
+    const int co = ok ? e % c_out : 0, k = ok ? e / c_out : 0;
+    float sp = 0.0f, sn = 0.0f;
+    if (ok)
+        for (int s = grp; s < splits; s += 8) {
             sp += part[s * stride + (long long)k * 2 * c_out + co];
             sn += part[s * stride + (long long)k * 2 * c_out + c_out + co];
+        }
+    red[0][grp][lane] = sp;
+    red[1][grp][lane] = sn;
+    __syncthreads();
+    if (grp == 0 && ok) {
+        sp = sn = 0.0f;
+#pragma unroll
+        for (int gidx = 0; gidx < 8; gidx++) {
+            sp += red[0][gidx][lane];
+            sn += red[1][gidx][lane];
         }
         const long long wi = ((long long)co * k_or + k) * h_k + v;
         const float wv = w[wi];
@@ -204,27 +310,28 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ 
 }
 
 // dL/dx[n][ci][p][q] (+)= sum_u dcol[ci*W+u][(n, p+pad_w-u, q+pad_h-v)] over the valid output
-// positions; the first kernel row writes, the others add.
+// positions; the first kernel row writes, the others add.  Blocks stride over the planes (n, ci).
 __global__ __launch_bounds__(256) void k_col2im_row(const float* __restrict__ dcol, float* __restrict__ gx, int v,
-                                                    long long total, long long m_total, int c_in, int w_in,
-                                                    int h_in, int pad_w, int pad_h, int w_k, int wo, int ho)
+                                                    long long m_total, int n_planes, int c_in, int w_in, int h_in,
+                                                    int pad_w, int pad_h, int w_k, int wo, int ho)
 {
-    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)gridDim.x * 256) {
-        const int qq = (int)(e % h_in);
-        long long t = e / h_in;
-        const int p = (int)(t % w_in);
-        t /= w_in;
-        const int ci = (int)(t % c_in);
-        const long long n = t / c_in;
-        const int b = qq + pad_h - v;
-        float s = 0.0f;
-        if (b >= 0 && b < ho) {
-            for (int u = 0; u < w_k; u++) {
-                const int a = p + pad_w - u;
-                if (a >= 0 && a < wo) s += dcol[(long long)(ci * w_k + u) * m_total + (n * wo + a) * ho + b];
+    const int plane = w_in * h_in;
+    for (int nc = blockIdx.x; nc < n_planes; nc += gridDim.x) {
+        const int n = nc / c_in, ci = nc - n * c_in;
+        float* dst = gx + (size_t)nc * plane;
+        const float* src = dcol + (size_t)ci * w_k * m_total + (size_t)n * wo * ho;
+        for (int e = blockIdx.y * 256 + threadIdx.x; e < plane; e += gridDim.y * 256) {
+            const int p = e / h_in, qq = e - p * h_in;
+            const int b = qq + pad_h - v;
+            float s = 0.0f;
+            if (b >= 0 && b < ho) {
+                for (int u = 0; u < w_k; u++) {
+                    const int a = p + pad_w - u;
+                    if (a >= 0 && a < wo) s += src[(size_t)u * m_total + a * ho + b];
+                }
             }
+            dst[e] = v == 0 ? s : dst[e] + s;
         }
-        gx[e] = v == 0 ? s : gx[e] + s;
     }
 }
 
@@ -239,7 +346,13 @@ template <bool AK, bool BK, int EPI>
 int launch_gemm(const GemmParams& q, int splits, hipStream_t s)
 {
     dim3 grid((q.I + kTile - 1) / kTile, (q.J + kTile - 1) / kTile, splits);
-    hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI>), grid, dim3(256), 0, s, q);
+    // float4 staging needs every row start and every chunk start on a 16-byte boundary
+    const bool a_vec = q.lda % 4 == 0 && ((uintptr_t)q.a & 15) == 0 && (AK ? q.I % 4 == 0 : true);
+    const bool b_vec = q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && (BK ? q.J % 4 == 0 : true);
+    if (a_vec && b_vec && q.k_per_split % 4 == 0)
+        hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
+    else
+        hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, false>), grid, dim3(256), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
@@ -248,7 +361,7 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 struct BwdLayout {
     long long m_total;
     int splits, m_per_split;
-    size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, bytes;
+    size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, bytes;
 };
 
 BwdLayout bwd_layout(const Geometry& g)
@@ -270,6 +383,7 @@ BwdLayout bwd_layout(const Geometry& g)
     b.off_part = o; o += align256(sizeof(float) * (size_t)b.splits * g.k_or * 2 * g.c_out);
     b.off_wcat = o; o += align256(sizeof(float) * (size_t)g.k_or * 2 * g.c_out);
     b.off_wd = o;   o += align256(sizeof(float) * (size_t)g.k_or * 2 * g.c_out);
+    b.off_pos = o;  o += 4 * align256(sizeof(int) * (size_t)b.m_total);
     b.bytes = o;
     return b;
 }
@@ -291,32 +405,42 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     float* wcat = (float*)(ws + L.off_wcat);
     float* wd = (float*)(ws + L.off_wd);
     const int M = (int)L.m_total, K = g.k_or, J = 2 * g.c_out;
-    const long long col_total = L.m_total * K;
     const long long x_total = (long long)g.n * g.c_in * g.w_in * g.h_in;
+    if (x_total > 0x7fffffffLL || g.c_in > 65535 * kIm2colChannels) return GEO_SC_ERR_UNSUPPORTED;
+    const size_t pos_stride = align256(sizeof(int) * (size_t)M) / sizeof(int);
+    int* pos_base = (int*)(ws + L.off_pos);
+    int* pos_arow = pos_base + pos_stride;
+    int* pos_bcol = pos_arow + pos_stride;
+    int* pos_goff = pos_bcol + pos_stride;
+    if ((long long)g.n * g.c_out * g.wo * g.ho > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
+    const int m_blocks = grid1d(M);
+    hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, pos_goff, M,
+                       g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
     int rc;
     for (int v = 0; v < g.h_k; v++) {
-        hipLaunchKernelGGL(k_im2col_row, dim3(grid1d(col_total)), dim3(256), 0, s, x, col, v, col_total, g.c_in,
-                           g.w_in, g.h_in, g.pad_w, g.pad_h, g.w_k, g.wo, g.ho);
+        hipLaunchKernelGGL(k_im2col_row,
+                           dim3(m_blocks > 1024 ? 1024 : m_blocks, (g.c_in + kIm2colChannels - 1) / kIm2colChannels),
+                           dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v, M, g.c_in, g.w_in, g.h_in, g.w_k);
         hipLaunchKernelGGL(k_weight_operands, dim3(grid1d((long long)K * g.c_out)), dim3(256), 0, s, w, wcat, wd, v,
                            g.c_out, g.c_in, g.w_k, g.h_k);
-        // E[m][j] = g * exp(-(col . wcat))
+        // E[m][j] = g * exp(-(col^T . wcat)), col stored [K][M]
         GemmParams q1 = {};
         q1.a = col; q1.b = wcat; q1.c = e;
         q1.I = M; q1.J = J; q1.K = K;
-        q1.lda = K; q1.ldb = J; q1.ldc = J;
+        q1.lda = M; q1.ldb = J; q1.ldc = J;
         q1.k_per_split = K; q1.c_split_stride = 0;
-        q1.g = gy; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
-        if ((rc = launch_gemm<false, true, EPI_EXP_TIMES_G>(q1, 1, s)) != GEO_SC_OK) return rc;
-        // partial Gw[s][k][j] = sum_{m in split s} col[m][k] * E[m][j]
-        GemmParams q2 = {};
-        q2.a = col; q2.b = e; q2.c = part;
-        q2.I = K; q2.J = J; q2.K = M;
-        q2.lda = K; q2.ldb = J; q2.ldc = J;
-        q2.k_per_split = L.m_per_split; q2.c_split_stride = (long long)K * J;
+        q1.g = gy; q1.goff = pos_goff; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
+        if ((rc = launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, 1, s)) != GEO_SC_OK) return rc;
         if (gw) {
-            if ((rc = launch_gemm<true, true, EPI_STORE>(q2, L.splits, s)) != GEO_SC_OK) return rc;
-            hipLaunchKernelGGL(k_reduce_wgrad, dim3(grid1d((long long)K * g.c_out)), dim3(256), 0, s, part, w, gw,
-                               v, L.splits, g.c_out, K, g.h_k);
+            // partial Gw[s][k][j] = sum_{m in split s} col[k][m] * E[m][j]
+            GemmParams q2 = {};
+            q2.a = col; q2.b = e; q2.c = part;
+            q2.I = K; q2.J = J; q2.K = M;
+            q2.lda = M; q2.ldb = J; q2.ldc = J;
+            q2.k_per_split = L.m_per_split; q2.c_split_stride = (long long)K * J;
+            if ((rc = launch_gemm<false, true, EPI_STORE>(q2, L.splits, s)) != GEO_SC_OK) return rc;
+            hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32), dim3(256), 0, s, part, w, gw, v,
+                               L.splits, g.c_out, K, g.h_k);
         }
         if (!gx) continue;
         // dcol[k][m] = sum_j wd[j][k] * E[m][j]
@@ -326,8 +450,12 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         q3.lda = K; q3.ldb = J; q3.ldc = M;
         q3.k_per_split = J; q3.c_split_stride = 0;
         if ((rc = launch_gemm<true, false, EPI_STORE>(q3, 1, s)) != GEO_SC_OK) return rc;
-        hipLaunchKernelGGL(k_col2im_row, dim3(grid1d(x_total)), dim3(256), 0, s, dcol, gx, v, x_total, L.m_total,
-                           g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, g.w_k, g.wo, g.ho);
+        const int plane_blocks = (g.w_in * g.h_in + 255) / 256;
+        const int n_planes = g.n * g.c_in;
+        const int pb = plane_blocks > 64 ? 64 : plane_blocks;
+        const int want = 256 * 16 / pb;  // a few thousand blocks in all
+        hipLaunchKernelGGL(k_col2im_row, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx, v,
+                           L.m_total, n_planes, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, g.w_k, g.wo, g.ho);
     }
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
