@@ -38,7 +38,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="C3", choices=["C1", "C3", "C4", "C5"])
+    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"],
+                    help="C3 (default): the headline layer; C2: the 4-layer SC CNN training step")
     ap.add_argument("--length", type=int, default=0, help="stream length (default: the workload's)")
     ap.add_argument("--pass", dest="passes", default="fwdbwd", choices=["fwd", "fwdbwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -102,6 +103,90 @@ def cpu_baseline(x, w, L, pad):
     return kind, threads, statistics.median(times), note
 
 
+C2_LAYERS = [  # (name, x shape, w shape, pad) of CONV_tiny_add_partial at batch 256
+    ("conv1", (256, 3, 32, 32), (32, 3, 5, 5), 2),
+    ("conv2", (256, 32, 16, 16), (32, 32, 5, 5), 2),
+    ("conv3", (256, 32, 8, 8), (64, 32, 5, 5), 2),
+    ("fc1", (256, 64, 4, 4), (10, 64, 4, 4), 0),
+]
+
+
+def bench_network_step(args, torch):
+    """4-layer SC CNN training step (network.py:126-190 topology, utils_own.py:81-114 step):
+    batch 256 synthetic 3x32x32 images U[0,1), 10 uniform random classes, stream length 64,
+    LFSR generators, progressive loading load_unit=2 / load_wait=2 (the training script's
+    defaults), Adam lr 2e-3 on full-precision master copies."""
+    from geo_amd import capi, network
+    from geo_amd import workloads as wl
+
+    L = args.length or 64
+    torch.manual_seed(0)
+    model = network.CONV_tiny_add_partial().cuda().train()
+    model.err = [L.bit_length() - 1] * 4
+    model.load_unit = [2] * 4
+    model.load_wait = [2] * 4
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand((256, 3, 32, 32), generator=g).cuda()
+    t = torch.randint(10, (256,), generator=g).cuda()
+    copies = network.make_param_copies(model)
+    opt = torch.optim.Adam(copies, lr=2e-3)
+    crit = torch.nn.CrossEntropyLoss()
+
+    def step():
+        return network.train_step(model, x.clone(), t, crit, opt, copies)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    layers = {}
+    B_total = 0
+    word_ops_total = 0.0
+    k_total = 0.0
+    for name, sx, sw, pad in C2_LAYERS:
+        xa, wa = wl.make_inputs(sx, sw, "q7", 0)
+        xa, wa = xa.cuda(), wa.cuda()
+        d = capi.make_desc(sx, sw, L, (pad, pad), 7, 2, 2, 2)
+        ws = torch.empty(capi.workspace_size(d), dtype=torch.uint8, device="cuda")
+        wsb = torch.empty(capi.backward_workspace_size(d), dtype=torch.uint8, device="cuda")
+        out = torch.empty(capi.output_shape(d), dtype=torch.int32, device="cuda")
+        gy = torch.randn(out.shape, device="cuda")
+        f = time_events(lambda: capi.conv2d_add_partial_forward(xa, wa, L, (pad, pad), out=out, workspace=ws, desc=d),
+                        args.steps, 2, torch)
+        b = time_events(lambda: capi.conv2d_add_partial_backward(xa, wa, gy, L, (pad, pad), workspace=wsb, desc=d,
+                                                                 need_grad_x=(name != "conv1")), args.steps, 2, torch)
+        act = capi.act_streams(xa, d)
+        wgt = capi.weight_streams(wa, d)
+        k = time_events(lambda: capi.conv2d_add_partial_from_streams(act, wgt, d, out=out), args.steps, 2, torch)
+        B = wl.bit_macs(sx, sw, pad, L)
+        B_total += B
+        word_ops_total += 2 * B / 32
+        k_total += sum(k) / len(k)
+        layers[name] = {"fwd_ms": sum(f) / len(f), "bwd_ms": sum(b) / len(b), "conv_kernel_ms": sum(k) / len(k),
+                        "bit_macs": B, "valu_frac": (2 * B / 32) / (sum(k) / len(k) * 1e-3) / PEAK_VALU_WORD_OPS}
+    achieved = word_ops_total / (k_total * 1e-3)
+    result = {
+        "metric": f"SC bit-MACs/sec over one training step of the 4-layer SC CNN at stream len {L}",
+        "value": B_total / (ms_per_step * 1e-3), "unit": "bit-MAC/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u32 bit-packed streams, int32 accumulate; fp32 backward",
+        "data": "synthetic (torch.manual_seed(0); images U[0,1), uniform random labels)",
+        "config": {"workload": "C2: 4-layer SC CNN (3->32 k5 @32, 32->32 k5 @16, 32->64 k5 @8, 64->10 k4 @4), batch "
+                               f"256, stream length {L}, load_unit 2 / load_wait 2, fwd+bwd+Adam step",
+                   "pass": "train step", "bit_macs_per_step": B_total},
+        "layers": layers,
+        "roofline": {"bound": "valu", "kernel": "k_conv_fwd, the four layers' launches together",
+                     "achieved": achieved / 1e12, "peak": PEAK_VALU_WORD_OPS / 1e12, "unit": "T word-op/s",
+                     "frac": achieved / PEAK_VALU_WORD_OPS, "kernel_ms_sum": k_total, "traffic": None},
+    }
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -114,6 +199,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "C2":
+        bench_network_step(args, torch)
+        return
     from geo_amd import capi
     from geo_amd import workloads as wl
 

@@ -38,8 +38,13 @@ struct GemmParams {
     float* __restrict__ c;
     int I, J, K;              // C[I][J] = sum_k A(k,i) * B(k,j)
     long long lda, ldb, ldc;  // leading dimensions (elements)
-    int k_per_split;          // K range of one blockIdx.z; c advances by c_split_stride per split
+    // blockIdx.z = batch * splits + split.  A batch member is one kernel row: its operands
+    // and result start batch_stride elements further; a split takes k_per_split of K and
+    // writes its own partial result c_split_stride further.
+    int splits;
+    int k_per_split;
     long long c_split_stride;
+    long long a_batch_stride, b_batch_stride, c_batch_stride;
     // EPI_EXP_TIMES_G: c[i][j] = g[goff[i] + (j % c_out) * npos] * exp(-acc)
     const float* __restrict__ g;
     const int* __restrict__ goff;
@@ -126,7 +131,8 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
     __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
     const int i0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile;
-    const int k_begin = blockIdx.z * q.k_per_split;
+    const int batch = blockIdx.z / q.splits, split = blockIdx.z - batch * q.splits;
+    const int k_begin = split * q.k_per_split;
     const int k_end = min(q.K, k_begin + q.k_per_split);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wave's 64x64 corner in the tile
@@ -142,8 +148,8 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
 
     Stager<A_KMAJOR, VEC> sa;
     Stager<B_KMAJOR, VEC> sb;
-    sa.init(q.a, q.lda, i0, k_begin, q.I);
-    sb.init(q.b, q.ldb, j0, k_begin, q.J);
+    sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, q.I);
+    sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, q.J);
     float ra[8], rb[8];
     if (k_begin < k_end) {
         sa.fetch(ra, k_end - k_begin);
@@ -179,7 +185,7 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
     }
 
     // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
-    float* c = q.c + (long long)blockIdx.z * q.c_split_stride;
+    float* c = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
 #pragma unroll
     for (int x = 0; x < 2; x++)
 #pragma unroll
@@ -221,24 +227,26 @@ __global__ __launch_bounds__(256) void k_position_table(int* __restrict__ base, 
     }
 }
 
-// col[k][m] = x~[n, ci, a+u, b+v] for kernel row v; k = ci*W + u, m = (n, a, b); x~ is the
-// zero-padded activation, read straight from the unpadded tensor.  blockIdx.y selects a group
-// of kIm2colChannels input channels; a thread reads its position's table entry once and moves
-// all kernel taps of those channels.  Reads and writes run along m.
+// col[v][k][m] = x~[n, ci, a+u, b+v] for kernel rows v0 + blockIdx.z; k = ci*W + u, m = (n, a, b);
+// x~ is the zero-padded activation, read straight from the unpadded tensor.  blockIdx.y selects
+// a group of kIm2colChannels input channels; a thread reads its position's table entry once
+// and moves all kernel taps of those channels.  Reads and writes run along m.
 constexpr int kIm2colChannels = 4;
-__global__ __launch_bounds__(256) void k_im2col_row(const float* __restrict__ x, float* __restrict__ col,
-                                                    const int* __restrict__ base, const int* __restrict__ arow,
-                                                    const int* __restrict__ bcol, int v, int m_total, int c_in,
-                                                    int w_in, int h_in, int w_k)
+__global__ __launch_bounds__(256) void k_im2col_rows(const float* __restrict__ x, float* __restrict__ col,
+                                                     const int* __restrict__ base, const int* __restrict__ arow,
+                                                     const int* __restrict__ bcol, int v0, int m_total, int c_in,
+                                                     int w_in, int h_in, int w_k, size_t v_stride)
 {
+    const int v = v0 + blockIdx.z;
     const int ci0 = blockIdx.y * kIm2colChannels;
     const int ci1 = min(c_in, ci0 + kIm2colChannels);
+    float* colv = col + (size_t)blockIdx.z * v_stride;
     for (int m = blockIdx.x * 256 + threadIdx.x; m < m_total; m += gridDim.x * 256) {
         const int r0 = arow[m], c = bcol[m] + v;
         const bool c_ok = c >= 0 && c < h_in;
         const float* src = x + base[m] + v;
         for (int ci = ci0; ci < ci1; ci++) {
-            float* dst = col + (size_t)ci * w_k * m_total + m;
+            float* dst = colv + (size_t)ci * w_k * m_total + m;
             for (int u = 0; u < w_k; u++) {
                 const int r = r0 + u;
                 float val = 0.0f;
@@ -249,37 +257,42 @@ __global__ __launch_bounds__(256) void k_im2col_row(const float* __restrict__ x,
     }
 }
 
-// Weight operands of kernel row v:
-//   wcat[k][j]: j < c_out -> clamp(w,0,100), j >= c_out -> -clamp(w,-100,0)   (utils_functional.py:611-612)
-//   wd[j][k]  : the same with the negative rail negated (it enters dL/dx with a minus sign)
+// Weight operands of kernel rows v0 + blockIdx.y:
+//   wcat[v][k][j]: j < c_out -> clamp(w,0,100), j >= c_out -> -clamp(w,-100,0)   (utils_functional.py:611-612)
+//   wd[v][j][k]  : the same with the negative rail negated (it enters dL/dx with a minus sign)
 __global__ __launch_bounds__(256) void k_weight_operands(const float* __restrict__ w, float* __restrict__ wcat,
-                                                         float* __restrict__ wd, int v, int c_out, int c_in, int w_k,
-                                                         int h_k)
+                                                         float* __restrict__ wd, int v0, int c_out, int c_in, int w_k,
+                                                         int h_k, size_t v_stride)
 {
     const int k_or = c_in * w_k;
     const int total = k_or * c_out;
+    const int v = v0 + blockIdx.y;
+    float* wcatv = wcat + (size_t)blockIdx.y * v_stride;
+    float* wdv = wd + (size_t)blockIdx.y * v_stride;
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
         const int co = e % c_out, k = e / c_out;
         const float wv = w[((long long)co * k_or + k) * h_k + v];
         const float wp = fminf(fmaxf(wv, 0.0f), 100.0f);
         const float wn = -fminf(fmaxf(wv, -100.0f), 0.0f);
-        wcat[(long long)k * 2 * c_out + co] = wp;
-        wcat[(long long)k * 2 * c_out + c_out + co] = wn;
-        wd[(long long)co * k_or + k] = wp;
-        wd[(long long)(c_out + co) * k_or + k] = -wn;
+        wcatv[(long long)k * 2 * c_out + co] = wp;
+        wcatv[(long long)k * 2 * c_out + c_out + co] = wn;
+        wdv[(long long)co * k_or + k] = wp;
+        wdv[(long long)(c_out + co) * k_or + k] = -wn;
     }
 }
 
-// dL/dw[co][ci][u][v] from the split partial sums part[s][k][j].  A block takes 32
-// consecutive (k, co) entries; 8 groups of threads each sum every 8th split, the groups are
-// then added in a fixed order, so the result does not depend on scheduling.
+// dL/dw[co][ci][u][v] from the split partial sums part[v][s][k][j], v = v0 + blockIdx.y.  A
+// block takes 32 consecutive (k, co) entries; 8 groups of threads each sum every 8th split,
+// the groups are then added in a fixed order, so the result does not depend on scheduling.
 __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ part, const float* __restrict__ w,
-                                                      float* __restrict__ gw, int v, int splits, int c_out, int k_or,
-                                                      int h_k)
+                                                      float* __restrict__ gw, int v0, int splits, int c_out, int k_or,
+                                                      int h_k, size_t v_stride)
 {
     __shared__ float red[2][8][32];
     const int total = k_or * c_out;
     const long long stride = (long long)k_or * 2 * c_out;
+    const int v = v0 + blockIdx.y;
+    const float* partv = part + (size_t)blockIdx.y * v_stride;
     const int lane = threadIdx.x & 31, grp = threadIdx.x >> 5;
     const int e = blockIdx.x * 32 + lane;
     const bool ok = e < total;
@@ -287,8 +300,8 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ 
     float sp = 0.0f, sn = 0.0f;
     if (ok)
         for (int s = grp; s < splits; s += 8) {
-            sp += part[s * stride + (long long)k * 2 * c_out + co];
-            sn += part[s * stride + (long long)k * 2 * c_out + c_out + co];
+            sp += partv[s * stride + (long long)k * 2 * c_out + co];
+            sn += partv[s * stride + (long long)k * 2 * c_out + c_out + co];
         }
     red[0][grp][lane] = sp;
     red[1][grp][lane] = sn;
@@ -309,11 +322,13 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ 
     }
 }
 
-// dL/dx[n][ci][p][q] (+)= sum_u dcol[ci*W+u][(n, p+pad_w-u, q+pad_h-v)] over the valid output
-// positions; the first kernel row writes, the others add.  Blocks stride over the planes (n, ci).
-__global__ __launch_bounds__(256) void k_col2im_row(const float* __restrict__ dcol, float* __restrict__ gx, int v,
-                                                    long long m_total, int n_planes, int c_in, int w_in, int h_in,
-                                                    int pad_w, int pad_h, int w_k, int wo, int ho)
+// dL/dx[n][ci][p][q] (+)= sum_{v in chunk} sum_u dcol[v][ci*W+u][(n, p+pad_w-u, q+pad_h-v)] over
+// the valid output positions; the first chunk of kernel rows writes, later chunks add.  Blocks
+// stride over the planes (n, ci).
+__global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ dcol, float* __restrict__ gx, int v0,
+                                                     int nv, long long m_total, int n_planes, int c_in, int w_in,
+                                                     int h_in, int pad_w, int pad_h, int w_k, int wo, int ho,
+                                                     size_t v_stride)
 {
     const int plane = w_in * h_in;
     for (int nc = blockIdx.x; nc < n_planes; nc += gridDim.x) {
@@ -322,15 +337,16 @@ __global__ __launch_bounds__(256) void k_col2im_row(const float* __restrict__ dc
         const float* src = dcol + (size_t)ci * w_k * m_total + (size_t)n * wo * ho;
         for (int e = blockIdx.y * 256 + threadIdx.x; e < plane; e += gridDim.y * 256) {
             const int p = e / h_in, qq = e - p * h_in;
-            const int b = qq + pad_h - v;
             float s = 0.0f;
-            if (b >= 0 && b < ho) {
+            for (int dv = 0; dv < nv; dv++) {
+                const int b = qq + pad_h - (v0 + dv);
+                if (b < 0 || b >= ho) continue;
                 for (int u = 0; u < w_k; u++) {
                     const int a = p + pad_w - u;
-                    if (a >= 0 && a < wo) s += src[(size_t)u * m_total + a * ho + b];
+                    if (a >= 0 && a < wo) s += src[dv * v_stride + (size_t)u * m_total + a * ho + b];
                 }
             }
-            dst[e] = v == 0 ? s : dst[e] + s;
+            dst[e] = v0 == 0 ? s : dst[e] + s;
         }
     }
 }
@@ -343,12 +359,12 @@ int grid1d(long long total)
 }
 
 template <bool AK, bool BK, int EPI>
-int launch_gemm(const GemmParams& q, int splits, hipStream_t s)
+int launch_gemm(const GemmParams& q, int batch, hipStream_t s)
 {
-    dim3 grid((q.I + kTile - 1) / kTile, (q.J + kTile - 1) / kTile, splits);
+    dim3 grid((q.I + kTile - 1) / kTile, (q.J + kTile - 1) / kTile, q.splits * batch);
     // float4 staging needs every row start and every chunk start on a 16-byte boundary
-    const bool a_vec = q.lda % 4 == 0 && ((uintptr_t)q.a & 15) == 0 && (AK ? q.I % 4 == 0 : true);
-    const bool b_vec = q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && (BK ? q.J % 4 == 0 : true);
+    const bool a_vec = q.lda % 4 == 0 && ((uintptr_t)q.a & 15) == 0 && q.a_batch_stride % 4 == 0 && (AK ? q.I % 4 == 0 : true);
+    const bool b_vec = q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0 && (BK ? q.J % 4 == 0 : true);
     if (a_vec && b_vec && q.k_per_split % 4 == 0)
         hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
     else
@@ -361,6 +377,8 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 struct BwdLayout {
     long long m_total;
     int splits, m_per_split;
+    int rows_per_chunk;  // kernel rows processed by one round of launches
+    size_t col_v, e_v, part_v, w_v;  // floats per kernel row of each scratch array
     size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, bytes;
 };
 
@@ -376,13 +394,27 @@ BwdLayout bwd_layout(const Geometry& g)
     if (per < 256) per = 256;
     b.m_per_split = (int)(per > 0x7fffffffLL ? 0x7fffffffLL : per);
     b.splits = (int)((b.m_total + b.m_per_split - 1) / b.m_per_split);
+    // per-row scratch, each row's part padded to 64 floats so that float4 staging stays aligned
+    auto pad64 = [](size_t v) { return (v + 63) & ~(size_t)63; };
+    b.col_v = pad64((size_t)b.m_total * g.k_or);
+    b.e_v = pad64((size_t)b.m_total * 2 * g.c_out);
+    b.part_v = pad64((size_t)b.splits * g.k_or * 2 * g.c_out);
+    b.w_v = pad64((size_t)g.k_or * 2 * g.c_out);
+    // all kernel rows in one round of launches unless that needs more than ~3 GB of scratch
+    const size_t per_row = sizeof(float) * (2 * b.col_v + b.e_v + b.part_v + 2 * b.w_v);
+    size_t rows = ((size_t)3 << 30) / per_row;
+    if (rows < 1) rows = 1;
+    if (rows > (size_t)g.h_k) rows = g.h_k;
+    if (rows * b.splits > 65535) rows = 65535 / b.splits;  // grid.z = rows * splits
+    if (rows < 1) rows = 1;
+    b.rows_per_chunk = (int)rows;
     size_t o = 0;
-    b.off_col = o;  o += align256(sizeof(float) * (size_t)b.m_total * g.k_or);
-    b.off_e = o;    o += align256(sizeof(float) * (size_t)b.m_total * 2 * g.c_out);
-    b.off_dcol = o; o += align256(sizeof(float) * (size_t)b.m_total * g.k_or);
-    b.off_part = o; o += align256(sizeof(float) * (size_t)b.splits * g.k_or * 2 * g.c_out);
-    b.off_wcat = o; o += align256(sizeof(float) * (size_t)g.k_or * 2 * g.c_out);
-    b.off_wd = o;   o += align256(sizeof(float) * (size_t)g.k_or * 2 * g.c_out);
+    b.off_col = o;  o += align256(sizeof(float) * rows * b.col_v);
+    b.off_e = o;    o += align256(sizeof(float) * rows * b.e_v);
+    b.off_dcol = o; o += align256(sizeof(float) * rows * b.col_v);
+    b.off_part = o; o += align256(sizeof(float) * rows * b.part_v);
+    b.off_wcat = o; o += align256(sizeof(float) * rows * b.w_v);
+    b.off_wd = o;   o += align256(sizeof(float) * rows * b.w_v);
     b.off_pos = o;  o += 4 * align256(sizeof(int) * (size_t)b.m_total);
     b.bytes = o;
     return b;
@@ -407,55 +439,66 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     const int M = (int)L.m_total, K = g.k_or, J = 2 * g.c_out;
     const long long x_total = (long long)g.n * g.c_in * g.w_in * g.h_in;
     if (x_total > 0x7fffffffLL || g.c_in > 65535 * kIm2colChannels) return GEO_SC_ERR_UNSUPPORTED;
+    if ((long long)g.n * g.c_out * g.wo * g.ho > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
     const size_t pos_stride = align256(sizeof(int) * (size_t)M) / sizeof(int);
     int* pos_base = (int*)(ws + L.off_pos);
     int* pos_arow = pos_base + pos_stride;
     int* pos_bcol = pos_arow + pos_stride;
     int* pos_goff = pos_bcol + pos_stride;
-    if ((long long)g.n * g.c_out * g.wo * g.ho > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
     const int m_blocks = grid1d(M);
     hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, pos_goff, M,
                        g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
     int rc;
-    for (int v = 0; v < g.h_k; v++) {
-        hipLaunchKernelGGL(k_im2col_row,
-                           dim3(m_blocks > 1024 ? 1024 : m_blocks, (g.c_in + kIm2colChannels - 1) / kIm2colChannels),
-                           dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v, M, g.c_in, g.w_in, g.h_in, g.w_k);
-        hipLaunchKernelGGL(k_weight_operands, dim3(grid1d((long long)K * g.c_out)), dim3(256), 0, s, w, wcat, wd, v,
-                           g.c_out, g.c_in, g.w_k, g.h_k);
-        // E[m][j] = g * exp(-(col^T . wcat)), col stored [K][M]
+    for (int v0 = 0; v0 < g.h_k; v0 += L.rows_per_chunk) {
+        const int nv = g.h_k - v0 < L.rows_per_chunk ? g.h_k - v0 : L.rows_per_chunk;
+        hipLaunchKernelGGL(k_im2col_rows,
+                           dim3(m_blocks > 1024 ? 1024 : m_blocks, (g.c_in + kIm2colChannels - 1) / kIm2colChannels, nv),
+                           dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, g.c_in, g.w_in, g.h_in,
+                           g.w_k, L.col_v);
+        {
+            int wb = grid1d((long long)K * g.c_out);
+            hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
+                               g.c_out, g.c_in, g.w_k, g.h_k, L.w_v);
+        }
+        // E[v][m][j] = g * exp(-(col_v^T . wcat_v)), col stored [K][M]
         GemmParams q1 = {};
         q1.a = col; q1.b = wcat; q1.c = e;
         q1.I = M; q1.J = J; q1.K = K;
         q1.lda = M; q1.ldb = J; q1.ldc = J;
-        q1.k_per_split = K; q1.c_split_stride = 0;
+        q1.splits = 1; q1.k_per_split = K; q1.c_split_stride = 0;
+        q1.a_batch_stride = (long long)L.col_v; q1.b_batch_stride = (long long)L.w_v;
+        q1.c_batch_stride = (long long)L.e_v;
         q1.g = gy; q1.goff = pos_goff; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
-        if ((rc = launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, 1, s)) != GEO_SC_OK) return rc;
+        if ((rc = launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, nv, s)) != GEO_SC_OK) return rc;
         if (gw) {
-            // partial Gw[s][k][j] = sum_{m in split s} col[k][m] * E[m][j]
+            // partial Gw[v][s][k][j] = sum_{m in split s} col_v[k][m] * E_v[m][j]
             GemmParams q2 = {};
             q2.a = col; q2.b = e; q2.c = part;
             q2.I = K; q2.J = J; q2.K = M;
             q2.lda = M; q2.ldb = J; q2.ldc = J;
-            q2.k_per_split = L.m_per_split; q2.c_split_stride = (long long)K * J;
-            if ((rc = launch_gemm<false, true, EPI_STORE>(q2, L.splits, s)) != GEO_SC_OK) return rc;
-            hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32), dim3(256), 0, s, part, w, gw, v,
-                               L.splits, g.c_out, K, g.h_k);
+            q2.splits = L.splits; q2.k_per_split = L.m_per_split; q2.c_split_stride = (long long)K * J;
+            q2.a_batch_stride = (long long)L.col_v; q2.b_batch_stride = (long long)L.e_v;
+            q2.c_batch_stride = (long long)L.part_v;
+            if ((rc = launch_gemm<false, true, EPI_STORE>(q2, nv, s)) != GEO_SC_OK) return rc;
+            hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
+                               L.splits, g.c_out, K, g.h_k, L.part_v);
         }
         if (!gx) continue;
-        // dcol[k][m] = sum_j wd[j][k] * E[m][j]
+        // dcol[v][k][m] = sum_j wd_v[j][k] * E_v[m][j]
         GemmParams q3 = {};
         q3.a = wd; q3.b = e; q3.c = dcol;
         q3.I = K; q3.J = M; q3.K = J;
         q3.lda = K; q3.ldb = J; q3.ldc = M;
-        q3.k_per_split = J; q3.c_split_stride = 0;
-        if ((rc = launch_gemm<true, false, EPI_STORE>(q3, 1, s)) != GEO_SC_OK) return rc;
+        q3.splits = 1; q3.k_per_split = J; q3.c_split_stride = 0;
+        q3.a_batch_stride = (long long)L.w_v; q3.b_batch_stride = (long long)L.e_v;
+        q3.c_batch_stride = (long long)L.col_v;
+        if ((rc = launch_gemm<true, false, EPI_STORE>(q3, nv, s)) != GEO_SC_OK) return rc;
         const int plane_blocks = (g.w_in * g.h_in + 255) / 256;
         const int n_planes = g.n * g.c_in;
         const int pb = plane_blocks > 64 ? 64 : plane_blocks;
         const int want = 256 * 16 / pb;  // a few thousand blocks in all
-        hipLaunchKernelGGL(k_col2im_row, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx, v,
-                           L.m_total, n_planes, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, g.w_k, g.wo, g.ho);
+        hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx, v0,
+                           nv, L.m_total, n_planes, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, g.w_k, g.wo, g.ho, L.col_v);
     }
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }

@@ -27,6 +27,7 @@ struct FwdParams {
     int row_groups;        // ceil(wo / R), or ceil(n / R) when the rows of a lane are batch items
     long long slots;       // lane slots: n * row_groups * ho, or row_groups * ho
     unsigned act_plane;    // c_in * wi * hi
+    int pv_per_block;      // (pack, kernel row) pairs per blockIdx.y
 };
 
 // acc |= a & w with w wave-uniform: a single v_and_or_b32 whose first source is the SGPR.
@@ -129,8 +130,13 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 #pragma unroll
         for (int c = 0; c < C; c++) sum[r][c] = 0;
 
-    for (int p = 0; p < q.packs; p++) {
-        for (int v = 0; v < q.h_k; v++) {
+    // (pack, kernel row) pairs are independent partial sums: blockIdx.y takes a contiguous
+    // range of them when the launch is split to fill the GPU
+    const int pv_begin = blockIdx.y * q.pv_per_block;
+    const int pv_end = min(q.packs * q.h_k, pv_begin + q.pv_per_block);
+    {
+        for (int pv = pv_begin; pv < pv_end; pv++) {
+            const int p = pv / q.h_k, v = pv - p * q.h_k;
             uint32_t orp[R][C], orn[R][C];
 #pragma unroll
             for (int r = 0; r < R; r++)
@@ -183,14 +189,20 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
         int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if (ROWS_IN_N) {
-                if (n + (long long)r * q.row_groups < q.n)
-                    yo[(size_t)r * q.row_groups * q.c_out * out_plane] = sum[r][c];
-            } else {
-                if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[r][c];
-            }
+            const bool row_ok = ROWS_IN_N ? n + (long long)r * q.row_groups < q.n : a0 + r < q.wo;
+            int32_t* dst = yo + (ROWS_IN_N ? (size_t)r * q.row_groups * q.c_out * out_plane : (size_t)r * q.ho);
+            if (!row_ok) continue;
+            if (gridDim.y == 1)
+                *dst = sum[r][c];
+            else
+                atomicAdd(dst, sum[r][c]);  // integer adds: order does not matter
         }
     }
+}
+
+__global__ __launch_bounds__(256) void k_zero_i32(int32_t* __restrict__ p, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0;
 }
 
 template <int R, int WK, int CU, bool ROWS_IN_N>
@@ -204,7 +216,22 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     // per-lane word offsets are 32-bit
     if ((unsigned long long)R * g.packs * g.act_plane >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
     if (ROWS_IN_N != g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
-    hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks), dim3(64), 0, s, q);
+    // Few waves (small layers): split the (pack, kernel row) sum over blockIdx.y until about four
+    // waves per SIMD exist; the partial sums meet in y through integer atomics.
+    const int pv = g.packs * g.h_k;
+    int splits = 1;
+    if (blocks < 2048) {
+        splits = (int)((4096 + blocks - 1) / blocks);
+        if (splits > pv) splits = pv;
+    }
+    q.pv_per_block = (pv + splits - 1) / splits;
+    splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
+    if (splits > 1) {
+        const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
+        size_t zb = (n_out + 255) / 256;
+        hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
+    }
+    hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
