@@ -130,6 +130,132 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 #pragma unroll
         for (int c = 0; c < C; c++) sum[r][c] = 0;
 
+    for (int p = 0; p < q.packs; p++) {
+        for (int v = 0; v < q.h_k; v++) {
+            uint32_t orp[R][C], orn[R][C];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int c = 0; c < C; c++) orp[r][c] = orn[r][c] = 0u;
+
+            const uint32_t* ap = act_n + (size_t)p * pack_stride + (size_t)v * v_stride;
+            const uint32_t* wp = q.wgt + ((size_t)(p * q.h_k + v) * k_or * q.n_cotile + cot) * (2 * C);
+
+            if constexpr (WK > 0) {
+                int ci = 0;
+                for (; ci + CU <= q.c_in; ci += CU)
+                    or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, ch_stride, k_stride);
+                if constexpr (CU > 1)
+                    for (; ci < q.c_in; ci++)
+                        or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, ch_stride, k_stride);
+            } else {
+                for (int ci = 0; ci < q.c_in; ci++) {
+                    for (int u = 0; u < q.w_k; u++) {
+                        uint32_t wv[2 * C];
+#pragma unroll
+                        for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
+                        int row = a0 + u;
+                        row = row < q.wi ? row : q.wi - 1;
+                        const uint32_t aw = ap[(unsigned)row * q.hi];
+#pragma unroll
+                        for (int c = 0; c < C; c++) {
+                            and_or(orp[0][c], aw, wv[c]);
+                            and_or(orn[0][c], aw, wv[C + c]);
+                        }
+                        wp += k_stride;
+                    }
+                    ap += ch_stride;
+                }
+            }
+            // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int c = 0; c < C; c++) sum[r][c] += __popc(orp[r][c]) - __popc(orn[r][c]);
+        }
+    }
+
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const int co = cot * C + c;
+        if (co >= q.c_out) break;
+        int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (ROWS_IN_N) {
+                if (n + (long long)r * q.row_groups < q.n)
+                    yo[(size_t)r * q.row_groups * q.c_out * out_plane] = sum[r][c];
+            } else {
+                if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[r][c];
+            }
+        }
+    }
+}
+
+// The same kernel for launches that are split over blockIdx.y: each workgroup sums a
+// contiguous range of (pack, kernel row) pairs and adds its partial result to y with integer
+// atomics (y is zeroed first).  Used for small layers that would otherwise leave most of the
+// GPU idle.
+// Template parameters:
+//   R   rows of accumulators per lane.  ROWS_IN_N == false: R consecutive output rows a
+//       (dim 2) of one item; the WK kernel taps slide over R+WK-1 activation words, so each
+//       word is loaded once per channel.  ROWS_IN_N == true (outputs with a single row, e.g.
+//       the SC-linear mapping): R consecutive batch items.
+//   WK  kernel extent in dim 2 (0: run-time extent, R == 1).
+//   CU  input channels per loop trip, chosen so that a trip holds ~192 and-or instructions.
+template <int R, int WK, int CU, bool ROWS_IN_N>
+__global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
+{
+    constexpr int C = kCoTile;
+    static_assert(WK > 0 || (R == 1 && !ROWS_IN_N), "run-time kernel extent handles one row per lane");
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long slot0 = (long long)(blockIdx.x / q.n_cotile) * 64 + threadIdx.x;
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : 0;
+    // lane slot -> (first item n, first output row a0, output column b).  With ROWS_IN_N the
+    // R rows of a lane are items n and n + row_groups, consecutive lanes are consecutive
+    // items, and the activation streams are stored item-innermost.
+    const int b = ROWS_IN_N ? (int)(slot / q.row_groups) : (int)(slot % q.ho);
+    const long long t = slot / q.ho;
+    const int a0 = ROWS_IN_N ? 0 : (int)(t % q.row_groups) * R;
+    const long long n = ROWS_IN_N ? slot % q.row_groups : t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
+
+    constexpr int NW = WK == 0 ? 1 : (ROWS_IN_N ? R * WK : R + WK - 1);
+    // word offsets inside one channel plane.  Rows past the end (partial last group) are
+    // clamped to valid ones: they only feed outputs that are never stored.
+    unsigned off[NW];
+    if constexpr (WK > 0) {
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            if (ROWS_IN_N) {
+                const int r = j / WK, u = j % WK;
+                off[j] = (n + (long long)r * q.row_groups < q.n ? (unsigned)r * q.row_groups : 0u) +
+                         (unsigned)u * q.hi * q.n;
+            } else {
+                const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+                off[j] = (unsigned)row * q.hi;
+            }
+        }
+    } else {
+        off[0] = 0;
+    }
+    // strides (words) of one pack, one kernel row step, one channel
+    const size_t pack_stride = ROWS_IN_N ? (size_t)q.act_plane * q.n : (size_t)q.act_plane;
+    const unsigned v_stride = ROWS_IN_N ? (unsigned)q.n : 1u;
+    const unsigned ch_stride = ROWS_IN_N ? (unsigned)q.wi * q.hi * q.n : (unsigned)q.wi * q.hi;
+    const uint32_t* act_n = ROWS_IN_N ? q.act + (size_t)b * q.n + n : q.act + (size_t)n * item_stride + b;
+    const int k_or = q.c_in * q.w_k;
+    const unsigned k_stride = (unsigned)q.n_cotile * 2 * C;
+
+    int sum[R][C];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int c = 0; c < C; c++) sum[r][c] = 0;
+
     // (pack, kernel row) pairs are independent partial sums: blockIdx.y takes a contiguous
     // range of them when the launch is split to fill the GPU
     const int pv_begin = blockIdx.y * q.pv_per_block;
@@ -192,10 +318,7 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
             const bool row_ok = ROWS_IN_N ? n + (long long)r * q.row_groups < q.n : a0 + r < q.wo;
             int32_t* dst = yo + (ROWS_IN_N ? (size_t)r * q.row_groups * q.c_out * out_plane : (size_t)r * q.ho);
             if (!row_ok) continue;
-            if (gridDim.y == 1)
-                *dst = sum[r][c];
-            else
-                atomicAdd(dst, sum[r][c]);  // integer adds: order does not matter
+            atomicAdd(dst, sum[r][c]);  // integer adds: order does not matter
         }
     }
 }
@@ -212,6 +335,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     q.slots = ROWS_IN_N ? (long long)q.row_groups * g.ho : (long long)g.n * q.row_groups * g.ho;
     const long long tiles = (q.slots + 63) / 64;
     const long long blocks = tiles * g.n_cotile;
+    const long long waves = blocks;
     if (blocks <= 0 || blocks > 0x7fffffffLL) return GEO_SC_ERR_INVALID_ARGUMENT;
     // per-lane word offsets are 32-bit
     if ((unsigned long long)R * g.packs * g.act_plane >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
@@ -220,8 +344,8 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     // waves per SIMD exist; the partial sums meet in y through integer atomics.
     const int pv = g.packs * g.h_k;
     int splits = 1;
-    if (blocks < 2048) {
-        splits = (int)((4096 + blocks - 1) / blocks);
+    if (waves < 2048) {
+        splits = (int)((4096 + waves - 1) / waves);
         if (splits > pv) splits = pv;
     }
     q.pv_per_block = (pv + splits - 1) / splits;
@@ -231,7 +355,11 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         size_t zb = (n_out + 255) / 256;
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
     }
-    hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s, q);
+    if (splits > 1)
+        hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
+                           0, s, q);
+    else
+        hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks), dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
