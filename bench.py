@@ -63,6 +63,17 @@ def time_events(fn, steps, warmup, torch):
     return [a.elapsed_time(b) for a, b in evs]
 
 
+def measured_traffic(workload, L):
+    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 counters
+    (profiles/traffic.json); None for a workload that has not been profiled."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f).get(f"{workload}_L{L}")
+    except OSError:
+        return None
+    return None if t is None else t["fetch_bytes"] + t["write_bytes"]
+
+
 def cpu_baseline(x, w, L, pad):
     """The reference's own CPU kernel (compiled from its source into oracle/_ref) when it is
     loadable here, else this repository's C restatement of it; timed on the host cores."""
@@ -263,6 +274,8 @@ def main():
     k_avg = sum(k_ms) / len(k_ms)
     word_ops = 2 * B / 32
     achieved = word_ops / (k_avg * 1e-3)
+    probe_rate = capi.probe_and_or_rate()
+    traffic = measured_traffic(args.workload, L)
     gen_ms = time_events(lambda: (capi.act_streams(xd, desc), capi.weight_streams(wd, desc)), min(args.steps, 10),
                          2, torch)
     N, Cin, Wx, Hx = xd.shape
@@ -295,13 +308,16 @@ def main():
             "peak": PEAK_VALU_WORD_OPS / 1e12,
             "unit": "T word-op/s",
             "frac": achieved / PEAK_VALU_WORD_OPS,
+            "measured_issue_rate": probe_rate / 1e12,
+            "frac_of_measured_issue_rate": achieved / probe_rate,
             "kernel_ms_avg": k_avg,
             "kernel_ms_min": min(k_ms),
             "algorithmic_word_ops": word_ops,
             "hbm_algorithmic_bytes": alg_bytes,
             "hbm_stream_bytes_read_by_kernel": stream_bytes,
-            "hbm_frac_of_peak": (stream_bytes + 4 * out.numel()) / (k_avg * 1e-3) / PEAK_HBM_BYTES,
-            "traffic": None,
+            "traffic": traffic,
+            "hbm_frac_of_peak": (traffic if traffic else stream_bytes + 4 * out.numel()) / (k_avg * 1e-3)
+                                / PEAK_HBM_BYTES,
         },
         "stages_ms": {"stream_generation": sum(gen_ms) / len(gen_ms), "conv_kernel": k_avg, "backward": bwd_avg},
         "backward_flops": {"algorithmic": 12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H,

@@ -158,3 +158,22 @@ def conv2d_add_partial_backward(x, w, grad_y, bit_length=128, padding=(0, 0), ne
                                                             _stream_ptr(stream)),
            "geo_sc_conv2d_add_partial_backward")
     return gx, gw
+
+
+def probe_and_or_rate(iters=20000, stream=None):
+    """Sustained v_and_or_b32 rate (32-bit lane operations per second) of a memory-free loop,
+    timed with events on the launch stream."""
+    scratch = torch.zeros(128 + 4096 * 64 * 4, dtype=torch.uint8, device="cuda")
+    ops = ctypes.c_double(0)
+
+    def launch(n):
+        _check(_native.lib().geo_sc_probe_and_or_rate(n, _ptr(scratch), scratch.numel(), ctypes.byref(ops),
+                                                      _stream_ptr(stream)), "geo_sc_probe_and_or_rate")
+    launch(200)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    launch(iters)
+    e1.record()
+    torch.cuda.synchronize()
+    return ops.value / (e0.elapsed_time(e1) * 1e-3)

@@ -154,6 +154,16 @@ GEO_SC_API int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, 
                                                   const float* grad_y, float* grad_x, float* grad_w,
                                                   void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: enqueues a loop of `iters` x 64
+ * v_and_or_b32 instructions per wave (SGPR weight operand, no memory traffic) on 4 waves per
+ * SIMD of 256 CUs and reports in *word_ops how many 32-bit lane operations that is; the
+ * caller times it.  scratch: at least 128 + 4096*64*4 bytes of device memory (its first 128
+ * bytes are read as operands, any content).
+ */
+GEO_SC_API int geo_sc_probe_and_or_rate(int iters, void* scratch, size_t scratch_bytes, double* word_ops,
+                                        geo_sc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
