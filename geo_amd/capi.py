@@ -27,15 +27,22 @@ def _check(status: int, what: str):
         raise GeoScError(status, what)
 
 
+# enum geo_sc_accumulate
+ACCUMULATE = {"y": 0, "z": 1, "yz": 2}
+
+
 def make_desc(x_shape, w_shape, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
-              load_wait_a=1) -> ConvDesc:
-    """``padding=(p0, p1)`` follows the reference: p0 pads the last dim, p1 the one before."""
+              load_wait_a=1, accumulate="y", z_unit=1) -> ConvDesc:
+    """``padding=(p0, p1)`` follows the reference: p0 pads the last dim, p1 the one before.
+    ``accumulate``: "y" (OR over c_in and w_k, add over h_k), "z" (OR over the kernel window, add
+    over c_in) or "yz" (OR over ``z_unit`` channels and w_k, add over h_k and channel groups)."""
     n, c_in, w_in, h_in = (int(v) for v in x_shape)
     c_out, c_in2, w_k, h_k = (int(v) for v in w_shape)
     if c_in != c_in2:
         raise ValueError(f"channel mismatch: {c_in} vs {c_in2}")
     return ConvDesc(n, c_in, w_in, h_in, c_out, w_k, h_k, int(padding[1]), int(padding[0]), int(bit_length),
-                    int(total_width), int(load_width), int(load_wait_w), int(load_wait_a))
+                    int(total_width), int(load_width), int(load_wait_w), int(load_wait_a),
+                    ACCUMULATE[accumulate] if isinstance(accumulate, str) else int(accumulate), int(z_unit))
 
 
 def _stream_ptr(stream=None):
@@ -68,12 +75,14 @@ def _require_gpu_f32(t, name):
 
 
 def conv2d_add_partial_forward(x, w, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
-                               load_wait_a=1, out=None, workspace=None, stream=None, desc=None):
+                               load_wait_a=1, out=None, workspace=None, stream=None, desc=None, accumulate="y",
+                               z_unit=1):
     """int32 (N, Cout, Wo, Ho) GPU tensor via geo_sc_conv2d_add_partial_forward."""
     _require_gpu_f32(x, "x")
     _require_gpu_f32(w, "w")
     if desc is None:
-        desc = make_desc(x.shape, w.shape, bit_length, padding, total_width, load_width, load_wait_w, load_wait_a)
+        desc = make_desc(x.shape, w.shape, bit_length, padding, total_width, load_width, load_wait_w, load_wait_a,
+                         accumulate, z_unit)
     ws_bytes = workspace_size(desc)
     if workspace is None:
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
@@ -107,7 +116,8 @@ def act_streams(x, desc: ConvDesc, stream=None):
 
 
 def weight_streams(w, desc: ConvDesc, stream=None):
-    """int32-typed tensor of stream words [P][H][Cin*W][ceil(Cout/16)][2][16]."""
+    """int32-typed tensor of stream words [P][H][Cin*W][ceil(Cout/16)][2][16] (the line order
+    inside a pack depends on the accumulation mode; the shape is that of mode "y")."""
     _require_gpu_f32(w, "w")
     n = ctypes.c_size_t(0)
     _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
@@ -139,14 +149,14 @@ def backward_workspace_size(desc: ConvDesc) -> int:
 
 
 def conv2d_add_partial_backward(x, w, grad_y, bit_length=128, padding=(0, 0), need_grad_x=True, need_grad_w=True,
-                                workspace=None, stream=None, desc=None):
+                                workspace=None, stream=None, desc=None, accumulate="y", z_unit=1):
     """(grad_x, grad_w) of the surrogate via geo_sc_conv2d_add_partial_backward; an output
     that is not needed is returned as None."""
     _require_gpu_f32(x, "x")
     _require_gpu_f32(w, "w")
     _require_gpu_f32(grad_y, "grad_y")
     if desc is None:
-        desc = make_desc(x.shape, w.shape, bit_length, padding)
+        desc = make_desc(x.shape, w.shape, bit_length, padding, accumulate=accumulate, z_unit=z_unit)
     if tuple(grad_y.shape) != output_shape(desc):
         raise ValueError(f"grad_y has shape {tuple(grad_y.shape)}, expected {output_shape(desc)}")
     if workspace is None:

@@ -44,6 +44,12 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     g->load_width = d->load_width > g->total_width + 1 ? g->total_width + 1 : d->load_width;
     g->load_wait_w = d->load_wait_w;
     g->load_wait_a = d->load_wait_a;
+    if (d->accumulate < GEO_SC_ACC_Y || d->accumulate > GEO_SC_ACC_YZ) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (d->accumulate == GEO_SC_ACC_YZ && d->z_unit < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
+    g->mode = d->accumulate;
+    g->z_unit = (d->accumulate == GEO_SC_ACC_YZ && d->z_unit < d->c_in) ? d->z_unit : d->c_in;
+    // YZ with a single channel group is exactly Y (same seeds, same groups)
+    if (g->mode == GEO_SC_ACC_YZ && g->z_unit == d->c_in) g->mode = GEO_SC_ACC_Y;
     const long long wi = (long long)d->w_in + 2LL * d->pad_w, hi = (long long)d->h_in + 2LL * d->pad_h;
     const long long wo = wi - d->w_k + 1, ho = hi - d->h_k + 1;
     if (wo < 1 || ho < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
@@ -59,7 +65,19 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     g->n_cotile = (d->c_out + kCoTile - 1) / kCoTile;
     g->act_plane = (size_t)plane;
     g->act_words = (size_t)d->n * g->packs * g->act_plane;
-    g->act_item_inner = wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
+    if (g->mode == GEO_SC_ACC_Z) {
+        g->add_outer = 1;
+        g->add_inner = d->c_in;
+        g->or_ch_total = d->h_k;
+        g->or_ch_per_group = d->h_k;
+    } else {
+        g->add_outer = (d->c_in + g->z_unit - 1) / g->z_unit;
+        g->add_inner = d->h_k;
+        g->or_ch_total = d->c_in;
+        g->or_ch_per_group = g->z_unit;
+    }
+    g->seed_wrap = g->mode == GEO_SC_ACC_YZ ? (size_t)g->z_unit * wi * hi : (size_t)plane;
+    g->act_item_inner = g->mode == GEO_SC_ACC_Y && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
     g->wgt_words = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile * 2 * kCoTile;
     g->off_tables = 0;
@@ -204,6 +222,7 @@ int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float
     const int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
     if (!x || !w || !grad_y || (!grad_x && !grad_w)) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (g.mode != GEO_SC_ACC_Y) return GEO_SC_ERR_UNSUPPORTED;
     if (!workspace || workspace_bytes < backward_workspace_bytes(g) || ((uintptr_t)workspace & 255u))
         return GEO_SC_ERR_WORKSPACE;
     return launch_conv_backward(g, x, w, grad_y, grad_x, grad_w, workspace, (hipStream_t)stream);

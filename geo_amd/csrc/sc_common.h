@@ -18,6 +18,15 @@ struct Geometry {
     int n, c_in, w_in, h_in, c_out, w_k, h_k, pad_w, pad_h;
     int L, n_bits, packs, bit_unit;
     int total_width, load_width, load_wait_w, load_wait_a;
+    int mode;            // geo_sc_accumulate
+    int z_unit;          // YZ: channels per OR group, clamped to c_in; otherwise c_in
+    // Loop nest of the accumulation as the kernels walk it: for pack, for outer add group go <
+    // add_outer, for inner add group gi < add_inner: OR over (or_ch channels of the group, w_k).
+    //   Y : add_outer 1,              add_inner h_k,  OR channels = input channels
+    //   YZ: add_outer channel groups, add_inner h_k,  OR channels = the group's input channels
+    //   Z : add_outer 1,              add_inner c_in, OR channels = kernel rows (h_k)
+    int add_outer, add_inner, or_ch_total, or_ch_per_group;
+    size_t seed_wrap;    // activation seed index is (flat index % seed_wrap)
     int wi, hi;          // padded activation dims 2 / 3
     int wo, ho;          // output dims 2 / 3
     int k_or;            // OR-group size c_in * w_k

@@ -27,7 +27,11 @@ struct FwdParams {
     int row_groups;        // ceil(wo / R), or ceil(n / R) when the rows of a lane are batch items
     long long slots;       // lane slots: n * row_groups * ho, or row_groups * ho
     unsigned act_plane;    // c_in * wi * hi
-    int pv_per_block;      // (pack, kernel row) pairs per blockIdx.y
+    int pv_per_block;      // (pack, add group) pairs per blockIdx.y
+    // accumulation structure (split kernel): add groups (outer, inner), OR channels in all and
+    // per outer group, and the activation strides of an inner add step / an OR channel step
+    int add_outer, add_inner, or_ch_total, or_ch_per_group;
+    unsigned add_stride, or_stride;
 };
 
 // acc |= a & w with w wave-uniform: a single v_and_or_b32 whose first source is the SGPR.
@@ -195,9 +199,15 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 }
 
 // The same kernel for launches that are split over blockIdx.y: each workgroup sums a
-// contiguous range of (pack, kernel row) pairs and adds its partial result to y with integer
+// contiguous range of (pack, add group) pairs and adds its partial result to y with integer
 // atomics (y is zeroed first).  Used for small layers that would otherwise leave most of the
-// GPU idle.
+// GPU idle, and for the accumulation modes other than "OR over (c_in, w_k), add over h_k":
+// the add groups are (outer, inner) pairs, an outer group owning a range of OR channels
+//   Y : outer 1,              inner kernel rows,     OR channels = input channels
+//   YZ: outer channel groups, inner kernel rows,     OR channels = the group's input channels
+//   Z : outer 1,              inner input channels,  OR channels = kernel rows
+// (sc_cuda_kernel.cu:176-349), expressed through the two activation strides in FwdParams; the
+// weight lines arrive in exactly the order the loop consumes them.
 // Template parameters:
 //   R   rows of accumulators per lane.  ROWS_IN_N == false: R consecutive output rows a
 //       (dim 2) of one item; the WK kernel taps slide over R+WK-1 activation words, so each
@@ -247,7 +257,6 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
     const unsigned v_stride = ROWS_IN_N ? (unsigned)q.n : 1u;
     const unsigned ch_stride = ROWS_IN_N ? (unsigned)q.wi * q.hi * q.n : (unsigned)q.wi * q.hi;
     const uint32_t* act_n = ROWS_IN_N ? q.act + (size_t)b * q.n + n : q.act + (size_t)n * item_stride + b;
-    const int k_or = q.c_in * q.w_k;
     const unsigned k_stride = (unsigned)q.n_cotile * 2 * C;
 
     int sum[R][C];
@@ -256,31 +265,39 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
 #pragma unroll
         for (int c = 0; c < C; c++) sum[r][c] = 0;
 
-    // (pack, kernel row) pairs are independent partial sums: blockIdx.y takes a contiguous
+    // (pack, add group) pairs are independent partial sums: blockIdx.y takes a contiguous
     // range of them when the launch is split to fill the GPU
+    const int groups = q.add_outer * q.add_inner;
     const int pv_begin = blockIdx.y * q.pv_per_block;
-    const int pv_end = min(q.packs * q.h_k, pv_begin + q.pv_per_block);
+    const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
+    const unsigned add_stride = ROWS_IN_N ? v_stride : q.add_stride;
+    const unsigned or_stride = ROWS_IN_N ? ch_stride : q.or_stride;
+    const size_t lines_per_pack = (size_t)q.add_inner * q.or_ch_total * q.w_k;
     {
         for (int pv = pv_begin; pv < pv_end; pv++) {
-            const int p = pv / q.h_k, v = pv - p * q.h_k;
+            const int p = pv / groups, g = pv - p * groups;
+            const int go = g / q.add_inner, gi = g - go * q.add_inner;
+            const int ch0 = go * q.or_ch_per_group;
+            const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
             uint32_t orp[R][C], orn[R][C];
 #pragma unroll
             for (int r = 0; r < R; r++)
 #pragma unroll
                 for (int c = 0; c < C; c++) orp[r][c] = orn[r][c] = 0u;
 
-            const uint32_t* ap = act_n + (size_t)p * pack_stride + (size_t)v * v_stride;
-            const uint32_t* wp = q.wgt + ((size_t)(p * q.h_k + v) * k_or * q.n_cotile + cot) * (2 * C);
+            const uint32_t* ap = act_n + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
+            const size_t line = p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k + (size_t)gi * chs * q.w_k;
+            const uint32_t* wp = q.wgt + (line * q.n_cotile + cot) * (2 * C);
 
             if constexpr (WK > 0) {
                 int ci = 0;
-                for (; ci + CU <= q.c_in; ci += CU)
-                    or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, ch_stride, k_stride);
+                for (; ci + CU <= chs; ci += CU)
+                    or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
                 if constexpr (CU > 1)
-                    for (; ci < q.c_in; ci++)
-                        or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, ch_stride, k_stride);
+                    for (; ci < chs; ci++)
+                        or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
             } else {
-                for (int ci = 0; ci < q.c_in; ci++) {
+                for (int ci = 0; ci < chs; ci++) {
                     for (int u = 0; u < q.w_k; u++) {
                         uint32_t wv[2 * C];
 #pragma unroll
@@ -295,7 +312,7 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
                         }
                         wp += k_stride;
                     }
-                    ap += ch_stride;
+                    ap += or_stride;
                 }
             }
             // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
@@ -342,7 +359,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     if (ROWS_IN_N != g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
     // Few waves (small layers): split the (pack, kernel row) sum over blockIdx.y until about four
     // waves per SIMD exist; the partial sums meet in y through integer atomics.
-    const int pv = g.packs * g.h_k;
+    const int pv = g.packs * g.add_outer * g.add_inner;
     int splits = 1;
     if (waves < 2048) {
         splits = (int)((4096 + waves - 1) / waves);
@@ -350,12 +367,13 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     }
     q.pv_per_block = (pv + splits - 1) / splits;
     splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
-    if (splits > 1) {
+    const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y;
+    if (!plain) {
         const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
         size_t zb = (n_out + 255) / 256;
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
     }
-    if (splits > 1)
+    if (!plain)
         hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
                            0, s, q);
     else
@@ -385,6 +403,13 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     q.row_groups = 0;
     q.slots = 0;
     q.n = g.n;
+    q.add_outer = g.add_outer;
+    q.add_inner = g.add_inner;
+    q.or_ch_total = g.or_ch_total;
+    q.or_ch_per_group = g.or_ch_per_group;
+    const unsigned ch_plane = (unsigned)g.wi * g.hi;
+    q.add_stride = g.mode == GEO_SC_ACC_Z ? ch_plane : 1u;
+    q.or_stride = g.mode == GEO_SC_ACC_Z ? 1u : ch_plane;
     // Two accumulator rows per lane halve the weight traffic per instruction.  Outputs with
     // several rows take them along dim 2 (sliding-window reuse of activation words); outputs
     // with a single row (the SC-linear mapping, classifier layers) take two batch items.

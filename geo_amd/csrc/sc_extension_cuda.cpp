@@ -6,26 +6,32 @@
 using namespace geo_sc_torch;
 
 // sc_cuda.cpp:47-63.  dim != 0: y-dimension partial binary accumulation (the default of the
-// reference's training script).  dim == 0 selects z-dimension accumulation there.
+// reference's training script): OR over (c_in, w_k), add over h_k.  dim == 0: z-dimension
+// accumulation: OR over the kernel window, add over c_in.
 at::Tensor conv2d_add_partial_variable_acc(torch::Tensor input, torch::Tensor weight, int64_t bit_length,
                                            at::IntArrayRef padding, at::IntArrayRef stride, int64_t total_width,
                                            int64_t load_width, int64_t load_wait, bool im2col, int64_t dim)
 {
     (void)stride;  // accepted and ignored, as in the reference (stride 1 only)
     (void)im2col;  // selects an equivalent kernel variant in the reference; no effect on results
-    TORCH_CHECK(dim != 0, "sc_extension_cuda.conv2d_add_partial_variable_acc: z-dimension accumulation (dim=0) is "
-                          "not implemented by this library");
-    // the y/z ops use one load_wait for weights and activations (sc_cuda_kernel.cu:1821-1823)
-    const geo_sc_conv_desc d = make_desc(input, weight, bit_length, padding, total_width, load_width, load_wait, load_wait);
+    // the y/z ops use one load_wait for weights and activations (sc_cuda_kernel.cu:1821-1823, :2119)
+    const geo_sc_conv_desc d = make_desc(input, weight, bit_length, padding, total_width, load_width, load_wait,
+                                         load_wait, dim == 0 ? GEO_SC_ACC_Z : GEO_SC_ACC_Y);
     return forward_on_device(input, weight, d);
 }
 
-at::Tensor conv2d_add_yz_variable_acc(torch::Tensor, torch::Tensor, int64_t, at::IntArrayRef, at::IntArrayRef,
-                                      int64_t, int64_t, int64_t, int64_t, bool, int64_t)
+// sc_cuda.cpp:34-45: OR over (z_unit consecutive input channels, w_k), add over h_k and over
+// the channel groups; separate load_wait for the weight and activation generators.
+at::Tensor conv2d_add_yz_variable_acc(torch::Tensor input, torch::Tensor weight, int64_t bit_length,
+                                      at::IntArrayRef padding, at::IntArrayRef stride, int64_t total_width,
+                                      int64_t load_width, int64_t load_wait_w, int64_t load_wait_a, bool im2col,
+                                      int64_t z_unit)
 {
-    TORCH_CHECK(false, "sc_extension_cuda.conv2d_add_yz_variable_acc: yz accumulation is not implemented by this "
-                       "library");
-    return at::Tensor();
+    (void)stride;
+    (void)im2col;
+    const geo_sc_conv_desc d = make_desc(input, weight, bit_length, padding, total_width, load_width, load_wait_w,
+                                         load_wait_a, GEO_SC_ACC_YZ, z_unit);
+    return forward_on_device(input, weight, d);
 }
 
 at::Tensor conv2d_add_partial_acc_acc(torch::Tensor, torch::Tensor, int64_t, at::IntArrayRef, at::IntArrayRef, bool,
@@ -46,8 +52,9 @@ at::Tensor conv2d_or_acc(torch::Tensor, torch::Tensor, int64_t, at::IntArrayRef,
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     m.def("conv2d_add_partial_variable_acc", &conv2d_add_partial_variable_acc,
-          "SC forward conv2d partial (y dimension) bin add, variable load, lfsr generator");
-    m.def("conv2d_add_yz_variable_acc", &conv2d_add_yz_variable_acc, "not implemented: raises");
+          "SC forward conv2d partial (y or z dimension) bin add, variable load, lfsr generator");
+    m.def("conv2d_add_yz_variable_acc", &conv2d_add_yz_variable_acc,
+          "SC forward conv2d partial (yz dimension) bin add, variable load, lfsr generator");
     m.def("conv2d_add_partial_acc_acc", &conv2d_add_partial_acc_acc, "not implemented: raises");
     m.def("conv2d_or_acc", &conv2d_or_acc, "not implemented: raises");
 }

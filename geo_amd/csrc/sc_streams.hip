@@ -115,7 +115,8 @@ template <bool ITEM_INNER>
 __global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __restrict__ x,
                                                             uint32_t* __restrict__ streams,
                                                             const uint32_t* __restrict__ tables, GenParams gp, int n,
-                                                            int c_in, int w_in, int h_in, int pad_w, int pad_h)
+                                                            int c_in, int w_in, int h_in, int pad_w, int pad_h,
+                                                            uint32_t seed_wrap)
 {
     extern __shared__ uint32_t lds[];
     load_tables_to_lds(lds, tables, gp.L, gp.wpc);
@@ -145,7 +146,9 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __rest
             // ceil(clamp(x*L, 0, L-1))  (sc.cpp:301)
             code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
         }
-        const int o = (int)posp1[i % (uint32_t)(gp.L - 1)];
+        // seed index: flat position in the item, restarting per channel group when seed_wrap is
+        // smaller than the item (sc_cuda_kernel.cu:1080)
+        const int o = (int)posp1[(i % seed_wrap) % (uint32_t)(gp.L - 1)];
         if (ITEM_INNER) {
             uint32_t* dst = streams + (size_t)i * n + item;
             for (int pk = 0; pk < gp.packs; pk++)
@@ -197,6 +200,57 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __r
     }
 }
 
+// Weight streams of the grouped accumulation modes, same line format, lines ordered as the
+// convolution kernel consumes them: [P][outer add group][inner add group][OR channel of the
+// group][w_k].  z_mode: inner group = input channel, OR channel = kernel row, seed index
+// u*h_k + v (sc_cuda_kernel.cu:322-324).  Otherwise: outer group = block of zu input channels,
+// inner group = kernel row, seed index (channel within the block)*w_k + u (:232).
+__global__ __launch_bounds__(kGenThreads) void k_weight_streams_grouped(
+    const float* __restrict__ w, uint32_t* __restrict__ streams, const uint32_t* __restrict__ tables, GenParams gp,
+    int c_out, int c_in, int w_k, int h_k, int n_cotile, int z_mode, int add_outer, int add_inner, int or_ch_total,
+    int zu)
+{
+    extern __shared__ uint32_t lds[];
+    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    const uint32_t* posp1 = lds;
+    const uint32_t* thr = lds + gp.L;
+    const int co_pad = n_cotile * kCoTile;
+    const size_t total = (size_t)add_outer * add_inner * zu * w_k * co_pad;
+    const size_t pack_stride = (size_t)add_inner * or_ch_total * w_k * n_cotile * 2 * kCoTile;
+    const float Lf = (float)gp.L, top = (float)(gp.L - 1);
+    for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
+        const int co = (int)(e % co_pad);
+        size_t r = e / co_pad;
+        const int u = (int)(r % w_k);
+        r /= w_k;
+        const int cl = (int)(r % zu);
+        r /= zu;
+        const int gi = (int)(r % add_inner);
+        const int go = (int)(r / add_inner);
+        const int ch0 = go * zu;
+        const int chs = min(zu, or_ch_total - ch0);
+        if (cl >= chs) continue;  // ragged last group: no padding lines
+        const int ci = z_mode ? gi : ch0 + cl;
+        const int v = z_mode ? cl : gi;
+        const int sidx = z_mode ? u * h_k + v : cl * w_k + u;
+        int cp = 0, cn = 0;
+        if (co < c_out) {
+            const float wv = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v];
+            const float t = wv * Lf;
+            cp = (int)ceilf(fminf(fmaxf(t, 0.0f), top));
+            cn = (int)ceilf(-fminf(fmaxf(t, -top), 0.0f));
+        }
+        const int op = (int)posp1[(67 + sidx) % (gp.L - 1)];
+        const int on = (int)posp1[(37 + sidx) % (gp.L - 1)];
+        const size_t line = (size_t)ch0 * add_inner * w_k + (size_t)gi * chs * w_k + (size_t)cl * w_k + u;
+        const size_t base = (line * n_cotile + co / kCoTile) * (2 * kCoTile) + (co % kCoTile);
+        for (int pk = 0; pk < gp.packs; pk++) {
+            streams[pk * pack_stride + base] = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
+            streams[pk * pack_stride + base + kCoTile] = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+        }
+    }
+}
+
 GenParams gen_params(const Geometry& g, int load_wait)
 {
     GenParams gp;
@@ -237,12 +291,13 @@ int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, con
 {
     const GenParams gp = gen_params(g, g.load_wait_a);
     const size_t total = (size_t)g.n * g.act_plane;
+    const uint32_t wrap = (uint32_t)g.seed_wrap;
     if (g.act_item_inner)
         hipLaunchKernelGGL(k_act_streams<true>, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
-                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     else
         hipLaunchKernelGGL(k_act_streams<false>, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
-                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
@@ -250,6 +305,14 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
                           hipStream_t s)
 {
     const GenParams gp = gen_params(g, g.load_wait_w);
+    if (g.mode != GEO_SC_ACC_Y) {
+        const size_t padded =
+            (size_t)g.add_outer * g.add_inner * g.or_ch_per_group * g.w_k * g.n_cotile * kCoTile;
+        hipLaunchKernelGGL(k_weight_streams_grouped, dim3(grid_for(padded)), dim3(kGenThreads), table_bytes(g.L), s,
+                           w, streams, tables, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile,
+                           g.mode == GEO_SC_ACC_Z ? 1 : 0, g.add_outer, g.add_inner, g.or_ch_total, g.or_ch_per_group);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
     const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
     hipLaunchKernelGGL(k_weight_streams, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, w, streams,
                        tables, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile);

@@ -20,7 +20,8 @@ inline void check_status(int rc, const char* what)
 
 inline geo_sc_conv_desc make_desc(const at::Tensor& input, const at::Tensor& weight, int64_t bit_length,
                                   at::IntArrayRef padding, int64_t total_width, int64_t load_width,
-                                  int64_t load_wait_w, int64_t load_wait_a)
+                                  int64_t load_wait_w, int64_t load_wait_a, int accumulate = GEO_SC_ACC_Y,
+                                  int64_t z_unit = 1)
 {
     TORCH_CHECK(input.dim() == 4, "input must be (N, C_in, W, H), got ", input.dim(), " dims");
     TORCH_CHECK(weight.dim() == 4, "weight must be (C_out, C_in, W, H), got ", weight.dim(), " dims");
@@ -49,6 +50,9 @@ inline geo_sc_conv_desc make_desc(const at::Tensor& input, const at::Tensor& wei
     d.load_width = (int32_t)load_width;
     d.load_wait_w = (int32_t)load_wait_w;
     d.load_wait_a = (int32_t)load_wait_a;
+    TORCH_CHECK(z_unit >= 1, "z_units must be >= 1, got ", z_unit);
+    d.accumulate = (int32_t)accumulate;
+    d.z_unit = (int32_t)(z_unit > input.size(1) ? input.size(1) : z_unit);
     return d;
 }
 

@@ -44,6 +44,23 @@ enum geo_sc_status {
 };
 
 /*
+ * Partial binary accumulation modes of the reference's LFSR ops.  Products of one OR group
+ * are OR-ed, groups (and stream packs) are added with binary adders.
+ *   GEO_SC_ACC_Y   OR over (c_in, w_k), add over h_k: conv2d_add_partial_new (sc.cpp:292) and
+ *                  conv2d_add_partial_variable_acc with dim != 0 (sc_cuda.cpp:47-63)
+ *   GEO_SC_ACC_Z   OR over (w_k, h_k), add over c_in: conv2d_add_partial_variable_acc with
+ *                  dim == 0 (sc_cuda.cpp:57-59, sc_cuda_kernel.cu:2119-2285)
+ *   GEO_SC_ACC_YZ  OR over (z_unit consecutive input channels, w_k), add over h_k and over the
+ *                  ceil(c_in / z_unit) channel groups: conv2d_add_yz_variable_acc
+ *                  (sc_cuda.cpp:34-45, sc_cuda_kernel.cu:1971-2116)
+ * Seeds.  Weights use (67+s) % (L-1) + 1 / (37+s) % (L-1) + 1 with s = c_in_index*w_k + w_index
+ * (Y), w_index*h_k + h_index (Z, sc_cuda_kernel.cu:322-324) or (c_in_index % z_unit)*w_k +
+ * w_index (YZ, :232).  Activations use i % (L-1) + 1 with i the flat index in the padded item
+ * (Y, Z) or that index taken inside the channel group, i % (z_unit*Wi*Hi) (YZ, :1080).
+ */
+enum geo_sc_accumulate { GEO_SC_ACC_Y = 0, GEO_SC_ACC_Z = 1, GEO_SC_ACC_YZ = 2 };
+
+/*
  * Problem description shared by all entry points.
  *
  * Progressive loading (sc_cuda_kernel.cu:155-165, :681-688): at stream cycle b = 1..L the
@@ -67,6 +84,8 @@ typedef struct geo_sc_conv_desc {
     int32_t load_width;
     int32_t load_wait_w;  /* load_wait of the weight generator */
     int32_t load_wait_a;  /* load_wait of the activation generator */
+    int32_t accumulate;   /* enum geo_sc_accumulate: which products are OR-ed and which are added */
+    int32_t z_unit;       /* GEO_SC_ACC_YZ: input channels per OR group (clamped to c_in); else unused */
 } geo_sc_conv_desc;
 
 /* Library version (GEO_SC_VERSION of the build). */
@@ -105,8 +124,9 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, c
  * The two stream generators on their own (the forward runs exactly these kernels).
  *
  * Activation streams: uint32 [n][P][c_in][Wi][Hi] over the PADDED item, P = ceil(L/32)
- * (when the output has a single row, Wo == 1, with n >= 2 and w_k in {1,3,5}, the same words are
- * stored batch-item-innermost, [P][c_in][Wi][Hi][n], which is what the convolution kernel reads then);
+ * (in mode Y, when the output has a single row, Wo == 1, with n >= 2 and w_k in {1,3,5}, the same
+ * words are stored batch-item-innermost, [P][c_in][Wi][Hi][n], which is what the convolution kernel
+ * reads then);
  * element i (flat index in the padded item) starts its LFSR at i % (L-1) + 1; the register
  * advances before each comparison; bits enter MSB-first; for L < 32 a word holds L bits
  * (sc.cpp:405-438, sc_cuda_kernel.cu:662-692).
@@ -115,7 +135,9 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, c
  * row, OR-group member k = c_in_index*w_k + w_index and tile of 16 output channels, the 16
  * positive-rail words followed by the 16 negative-rail words (zero for c_out padding).
  * Seeds (67+k) % (L-1) + 1 / (37+k) % (L-1) + 1, one sequence per k shared by every h and
- * c_out (sc.cpp:336-388, sc_cuda_kernel.cu:91-170).
+ * c_out (sc.cpp:336-388, sc_cuda_kernel.cu:91-170).  Modes Z and YZ keep the line format and
+ * order the lines by (pack, add group, OR member): Z [P][c_in][h_k*w_k] with member
+ * h_index*w_k + w_index; YZ [P][channel group][h_k][channels of the group * w_k].
  *
  * `tables` is scratch of geo_sc_stream_tables_size(L) bytes.
  */

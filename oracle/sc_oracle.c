@@ -370,3 +370,90 @@ int sco_max_threads(void)
     return 1;
 #endif
 }
+
+/* ------------------------------------------------------------------------------------------
+ * The other two LFSR accumulation modes of the reference's GPU extension.  PARITY PINNED BY
+ * SPEC TEXT ONLY: the reference has no CPU code for them; this follows the CUDA source text.
+ *
+ *   mode 0  y   OR over (c_in, w), add over h                      (above; sc.cpp)
+ *   mode 1  z   OR over (w, h), add over c_in                      (sc_cuda_kernel.cu:272-349, :1141-1271)
+ *   mode 2  yz  OR over (z_unit channels, w), add over h and over
+ *               the ceil(c_in/z_unit) channel groups               (sc_cuda_kernel.cu:176-267, :1007-1138)
+ *
+ * Seeds.  Weights: index s into (67+s)%(L-1)+1 / (37+s)%(L-1)+1 is c_in*W+w (y), w*H+h (z:
+ * sc_cuda_kernel.cu:322-324), (c_in % z_unit)*W+w (yz: :232).  The reference sizes the z-mode
+ * seed array for c_in*W entries and reads past it when W*H is larger; here the same formula
+ * is simply evaluated for every (w, h).  Activations: flat index in the padded item (y, z);
+ * for yz the index wraps at z_unit*Wi*Hi (:1080), i.e. it is taken inside the channel group.
+ * z_unit is clamped to c_in (:1987).
+ * ------------------------------------------------------------------------------------------ */
+int sco_conv2d_modes(const float* x, const float* w, int32_t* y, int N, int Cin, int Wx, int Hx, int Cout, int W,
+                     int H, int pad_w, int pad_h, int L, int total_width, int load_width, int load_wait_w,
+                     int load_wait_a, int mode, int z_unit)
+{
+    int n_bits = sco_nbits_for_length(L);
+    if (n_bits < 0 || load_width < 1 || load_wait_w < 1 || load_wait_a < 1 || mode < 0 || mode > 2) return -1;
+    if (mode == 2 && z_unit < 1) return -1;
+    int Wi = Wx + 2 * pad_w, Hi = Hx + 2 * pad_h;
+    int Wo = Wi - W + 1, Ho = Hi - H + 1;
+    if (Wo < 1 || Ho < 1) return -1;
+    int P = (L + 31) / 32;
+    int zu = mode == 2 ? (z_unit < Cin ? z_unit : Cin) : Cin;
+    int zp_n = (Cin + zu - 1) / zu;
+    /* weight words [co][ci][u][v][p], both rails */
+    size_t wn_el = (size_t)Cout * Cin * W * H;
+    uint32_t* wp = (uint32_t*)malloc(sizeof(uint32_t) * wn_el * P);
+    uint32_t* wn = (uint32_t*)malloc(sizeof(uint32_t) * wn_el * P);
+    for (int co = 0; co < Cout; co++)
+        for (int ci = 0; ci < Cin; ci++)
+            for (int u = 0; u < W; u++)
+                for (int v = 0; v < H; v++) {
+                    size_t e = (((size_t)co * Cin + ci) * W + u) * H + v;
+                    int s = mode == 0 ? ci * W + u : (mode == 1 ? u * H + v : (ci % zu) * W + u);
+                    sco_stream_words(sco_code_wpos(w[e], L), (67 + s) % (L - 1) + 1, L, n_bits, total_width,
+                                     load_width, load_wait_w, wp + e * P);
+                    sco_stream_words(sco_code_wneg(w[e], L), (37 + s) % (L - 1) + 1, L, n_bits, total_width,
+                                     load_width, load_wait_w, wn + e * P);
+                }
+    size_t plane = (size_t)Cin * Wi * Hi;
+    size_t wrap = mode == 2 ? (size_t)zu * Wi * Hi : plane;
+    float* xp = (float*)malloc(sizeof(float) * plane);
+    uint32_t* A = (uint32_t*)malloc(sizeof(uint32_t) * plane * P); /* [i][p] */
+    for (int n = 0; n < N; n++) {
+        sco_pad_item(x + (size_t)n * Cin * Wx * Hx, Cin, Wx, Hx, pad_w, pad_h, xp);
+        for (size_t i = 0; i < plane; i++)
+            sco_stream_words(sco_code_act(xp[i], L), (int)((i % wrap) % (size_t)(L - 1)) + 1, L, n_bits, total_width,
+                             load_width, load_wait_a, A + i * P);
+        for (int co = 0; co < Cout; co++)
+            for (int a = 0; a < Wo; a++)
+                for (int b = 0; b < Ho; b++) {
+                    int32_t acc = 0;
+                    /* add-groups: y: v; z: ci; yz: (channel group, v) */
+                    int g_outer = mode == 1 ? Cin : zp_n;
+                    int g_inner = mode == 1 ? 1 : H;
+                    for (int go = 0; go < g_outer; go++)
+                        for (int gi = 0; gi < g_inner; gi++)
+                            for (int p = 0; p < P; p++) {
+                                uint32_t orp = 0, orn = 0;
+                                int c0 = mode == 1 ? go : go * zu;
+                                int c1 = mode == 1 ? go + 1 : (c0 + zu < Cin ? c0 + zu : Cin);
+                                int v0 = mode == 1 ? 0 : gi, v1 = mode == 1 ? H : gi + 1;
+                                for (int ci = c0; ci < c1; ci++)
+                                    for (int u = 0; u < W; u++)
+                                        for (int v = v0; v < v1; v++) {
+                                            uint32_t aw = A[(((size_t)ci * Wi + a + u) * Hi + b + v) * P + p];
+                                            size_t e = (((size_t)co * Cin + ci) * W + u) * H + v;
+                                            orp |= aw & wp[e * P + p];
+                                            orn |= aw & wn[e * P + p];
+                                        }
+                                acc += __builtin_popcount(orp) - __builtin_popcount(orn);
+                            }
+                    y[(((size_t)n * Cout + co) * Wo + a) * Ho + b] = acc;
+                }
+    }
+    free(wp);
+    free(wn);
+    free(xp);
+    free(A);
+    return 0;
+}

@@ -50,6 +50,8 @@ def lib():
     L.sco_act_streams.restype = i
     L.sco_conv2d_add_partial.argtypes = [fp, fp, ip] + [i] * 16
     L.sco_conv2d_add_partial.restype = i
+    L.sco_conv2d_modes.argtypes = [fp, fp, ip] + [i] * 16
+    L.sco_conv2d_modes.restype = i
     L.sco_max_threads.argtypes = []
     L.sco_max_threads.restype = i
     _lib = L
@@ -138,6 +140,29 @@ def conv2d_add_partial(x, w, L: int, padding=(0, 0), total_width=7, load_width=8
     rc = lib().sco_conv2d_add_partial(_ptr(x, ctypes.c_float), _ptr(w, ctypes.c_float), _ptr(y, ctypes.c_int32),
                                       N, Cin, Wx, Hx, Cout, W, H, pad_w, pad_h, L, total_width, load_width,
                                       load_wait_w, load_wait_a, int(bool(fast)), int(n_threads))
+    if rc != 0:
+        raise ValueError("unsupported stream length or bad arguments")
+    return y
+
+
+MODES = {"y": 0, "z": 1, "yz": 2}
+
+
+def conv2d_modes(x, w, L: int, padding=(0, 0), mode="y", z_unit=1, total_width=7, load_width=8, load_wait_w=1,
+                 load_wait_a=1):
+    """int32 (N,Cout,Wo,Ho) for accumulation mode "y" | "z" | "yz" (scalar loops: small shapes).
+    "z"/"yz" follow the reference's CUDA source text only (no executable reference)."""
+    x = _f32(x)
+    w = _f32(w)
+    N, Cin, Wx, Hx = x.shape
+    Cout, _, W, H = w.shape
+    pad_h, pad_w = int(padding[0]), int(padding[1])
+    Wo = Wx + 2 * pad_w - W + 1
+    Ho = Hx + 2 * pad_h - H + 1
+    y = np.zeros((N, Cout, max(Wo, 0), max(Ho, 0)), dtype=np.int32)
+    rc = lib().sco_conv2d_modes(_ptr(x, ctypes.c_float), _ptr(w, ctypes.c_float), _ptr(y, ctypes.c_int32), N, Cin, Wx,
+                                Hx, Cout, W, H, pad_w, pad_h, L, total_width, load_width, load_wait_w, load_wait_a,
+                                MODES[mode], int(z_unit))
     if rc != 0:
         raise ValueError("unsupported stream length or bad arguments")
     return y

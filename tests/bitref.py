@@ -88,3 +88,53 @@ def conv_bits(x, w, L, pad=(0, 0), tw=7, lw=8, wait_w=1, wait_a=1):
             sn += np.einsum("ncabt,oct->noabt", a, wnb[:, :, u, v, :])
         y += np.sign(sp).sum(-1) - np.sign(sn).sum(-1)
     return y
+
+
+def conv_bits_modes(x, w, L, pad=(0, 0), mode="y", z_unit=1, tw=7, lw=8, wait_w=1, wait_a=1):
+    """The accumulation modes of the reference's GPU kernels written as one dense tensor of
+    product bits T[n,o,a,b,c,u,v,t] that is OR-ed (sign of a sum) over one set of axes and
+    added over the rest.  "y": OR (c,u), add v (sc_cuda_kernel.cu:91-170); "z": OR (u,v), add c
+    (:270-349); "yz": OR (c within a block of z_unit channels, u), add v and blocks (:176-268).
+    Seed numbering per mode as in those kernels and their host code (:1080)."""
+    x = np.asarray(x, dtype=np.float32)
+    w = np.asarray(w, dtype=np.float32)
+    x = np.pad(x, ((0, 0), (0, 0), (pad[1], pad[1]), (pad[0], pad[0])))
+    N, Cin, Wi, Hi = x.shape
+    Cout, _, W, H = w.shape
+    Wo, Ho = Wi - W + 1, Hi - H + 1
+    zu = min(z_unit, Cin)
+    xa, wp, wn = codes(x, w, L)
+    abits = np.zeros((N, Cin, Wi, Hi, L), dtype=np.int64)
+    for c in range(Cin):
+        for p in range(Wi):
+            for q in range(Hi):
+                i = (c * Wi + p) * Hi + q
+                if mode == "yz":
+                    i %= zu * Wi * Hi
+                for n in range(N):
+                    abits[n, c, p, q] = bits_of(int(xa[n, c, p, q]), i % (L - 1) + 1, L, tw, lw, wait_a)
+    wbits = np.zeros((2, Cout, Cin, W, H, L), dtype=np.int64)
+    for c in range(Cin):
+        for u in range(W):
+            for v in range(H):
+                f = {"y": c * W + u, "z": u * H + v, "yz": (c % zu) * W + u}[mode]
+                for co in range(Cout):
+                    wbits[0, co, c, u, v] = bits_of(int(wp[co, c, u, v]), (67 + f) % (L - 1) + 1, L, tw, lw, wait_w)
+                    wbits[1, co, c, u, v] = bits_of(int(wn[co, c, u, v]), (37 + f) % (L - 1) + 1, L, tw, lw, wait_w)
+    y = np.zeros((N, Cout, Wo, Ho), dtype=np.int64)
+    for rail, sgn in ((0, 1), (1, -1)):
+        T = np.zeros((N, Cout, Wo, Ho, Cin, W, H, L), dtype=np.int64)
+        for u in range(W):
+            for v in range(H):
+                a = abits[:, :, u:u + Wo, v:v + Ho, :]                       # n c a b t
+                T[:, :, :, :, :, u, v, :] = np.einsum("ncabt,oct->noabct", a, wbits[rail, :, :, u, v, :])
+        if mode == "y":
+            r = np.sign(T.sum(axis=(4, 5))).sum(axis=(4, 5))
+        elif mode == "z":
+            r = np.sign(T.sum(axis=(5, 6))).sum(axis=(4, 5))
+        else:
+            r = 0
+            for c0 in range(0, Cin, zu):
+                r = r + np.sign(T[:, :, :, :, c0:c0 + zu].sum(axis=(4, 5))).sum(axis=(4, 5))
+        y += sgn * r
+    return y

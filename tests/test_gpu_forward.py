@@ -238,8 +238,6 @@ def test_torch_modules_with_reference_names(capi, so, fixtures_small):
     with pytest.raises(RuntimeError):
         sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), 100, (pad, pad), (1, 1), 7, 8, 1, False, 2)
     with pytest.raises(RuntimeError):
-        sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), 64, (pad, pad), (1, 1), 7, 8, 1, False, 0)
-    with pytest.raises(RuntimeError):
         sc_cuda.conv2d_or_acc(x.cuda(), w.cuda(), 64, (pad, pad), (1, 1), False)
 
 

@@ -250,3 +250,69 @@ def test_bad_arguments():
         so.conv2d_add_partial(x.numpy(), w.numpy()[:, :, :, :], 64, load_wait_w=0)
     with pytest.raises(ValueError):
         so.conv2d_add_partial(x.numpy()[:, :, :2], w.numpy(), 64)
+
+
+# ------------------------------------------------------------------ z / yz accumulation modes
+# No executable reference exists for these (GPU-only ops of the reference); they are pinned by
+# reductions to the y-mode path, which the compiled reference pins bit for bit.
+def test_modes_y_is_the_pinned_path():
+    x, w = wl.make_inputs((2, 5, 6, 7), (4, 5, 3, 2), "prescribed", seed=31)
+    for L in (8, 64, 256):
+        y = so.conv2d_add_partial(x.numpy(), w.numpy(), L, (1, 2), 7, 2, 2, 3)
+        assert np.array_equal(so.conv2d_modes(x.numpy(), w.numpy(), L, (1, 2), "y", 1, 7, 2, 2, 3), y)
+        # a single channel group is y-mode exactly (same groups, same seeds)
+        for zu in (5, 9):
+            assert np.array_equal(so.conv2d_modes(x.numpy(), w.numpy(), L, (1, 2), "yz", zu, 7, 2, 2, 3), y)
+
+
+@pytest.mark.parametrize("zu", [1, 2, 3, 4])
+@pytest.mark.parametrize("L", [16, 128])
+def test_yz_decomposes_into_y_mode_over_channel_blocks(zu, L):
+    """Seeds restart in every block of z_unit channels (weights: (c % zu)*W + u, activations:
+    index inside the block), blocks are added: yz(x, w) == sum over blocks of y(x[block], w[block])."""
+    x, w = wl.make_inputs((2, 7, 5, 6), (3, 7, 3, 3), "prescribed", seed=40 + zu)
+    x, w = x.numpy(), w.numpy()
+    got = so.conv2d_modes(x, w, L, (1, 1), "yz", zu, 7, 3, 2, 5)
+    exp = 0
+    for c0 in range(0, 7, zu):
+        exp = exp + so.conv2d_add_partial(x[:, c0:c0 + zu], w[:, c0:c0 + zu], L, (1, 1), 7, 3, 2, 5)
+    assert np.array_equal(got, exp)
+
+
+def test_z_reduces_to_y_mode_where_the_window_is_one_dimensional():
+    L = 32
+    # H = 1, Cin = 1: OR over u with seed u, nothing to add
+    x, w = wl.make_inputs((2, 1, 6, 5), (3, 1, 3, 1), "prescribed", seed=51)
+    assert np.array_equal(so.conv2d_modes(x.numpy(), w.numpy(), L, (0, 1), "z"),
+                          so.conv2d_add_partial(x.numpy(), w.numpy(), L, (0, 1)))
+    # W = 1 on a signal with a single row: OR over v with seed v; the transposed problem is y-mode
+    x, w = wl.make_inputs((2, 1, 1, 9), (3, 1, 1, 4), "prescribed", seed=52)
+    yz = so.conv2d_modes(x.numpy(), w.numpy(), L, (0, 0), "z")
+    yt = so.conv2d_add_partial(x.numpy().transpose(0, 1, 3, 2).copy(), w.numpy().transpose(0, 1, 3, 2).copy(), L)
+    assert np.array_equal(yz, yt.transpose(0, 1, 3, 2))
+    # channel planes of 7*k words with L = 8: activation seeds restart per channel, so z-mode is
+    # the sum over channels of single-channel z-mode
+    x, w = wl.make_inputs((2, 3, 7, 3), (2, 3, 3, 1), "prescribed", seed=53)
+    x, w = x.numpy(), w.numpy()
+    exp = 0
+    for c in range(3):
+        exp = exp + so.conv2d_add_partial(x[:, c:c + 1], w[:, c:c + 1], 8)
+    assert np.array_equal(so.conv2d_modes(x, w, 8, (0, 0), "z"), exp)
+
+
+@pytest.mark.parametrize("mode,zu", [("z", 1), ("yz", 2), ("yz", 3), ("y", 1)])
+def test_modes_against_independent_per_bit_formulation(mode, zu):
+    for (sx, sw, pad, L) in [((2, 3, 4, 5), (2, 3, 3, 2), (1, 0), 8), ((1, 5, 4, 4), (3, 5, 2, 3), (0, 1), 32)]:
+        x, w = wl.make_inputs(sx, sw, "prescribed", seed=61)
+        yb = bitref.conv_bits_modes(x.numpy(), w.numpy(), L, pad, mode, zu, 7, 2, 2, 3)
+        y = so.conv2d_modes(x.numpy(), w.numpy(), L, pad, mode, zu, 7, 2, 2, 3)
+        assert np.array_equal(y.astype(np.int64), yb), (mode, zu, sx)
+
+
+def test_modes_bounds():
+    x, w = wl.make_inputs((1, 6, 5, 5), (2, 6, 3, 3), "prescribed", seed=70)
+    L = 64
+    assert np.abs(so.conv2d_modes(x.numpy(), w.numpy(), L, (1, 1), "z")).max() <= 6 * L
+    assert np.abs(so.conv2d_modes(x.numpy(), w.numpy(), L, (1, 1), "yz", 4)).max() <= 2 * 3 * L
+    with pytest.raises(ValueError):
+        so.conv2d_modes(x.numpy(), w.numpy(), L, (1, 1), "yz", 0)
