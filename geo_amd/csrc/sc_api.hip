@@ -222,7 +222,6 @@ int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float
     const int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
     if (!x || !w || !grad_y || (!grad_x && !grad_w)) return GEO_SC_ERR_INVALID_ARGUMENT;
-    if (g.mode != GEO_SC_ACC_Y) return GEO_SC_ERR_UNSUPPORTED;
     if (!workspace || workspace_bytes < backward_workspace_bytes(g) || ((uintptr_t)workspace & 255u))
         return GEO_SC_ERR_WORKSPACE;
     return launch_conv_backward(g, x, w, grad_y, grad_x, grad_w, workspace, (hipStream_t)stream);

@@ -18,6 +18,14 @@
 // All three run on one MFMA kernel (v_mfma_f32_32x32x2_f32, fp32 in, fp32 accumulate) that
 // takes each operand either K-major or I-major; exp and the product with g are fused into
 // the first GEMM's epilogue; the second is split over m and reduced deterministically.
+//
+// The other accumulation modes have the same surrogate with other add groups
+// (utils_functional.py:254-299): one exponential per add group, whose argument sums the OR
+// members of the group.  "Kernel row" above generalises to a group g with members k:
+//     Y : g = v,                      k = ci*w_k + u                       (conv2d_or_bin_1d)
+//     Z : g = ci,                     k = u*h_k + v                        (conv2d_or_bin_z)
+//     YZ: g = (ci / z_unit)*h_k + v,  k = (ci % z_unit)*w_k + u            (conv2d_or_bin_yz)
+// Members of a ragged last channel block that do not exist carry zero weights.
 #include "sc_common.h"
 
 namespace geo_sc {
@@ -227,72 +235,138 @@ __global__ __launch_bounds__(256) void k_position_table(int* __restrict__ base, 
     }
 }
 
-// col[v][k][m] = x~[n, ci, a+u, b+v] for kernel rows v0 + blockIdx.z; k = ci*W + u, m = (n, a, b);
-// x~ is the zero-padded activation, read straight from the unpadded tensor.  blockIdx.y selects
-// a group of kIm2colChannels input channels; a thread reads its position's table entry once
-// and moves all kernel taps of those channels.  Reads and writes run along m.
-constexpr int kIm2colChannels = 4;
+// Group structure of one accumulation mode: which weight element (ci, u, v) member k of add
+// group g is, and the inverse.
+struct Groups {
+    int mode, c_in, w_k, h_k, zu;
+    int n_groups, n_members;
+};
+
+struct Member {
+    int ci, u, v;
+    bool ok;
+};
+
+__host__ __device__ inline Member member_of(const Groups& G, int g, int k)
+{
+    Member e;
+    if (G.mode == GEO_SC_ACC_Z) {
+        e.ci = g;
+        e.u = k / G.h_k;
+        e.v = k - e.u * G.h_k;
+        e.ok = true;
+    } else if (G.mode == GEO_SC_ACC_YZ) {
+        const int blk = g / G.h_k;
+        const int cl = k / G.w_k;
+        e.v = g - blk * G.h_k;
+        e.u = k - cl * G.w_k;
+        e.ci = blk * G.zu + cl;
+        e.ok = e.ci < G.c_in;
+    } else {
+        e.ci = k / G.w_k;
+        e.u = k - e.ci * G.w_k;
+        e.v = g;
+        e.ok = true;
+    }
+    return e;
+}
+
+// member k+1 of the same group from member k
+__host__ __device__ inline void next_member(const Groups& G, Member& e)
+{
+    if (G.mode == GEO_SC_ACC_Z) {
+        if (++e.v == G.h_k) {
+            e.v = 0;
+            ++e.u;
+        }
+    } else if (++e.u == G.w_k) {
+        e.u = 0;
+        ++e.ci;
+        e.ok = e.ci < G.c_in;
+    }
+}
+
+__host__ __device__ inline void group_of(const Groups& G, int ci, int u, int v, int& g, int& k)
+{
+    if (G.mode == GEO_SC_ACC_Z) {
+        g = ci;
+        k = u * G.h_k + v;
+    } else if (G.mode == GEO_SC_ACC_YZ) {
+        const int blk = ci / G.zu;
+        g = blk * G.h_k + v;
+        k = (ci - blk * G.zu) * G.w_k + u;
+    } else {
+        g = v;
+        k = ci * G.w_k + u;
+    }
+}
+
+// col[g][k][m] = x~[n, ci, a+u, b+v] for groups g0 + blockIdx.z, (ci, u, v) = member k of the
+// group, m = (n, a, b); x~ is the zero-padded activation, read straight from the unpadded
+// tensor.  blockIdx.y selects kIm2colMembers consecutive members; a thread reads its position's
+// table entry once and moves those members.  Reads and writes run along m.
+constexpr int kIm2colMembers = 12;
 __global__ __launch_bounds__(256) void k_im2col_rows(const float* __restrict__ x, float* __restrict__ col,
                                                      const int* __restrict__ base, const int* __restrict__ arow,
-                                                     const int* __restrict__ bcol, int v0, int m_total, int c_in,
-                                                     int w_in, int h_in, int w_k, size_t v_stride)
+                                                     const int* __restrict__ bcol, int g0, int m_total, Groups G,
+                                                     int w_in, int h_in, size_t g_stride)
 {
-    const int v = v0 + blockIdx.z;
-    const int ci0 = blockIdx.y * kIm2colChannels;
-    const int ci1 = min(c_in, ci0 + kIm2colChannels);
-    float* colv = col + (size_t)blockIdx.z * v_stride;
+    const int g = g0 + blockIdx.z;
+    const int k0 = blockIdx.y * kIm2colMembers;
+    const int k1 = min(G.n_members, k0 + kIm2colMembers);
+    float* colg = col + (size_t)blockIdx.z * g_stride;
     for (int m = blockIdx.x * 256 + threadIdx.x; m < m_total; m += gridDim.x * 256) {
-        const int r0 = arow[m], c = bcol[m] + v;
-        const bool c_ok = c >= 0 && c < h_in;
-        const float* src = x + base[m] + v;
-        for (int ci = ci0; ci < ci1; ci++) {
-            float* dst = colv + (size_t)ci * w_k * m_total + m;
-            for (int u = 0; u < w_k; u++) {
-                const int r = r0 + u;
-                float val = 0.0f;
-                if (c_ok && r >= 0 && r < w_in) val = src[(ci * w_in + u) * h_in];
-                dst[(size_t)u * m_total] = val;
-            }
+        const int r0 = arow[m], c0 = bcol[m];
+        const float* src = x + base[m];
+        Member e = member_of(G, g, k0);
+        for (int k = k0; k < k1; k++, next_member(G, e)) {
+            const int r = r0 + e.u, c = c0 + e.v;
+            float val = 0.0f;
+            if (e.ok && c >= 0 && c < h_in && r >= 0 && r < w_in) val = src[(e.ci * w_in + e.u) * h_in + e.v];
+            colg[(size_t)k * m_total + m] = val;
         }
     }
 }
 
-// Weight operands of kernel rows v0 + blockIdx.y:
-//   wcat[v][k][j]: j < c_out -> clamp(w,0,100), j >= c_out -> -clamp(w,-100,0)   (utils_functional.py:611-612)
-//   wd[v][j][k]  : the same with the negative rail negated (it enters dL/dx with a minus sign)
+// Weight operands of groups g0 + blockIdx.y:
+//   wcat[g][k][j]: j < c_out -> clamp(w,0,100), j >= c_out -> -clamp(w,-100,0)   (utils_functional.py:611-612)
+//   wd[g][j][k]  : the same with the negative rail negated (it enters dL/dx with a minus sign)
+// Members that do not exist (ragged last channel block) get zeros.
 __global__ __launch_bounds__(256) void k_weight_operands(const float* __restrict__ w, float* __restrict__ wcat,
-                                                         float* __restrict__ wd, int v0, int c_out, int c_in, int w_k,
-                                                         int h_k, size_t v_stride)
+                                                         float* __restrict__ wd, int g0, int c_out, Groups G,
+                                                         size_t g_stride)
 {
-    const int k_or = c_in * w_k;
-    const int total = k_or * c_out;
-    const int v = v0 + blockIdx.y;
-    float* wcatv = wcat + (size_t)blockIdx.y * v_stride;
-    float* wdv = wd + (size_t)blockIdx.y * v_stride;
+    const int K = G.n_members;
+    const int total = K * c_out;
+    const int g = g0 + blockIdx.y;
+    float* wcatg = wcat + (size_t)blockIdx.y * g_stride;
+    float* wdg = wd + (size_t)blockIdx.y * g_stride;
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
         const int co = e % c_out, k = e / c_out;
-        const float wv = w[((long long)co * k_or + k) * h_k + v];
+        const Member mb = member_of(G, g, k);
+        const float wv = mb.ok ? w[(((long long)co * G.c_in + mb.ci) * G.w_k + mb.u) * G.h_k + mb.v] : 0.0f;
         const float wp = fminf(fmaxf(wv, 0.0f), 100.0f);
         const float wn = -fminf(fmaxf(wv, -100.0f), 0.0f);
-        wcatv[(long long)k * 2 * c_out + co] = wp;
-        wcatv[(long long)k * 2 * c_out + c_out + co] = wn;
-        wdv[(long long)co * k_or + k] = wp;
-        wdv[(long long)(c_out + co) * k_or + k] = -wn;
+        wcatg[(long long)k * 2 * c_out + co] = wp;
+        wcatg[(long long)k * 2 * c_out + c_out + co] = wn;
+        wdg[(long long)co * K + k] = wp;
+        wdg[(long long)(c_out + co) * K + k] = -wn;
     }
 }
 
-// dL/dw[co][ci][u][v] from the split partial sums part[v][s][k][j], v = v0 + blockIdx.y.  A
-// block takes 32 consecutive (k, co) entries; 8 groups of threads each sum every 8th split,
-// the groups are then added in a fixed order, so the result does not depend on scheduling.
+// dL/dw of the members of group g0 + blockIdx.y from the split partial sums part[g][s][k][j].  A
+// block takes 32 consecutive (k, co) entries; 8 sets of threads each sum every 8th split, the
+// sets are then added in a fixed order, so the result does not depend on scheduling.
 __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ part, const float* __restrict__ w,
-                                                      float* __restrict__ gw, int v0, int splits, int c_out, int k_or,
-                                                      int h_k, size_t v_stride)
+                                                      float* __restrict__ gw, int g0, int splits, int c_out, Groups G,
+                                                      size_t g_stride)
 {
     __shared__ float red[2][8][32];
-    const int total = k_or * c_out;
-    const long long stride = (long long)k_or * 2 * c_out;
-    const int v = v0 + blockIdx.y;
-    const float* partv = part + (size_t)blockIdx.y * v_stride;
+    const int K = G.n_members;
+    const int total = K * c_out;
+    const long long stride = (long long)K * 2 * c_out;
+    const int g = g0 + blockIdx.y;
+    const float* partg = part + (size_t)blockIdx.y * g_stride;
     const int lane = threadIdx.x & 31, grp = threadIdx.x >> 5;
     const int e = blockIdx.x * 32 + lane;
     const bool ok = e < total;
@@ -300,20 +374,21 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ 
     float sp = 0.0f, sn = 0.0f;
     if (ok)
         for (int s = grp; s < splits; s += 8) {
-            sp += partv[s * stride + (long long)k * 2 * c_out + co];
-            sn += partv[s * stride + (long long)k * 2 * c_out + c_out + co];
+            sp += partg[s * stride + (long long)k * 2 * c_out + co];
+            sn += partg[s * stride + (long long)k * 2 * c_out + c_out + co];
         }
     red[0][grp][lane] = sp;
     red[1][grp][lane] = sn;
     __syncthreads();
-    if (grp == 0 && ok) {
+    const Member mb = member_of(G, g, k);
+    if (grp == 0 && ok && mb.ok) {
         sp = sn = 0.0f;
 #pragma unroll
         for (int gidx = 0; gidx < 8; gidx++) {
             sp += red[0][gidx][lane];
             sn += red[1][gidx][lane];
         }
-        const long long wi = ((long long)co * k_or + k) * h_k + v;
+        const long long wi = (((long long)co * G.c_in + mb.ci) * G.w_k + mb.u) * G.h_k + mb.v;
         const float wv = w[wi];
         float r = 0.0f;
         if (wv >= 0.0f && wv <= 100.0f) r += sp;
@@ -322,31 +397,35 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad(const float* __restrict__ 
     }
 }
 
-// dL/dx[n][ci][p][q] (+)= sum_{v in chunk} sum_u dcol[v][ci*W+u][(n, p+pad_w-u, q+pad_h-v)] over
-// the valid output positions; the first chunk of kernel rows writes, later chunks add.  Blocks
-// stride over the planes (n, ci).
-__global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ dcol, float* __restrict__ gx, int v0,
-                                                     int nv, long long m_total, int n_planes, int c_in, int w_in,
-                                                     int h_in, int pad_w, int pad_h, int w_k, int wo, int ho,
-                                                     size_t v_stride)
+// dL/dx[n][ci][p][q] (+)= sum over the kernel taps (u, v) whose group lies in [g0, g0 + ng) of
+// dcol[g][k][(n, p+pad_w-u, q+pad_h-v)] over the valid output positions; the first chunk of
+// groups writes, later chunks add.  Blocks stride over the planes (n, ci).
+__global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ dcol, float* __restrict__ gx, int g0,
+                                                     int ng, long long m_total, int n_planes, Groups G, int w_in,
+                                                     int h_in, int pad_w, int pad_h, int wo, int ho, size_t g_stride)
 {
     const int plane = w_in * h_in;
+    const int k_step = G.mode == GEO_SC_ACC_Z ? G.h_k : 1;
     for (int nc = blockIdx.x; nc < n_planes; nc += gridDim.x) {
-        const int n = nc / c_in, ci = nc - n * c_in;
+        const int n = nc / G.c_in, ci = nc - n * G.c_in;
         float* dst = gx + (size_t)nc * plane;
-        const float* src = dcol + (size_t)ci * w_k * m_total + (size_t)n * wo * ho;
+        const float* src = dcol + (size_t)n * wo * ho;
         for (int e = blockIdx.y * 256 + threadIdx.x; e < plane; e += gridDim.y * 256) {
             const int p = e / h_in, qq = e - p * h_in;
             float s = 0.0f;
-            for (int dv = 0; dv < nv; dv++) {
-                const int b = qq + pad_h - (v0 + dv);
-                if (b < 0 || b >= ho) continue;
-                for (int u = 0; u < w_k; u++) {
+            for (int v = 0; v < G.h_k; v++) {
+                const int b = qq + pad_h - v;
+                // the group does not depend on u, and the member index advances by k_step per tap
+                int g, k;
+                group_of(G, ci, 0, v, g, k);
+                if (g < g0 || g >= g0 + ng || b < 0 || b >= ho) continue;
+                const float* sg = src + (size_t)(g - g0) * g_stride + (size_t)k * m_total + b;
+                for (int u = 0; u < G.w_k; u++) {
                     const int a = p + pad_w - u;
-                    if (a >= 0 && a < wo) s += src[dv * v_stride + (size_t)u * m_total + a * ho + b];
+                    if (a >= 0 && a < wo) s += sg[(size_t)u * k_step * m_total + a * ho];
                 }
             }
-            dst[e] = v0 == 0 ? s : dst[e] + s;
+            dst[e] = g0 == 0 ? s : dst[e] + s;
         }
     }
 }
@@ -377,8 +456,9 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 struct BwdLayout {
     long long m_total;
     int splits, m_per_split;
-    int rows_per_chunk;  // kernel rows processed by one round of launches
-    size_t col_v, e_v, part_v, w_v;  // floats per kernel row of each scratch array
+    Groups G;
+    int rows_per_chunk;  // add groups processed by one round of launches
+    size_t col_v, e_v, part_v, w_v;  // floats per add group of each scratch array
     size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, bytes;
 };
 
@@ -386,8 +466,24 @@ BwdLayout bwd_layout(const Geometry& g)
 {
     BwdLayout b;
     b.m_total = (long long)g.n * g.wo * g.ho;
+    b.G.mode = g.mode;
+    b.G.c_in = g.c_in;
+    b.G.w_k = g.w_k;
+    b.G.h_k = g.h_k;
+    b.G.zu = g.z_unit;
+    if (g.mode == GEO_SC_ACC_Z) {
+        b.G.n_groups = g.c_in;
+        b.G.n_members = g.w_k * g.h_k;
+    } else if (g.mode == GEO_SC_ACC_YZ) {
+        b.G.n_groups = g.add_outer * g.h_k;
+        b.G.n_members = g.z_unit * g.w_k;
+    } else {
+        b.G.n_groups = g.h_k;
+        b.G.n_members = g.k_or;
+    }
+    const int K = b.G.n_members;
     // split the m-reduction of the weight gradient so that the grid covers the GPU
-    const long long tiles = (long long)((g.k_or + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
+    const long long tiles = (long long)((K + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
     long long want = (1024 + tiles - 1) / tiles;
     long long per = (b.m_total + want - 1) / want;
     per = (per + kChunk - 1) / kChunk * kChunk;
@@ -396,15 +492,15 @@ BwdLayout bwd_layout(const Geometry& g)
     b.splits = (int)((b.m_total + b.m_per_split - 1) / b.m_per_split);
     // per-row scratch, each row's part padded to 64 floats so that float4 staging stays aligned
     auto pad64 = [](size_t v) { return (v + 63) & ~(size_t)63; };
-    b.col_v = pad64((size_t)b.m_total * g.k_or);
+    b.col_v = pad64((size_t)b.m_total * K);
     b.e_v = pad64((size_t)b.m_total * 2 * g.c_out);
-    b.part_v = pad64((size_t)b.splits * g.k_or * 2 * g.c_out);
-    b.w_v = pad64((size_t)g.k_or * 2 * g.c_out);
-    // all kernel rows in one round of launches unless that needs more than ~3 GB of scratch
+    b.part_v = pad64((size_t)b.splits * K * 2 * g.c_out);
+    b.w_v = pad64((size_t)K * 2 * g.c_out);
+    // all groups in one round of launches unless that needs more than ~3 GB of scratch
     const size_t per_row = sizeof(float) * (2 * b.col_v + b.e_v + b.part_v + 2 * b.w_v);
     size_t rows = ((size_t)3 << 30) / per_row;
     if (rows < 1) rows = 1;
-    if (rows > (size_t)g.h_k) rows = g.h_k;
+    if (rows > (size_t)b.G.n_groups) rows = b.G.n_groups;
     if (rows * b.splits > 65535) rows = 65535 / b.splits;  // grid.z = rows * splits
     if (rows < 1) rows = 1;
     b.rows_per_chunk = (int)rows;
@@ -436,9 +532,10 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     float* part = (float*)(ws + L.off_part);
     float* wcat = (float*)(ws + L.off_wcat);
     float* wd = (float*)(ws + L.off_wd);
-    const int M = (int)L.m_total, K = g.k_or, J = 2 * g.c_out;
+    const Groups& G = L.G;
+    const int M = (int)L.m_total, K = G.n_members, J = 2 * g.c_out;
     const long long x_total = (long long)g.n * g.c_in * g.w_in * g.h_in;
-    if (x_total > 0x7fffffffLL || g.c_in > 65535 * kIm2colChannels) return GEO_SC_ERR_UNSUPPORTED;
+    if (x_total > 0x7fffffffLL || K > 65535 * kIm2colMembers) return GEO_SC_ERR_UNSUPPORTED;
     if ((long long)g.n * g.c_out * g.wo * g.ho > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
     const size_t pos_stride = align256(sizeof(int) * (size_t)M) / sizeof(int);
     int* pos_base = (int*)(ws + L.off_pos);
@@ -449,16 +546,15 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, pos_goff, M,
                        g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
     int rc;
-    for (int v0 = 0; v0 < g.h_k; v0 += L.rows_per_chunk) {
-        const int nv = g.h_k - v0 < L.rows_per_chunk ? g.h_k - v0 : L.rows_per_chunk;
+    for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
+        const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
         hipLaunchKernelGGL(k_im2col_rows,
-                           dim3(m_blocks > 1024 ? 1024 : m_blocks, (g.c_in + kIm2colChannels - 1) / kIm2colChannels, nv),
-                           dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, g.c_in, g.w_in, g.h_in,
-                           g.w_k, L.col_v);
+                           dim3(m_blocks > 1024 ? 1024 : m_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
+                           dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, G, g.w_in, g.h_in, L.col_v);
         {
             int wb = grid1d((long long)K * g.c_out);
             hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
-                               g.c_out, g.c_in, g.w_k, g.h_k, L.w_v);
+                               g.c_out, G, L.w_v);
         }
         // E[v][m][j] = g * exp(-(col_v^T . wcat_v)), col stored [K][M]
         GemmParams q1 = {};
@@ -481,7 +577,7 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             q2.c_batch_stride = (long long)L.part_v;
             if ((rc = launch_gemm<false, true, EPI_STORE>(q2, nv, s)) != GEO_SC_OK) return rc;
             hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
-                               L.splits, g.c_out, K, g.h_k, L.part_v);
+                               L.splits, g.c_out, G, L.part_v);
         }
         if (!gx) continue;
         // dcol[v][k][m] = sum_j wd_v[j][k] * E_v[m][j]
@@ -498,7 +594,7 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         const int pb = plane_blocks > 64 ? 64 : plane_blocks;
         const int want = 256 * 16 / pb;  // a few thousand blocks in all
         hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx, v0,
-                           nv, L.m_total, n_planes, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, g.w_k, g.wo, g.ho, L.col_v);
+                           nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
     }
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }

@@ -1,11 +1,14 @@
-"""Functional SC layer with the reference's interface (utils_functional.py), for the one
-configuration this build accelerates: ``forward='1d_bin'`` (OR over input channels and
-kernel dim 2, binary add over kernel dim 3), ``generator='lfsr'``, ``legacy=False``.
+"""Functional SC layer with the reference's interface (utils_functional.py), for the
+configurations this build accelerates, all with the LFSR generators and ``legacy=False``:
+``forward='1d_bin'`` (OR over input channels and kernel dim 2, binary add over kernel dim 3),
+``forward='z_bin'`` (OR over the kernel window, add over input channels) and
+``forward='yz_bin'`` (OR over ``z_unit`` input channels and kernel dim 2, add over kernel dim 3
+and channel blocks).
 
 Forward values come from the HIP SC kernels (integer counts / stream length); gradients
-are those of the reference's floating-point surrogate ``conv2d_or_bin_1d``
-(utils_functional.py:235-252), computed by the HIP backward kernels instead of autograd
-over 2*H dense convolutions.  The surrogate's own forward is never evaluated: the
+are those of the reference's floating-point surrogates ``conv2d_or_bin_1d`` / ``_z`` / ``_yz``
+(utils_functional.py:235-299), computed by the HIP backward kernels instead of autograd
+over two dense convolutions per add group.  The surrogate's own forward is never evaluated: the
 reference overwrites its value with the SC result anyway (utils_functional.py:631-634).
 """
 from __future__ import annotations
@@ -51,11 +54,39 @@ def conv2d_or_bin_1d(activation, w_pos, w_neg, padding, stride):
     return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
 
 
+def conv2d_or_bin_z(activation, w_pos, w_neg, padding, stride):
+    """Surrogate of z-dimension accumulation (utils_functional.py:254-270): one single-channel
+    convolution per input channel and rail, 1 - exp(-z), summed over channels."""
+    pos, neg = [], []
+    for c in range(activation.size(1)):
+        a_sec = activation[:, c:c + 1]
+        pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[:, c:c + 1], stride=stride)))
+        neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[:, c:c + 1], stride=stride)))
+    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
+
+
+def conv2d_or_bin_yz(activation, w_pos, w_neg, padding, stride, z_unit):
+    """Surrogate of yz accumulation (utils_functional.py:272-299): one W x 1 convolution per
+    block of ``z_unit`` input channels, kernel row and rail, 1 - exp(-z), summed."""
+    c_in = activation.size(1)
+    i_y = activation.size(3)
+    f_y = w_pos.size(3)
+    pos, neg = [], []
+    for c in range(0, c_in, z_unit):
+        c_end = min(c + z_unit, c_in)
+        for j in range(f_y):
+            a_sec = activation[:, c:c_end, :, j:i_y - f_y + j + 1]
+            pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[:, c:c_end, :, j:j + 1], stride=stride)))
+            neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[:, c:c_end, :, j:j + 1], stride=stride)))
+    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
+
+
 class _SCConv2dAddPartial(torch.autograd.Function):
     """value: SC count / L  (HIP forward);  gradient: surrogate (HIP backward)."""
 
     @staticmethod
-    def forward(ctx, activation, weight, bit_length, padding, load_unit, load_wait):
+    def forward(ctx, activation, weight, bit_length, padding, load_unit, load_wait, accumulate="y", z_unit=1,
+                load_wait_a=None):
         origin = activation.device
         dev = origin if activation.is_cuda else torch.device("cuda", torch.cuda.current_device())
         x = activation.detach().to(dev, torch.float32).contiguous()
@@ -64,14 +95,19 @@ class _SCConv2dAddPartial(torch.autograd.Function):
         if activation.is_cuda:
             # sc_extension_cuda.conv2d_add_partial_variable_acc(..., prec_default, load_unit,
             # load_wait_w, False, 2): one wait for both generators (utils_functional.py:497)
+            # (:504), and conv2d_add_yz_variable_acc(..., load_wait_w, load_wait_a, False, z_unit) (:508)
             loading = dict(total_width=prec_default, load_width=int(load_unit), load_wait_w=int(load_wait),
-                           load_wait_a=int(load_wait))
+                           load_wait_a=int(load_wait if load_wait_a is None else load_wait_a))
         else:
             # host tensors take the reference's CPU entry point, which has no progressive
             # loading (utils_functional.py:493)
             loading = dict(capi.NEUTRAL_LOADING)
-        counts = capi.conv2d_add_partial_forward(x, w, int(bit_length), pad, **loading)
+        z_unit = max(1, min(int(z_unit), x.shape[1]))
+        counts = capi.conv2d_add_partial_forward(x, w, int(bit_length), pad, accumulate=accumulate, z_unit=z_unit,
+                                                 **loading)
         ctx.save_for_backward(x, w)
+        ctx.accumulate = accumulate
+        ctx.z_unit = z_unit
         ctx.pad = pad
         ctx.origin = origin
         ctx.bit_length = int(bit_length)
@@ -87,21 +123,24 @@ class _SCConv2dAddPartial(torch.autograd.Function):
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         gx = gw = None
         if need_x or need_w:
-            gx, gw = capi.conv2d_add_partial_backward(x, w, g, ctx.bit_length, ctx.pad, need_x, need_w)
+            gx, gw = capi.conv2d_add_partial_backward(x, w, g, ctx.bit_length, ctx.pad, need_x, need_w,
+                                                      accumulate=ctx.accumulate, z_unit=ctx.z_unit)
         if gx is not None:
             gx = gx.to(ctx.origin, ctx.act_dtype)
         if gw is not None:
             gw = gw.to(ctx.w_device, ctx.w_dtype)
-        return gx, gw, None, None, None, None
+        return gx, gw, None, None, None, None, None, None, None
 
 
 def conv2d_generic(activation, weight, padding, stride, **kwargs):
     """Generic SC conv2d layer, same call as the reference's (utils_functional.py:406-634).
 
     Keyword arguments read: bit_length (128), generator (None), forward ('full_or'), legacy
-    (False), load_unit (8), load_wait_w (1), load_wait_a (1); prec/acc/share/z_unit are
-    accepted and unused on this path.  Only forward='1d_bin', generator='lfsr',
-    legacy=False is implemented; anything else raises NotImplementedError.
+    (False), load_unit (8), load_wait_w (1), load_wait_a (1), z_unit (1024); prec/acc/share are
+    accepted and unused on these paths.  Implemented: forward='1d_bin' with generator='lfsr', and
+    forward='z_bin' / 'yz_bin' on GPU tensors (the reference sends those to its LFSR GPU ops
+    whatever the generator, utils_functional.py:503-510), all with legacy=False; anything else
+    raises NotImplementedError.
     """
     bit_length = kwargs.get("bit_length", 128)
     generator = kwargs.get("generator", None)
@@ -109,16 +148,26 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     legacy = kwargs.get("legacy", False)
     load_unit = kwargs.get("load_unit", 8)
     load_wait_w = kwargs.get("load_wait_w", 1)
-    if forward != "1d_bin" or generator != "lfsr" or legacy:
+    load_wait_a = kwargs.get("load_wait_a", 1)
+    z_unit = kwargs.get("z_unit", 1024)
+    ok_1d = forward == "1d_bin" and generator == "lfsr"
+    ok_zyz = forward in ("z_bin", "yz_bin") and activation.is_cuda
+    if legacy or not (ok_1d or ok_zyz):
         raise NotImplementedError(
-            f"conv2d_generic(forward={forward!r}, generator={generator!r}, legacy={legacy}): this build implements "
-            "forward='1d_bin', generator='lfsr', legacy=False only")
+            f"conv2d_generic(forward={forward!r}, generator={generator!r}, legacy={legacy}, "
+            f"cuda={activation.is_cuda}): this build implements forward='1d_bin' with generator='lfsr' and "
+            "forward='z_bin'/'yz_bin' on GPU tensors, legacy=False")
     if isinstance(stride, int):
         stride = (stride, stride)
     if tuple(stride) != (1, 1):
         raise NotImplementedError("the SC kernels compute stride 1 only (the reference's native code ignores stride)")
     if isinstance(padding, int):
         padding = (padding, padding)
+    if forward == "z_bin":
+        return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), load_unit, load_wait_w, "z")
+    if forward == "yz_bin":
+        return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), load_unit, load_wait_w,
+                                         "yz", z_unit, load_wait_a)
     return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), load_unit, load_wait_w)
 
 

@@ -99,3 +99,71 @@ def test_torch_module_ops(so):
                               so.conv2d_modes(x.numpy(), w.numpy(), 64, (1, 1), "yz", zu, 7, 2, 3, 5)), zu
     with pytest.raises(RuntimeError):
         ext.conv2d_add_yz_variable_acc(xd, wd, 64, (1, 1), (1, 1), 7, 2, 3, 5, True, 0)
+
+
+# ------------------------------------------------------------------ surrogate backward
+RTOL = 1e-5  # fp32 gradients: max|got - ref| <= 1e-5 * max|ref| against the float64 oracle
+
+
+def rel_err(got, ref):
+    ref = ref.double().cpu()
+    return ((got.double().cpu() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+
+
+BWD_CASES = [
+    # shape_x, shape_w, pad, input kind, weight scale
+    ((2, 7, 5, 6), (4, 7, 3, 2), (1, 1), "q7", 3.0),
+    ((3, 8, 9, 9), (10, 8, 3, 3), (1, 1), "q7", 4.0),
+    ((1, 4, 7, 8), (3, 4, 2, 3), (2, 0), "prescribed", 0.5),
+    ((6, 16, 1, 8), (40, 16, 1, 8), (0, 0), "prescribed", 0.3),
+    ((3, 70, 6, 6), (140, 70, 3, 3), (1, 1), "kaiming", 3.0),
+]
+
+
+@pytest.mark.parametrize("case", range(len(BWD_CASES)))
+@pytest.mark.parametrize("mode,zu", [("z", 1), ("yz", 1), ("yz", 3), ("yz", 4), ("yz", 64)])
+def test_backward_modes_match_float64_oracle(capi, case, mode, zu):
+    from oracle import surrogate
+    shape_x, shape_w, pad, kind, scale = BWD_CASES[case]
+    print(f"backward {mode} z_unit {zu} case {shape_x} {shape_w} pad {pad}", flush=True)
+    x, w = wl.make_inputs(shape_x, shape_w, kind, seed=shape_x[1])
+    w = (w * scale).contiguous()
+    w.view(-1)[::7] = 0.0
+    d = capi.make_desc(x.shape, w.shape, 128, pad)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(1))
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, accumulate=mode, z_unit=zu)
+    torch.cuda.synchronize()
+    rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=min(zu, shape_x[1]))
+    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
+    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    gx2, none = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_w=False,
+                                                 accumulate=mode, z_unit=zu)
+    none2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_x=False,
+                                                  accumulate=mode, z_unit=zu)
+    assert none is None and none2 is None
+    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)
+
+
+@pytest.mark.parametrize("forward,kw", [("z_bin", {}), ("yz_bin", {"z_unit": 4, "load_wait_a": 3}),
+                                        ("yz_bin", {})])
+def test_conv2d_generic_modes(so, forward, kw):
+    """The functional layer: SC value from the kernels, gradient of the matching surrogate."""
+    from geo_amd import utils_functional as uf
+    from oracle import surrogate
+    x, w = wl.make_inputs((3, 6, 6, 6), (8, 6, 3, 3), "prescribed", seed=5)
+    w = (w * 2).contiguous()
+    xd = x.cuda().requires_grad_(True)
+    wd = w.cuda().requires_grad_(True)
+    y = uf.conv2d_generic(xd, wd, (1, 1), (1, 1), bit_length=64, forward=forward, generator="lfsr", load_unit=2,
+                          load_wait_w=2, **kw)
+    mode = "z" if forward == "z_bin" else "yz"
+    zu = min(kw.get("z_unit", 1024), 6)
+    wa = kw.get("load_wait_a", 1) if mode == "yz" else 2
+    exp = so.conv2d_modes(x.numpy(), w.numpy(), 64, (1, 1), mode, zu, 7, 2, 2, wa)
+    assert np.array_equal((y.detach().cpu() * 64).round().int().numpy(), exp)
+    g = torch.randn(y.shape, generator=torch.Generator().manual_seed(3))
+    y.backward(g.cuda())
+    rx, rw, _ = surrogate.surrogate_autograd(x, w, g, (1, 1), mode=mode, z_unit=zu)
+    assert rel_err(xd.grad, rx) <= RTOL and rel_err(wd.grad, rw) <= RTOL
+    with pytest.raises(NotImplementedError):
+        uf.conv2d_generic(x, w, (1, 1), (1, 1), bit_length=64, forward=forward, generator="lfsr")
