@@ -24,6 +24,20 @@
  *                        reference executes it; checked for neutrality at
  *                        load_width >= total_width+1 and for the width
  *                        sequence 1,3,3,5,5,7,7.. of (7,2,2).
+ *   sco_conv2d_modes, mode yz
+ *                        pinned  - equals the sum over channel blocks of the
+ *                                  pinned y-mode path on the blocks, for every
+ *                                  z_unit (seeds restart per block); one block
+ *                                  is y-mode itself (tests/test_oracle.py)
+ *   sco_conv2d_modes, mode z
+ *                        pinned where the OR window is one-dimensional (H = 1;
+ *                        W = 1 on single-row signals; per-channel
+ *                        decomposition when seeds restart per channel).  For
+ *                        general W x H windows (joint OR over (u,v), seed
+ *                        index u*H+v) PARITY UNPINNED: the reference has no
+ *                        executable z-mode code outside its CUDA kernels
+ *                        (sc_cuda_kernel.cu:270-349); an independent per-bit
+ *                        formulation of the same reading agrees.
  *
  * Conventions (same names as the reference): weight (Cout, Cin, W, H) with
  * W = dim 2 and H = dim 3 (the binary-add dimension); padded activation
