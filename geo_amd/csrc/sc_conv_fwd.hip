@@ -357,12 +357,14 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     // per-lane word offsets are 32-bit
     if ((unsigned long long)R * g.packs * g.act_plane >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
     if (ROWS_IN_N != g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
-    // Few waves (small layers): split the (pack, kernel row) sum over blockIdx.y until about four
-    // waves per SIMD exist; the partial sums meet in y through integer atomics.
+    // Fewer than four waves per SIMD (small layers, the SC-linear mapping): split the (pack, add
+    // group) sum over blockIdx.y until about twelve waves per SIMD exist, so that three resident
+    // waves per SIMD stay available through the tail; the partial sums meet in y through integer
+    // atomics.  Measured on MI355X: 4096x4096 linear at batch 1024 7.05 -> 6.24 ms.
     const int pv = g.packs * g.add_outer * g.add_inner;
     int splits = 1;
-    if (waves < 2048) {
-        splits = (int)((4096 + waves - 1) / waves);
+    if (waves < 4096) {
+        splits = (int)((12288 + waves - 1) / waves);
         if (splits > pv) splits = pv;
     }
     q.pv_per_block = (pv + splits - 1) / splits;
