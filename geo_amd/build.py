@@ -20,7 +20,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 INCLUDE = os.path.join(ROOT, "include")
 
-HIP_SOURCES = ["sc_streams.hip", "sc_conv_fwd.hip", "sc_conv_bwd.hip", "sc_probe.hip", "sc_api.hip"]
+HIP_SOURCES = ["sc_streams.hip", "sc_conv_fwd.hip", "sc_conv_bwd.hip", "sc_probe.hip", "sc_epilogue.hip", "sc_api.hip"]
 TORCH_MODULES = {"sc_extension_cuda": "sc_extension_cuda.cpp", "sc_extension": "sc_extension.cpp"}
 
 # gfx950 only; packed-FP32 instruction selection is switched off for every device pass

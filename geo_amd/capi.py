@@ -94,6 +94,52 @@ def conv2d_add_partial_forward(x, w, bit_length, padding=(0, 0), total_width=7, 
     return out
 
 
+def conv2d_add_partial_forward_q7(x_q7, w, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
+                                  load_wait_a=1, out=None, workspace=None, stream=None, accumulate="y", z_unit=1):
+    """The forward for activations given as uint8 integers k = round(x * 128), k <= 127
+    (geo_sc_conv2d_add_partial_forward_q7): same counts as the fp32 entry point on k / 128."""
+    if not (x_q7.is_cuda and x_q7.dtype == torch.uint8 and x_q7.is_contiguous()):
+        raise ValueError("x_q7 must be a contiguous uint8 GPU tensor")
+    _require_gpu_f32(w, "w")
+    desc = make_desc(x_q7.shape, w.shape, bit_length, padding, total_width, load_width, load_wait_w, load_wait_a,
+                     accumulate, z_unit)
+    if workspace is None:
+        workspace = torch.empty(workspace_size(desc), dtype=torch.uint8, device=w.device)
+    if out is None:
+        out = torch.empty(output_shape(desc), dtype=torch.int32, device=w.device)
+    _check(_native.lib().geo_sc_conv2d_add_partial_forward_q7(ctypes.byref(desc), _ptr(x_q7), _ptr(w), _ptr(out),
+                                                              _ptr(workspace), workspace.numel(),
+                                                              _stream_ptr(stream)),
+           "geo_sc_conv2d_add_partial_forward_q7")
+    return out
+
+
+# enum geo_sc_epilogue_flags
+EPI_RELU, EPI_POOL2, EPI_HARDTANH01, EPI_QUANT7 = 1, 2, 4, 8
+
+
+def layer_epilogue(counts, bit_length, w_n, b_n, relu=False, pool=True, hardtanh=True, quant7=True, want_act=True,
+                   want_q7=False, stream=None):
+    """geo_sc_layer_epilogue: int32 counts (N, C, W, H) -> (fp32 activation or None, uint8 7-bit
+    integers or None), each (N, C, W', H'): count / L, per-channel w_n, b_n, then the selected
+    relu / AvgPool2d(2) / Hardtanh(0, 1) / 7-bit quantisation."""
+    if not (counts.is_cuda and counts.dtype == torch.int32 and counts.is_contiguous() and counts.dim() == 4):
+        raise ValueError("counts must be a contiguous int32 GPU tensor (N, C, W, H)")
+    n, c, w, h = counts.shape
+    w_n = w_n.to(counts.device, torch.float32).contiguous()
+    b_n = b_n.to(counts.device, torch.float32).contiguous()
+    if w_n.numel() != c or b_n.numel() != c:
+        raise ValueError("w_n and b_n need one entry per channel")
+    flags = (EPI_RELU if relu else 0) | (EPI_POOL2 if pool else 0) | (EPI_HARDTANH01 if hardtanh else 0) | \
+        (EPI_QUANT7 if quant7 else 0)
+    shape = (n, c, w // 2, h // 2) if pool else (n, c, w, h)
+    act = torch.empty(shape, dtype=torch.float32, device=counts.device) if want_act else None
+    q7 = torch.empty(shape, dtype=torch.uint8, device=counts.device) if want_q7 else None
+    _check(_native.lib().geo_sc_layer_epilogue(_ptr(counts), n, c, w, h, int(bit_length), _ptr(w_n), _ptr(b_n), flags,
+                                               _ptr(act), _ptr(q7), _stream_ptr(stream)), "geo_sc_layer_epilogue")
+    return act, q7
+
+
 def _tables(bit_length, device):
     n = ctypes.c_size_t(0)
     _check(_native.lib().geo_sc_stream_tables_size(int(bit_length), ctypes.byref(n)), "tables size")

@@ -91,6 +91,31 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
 
 using namespace geo_sc;
 
+namespace {
+// x is fp32, or with Q7 the uint8 integers k of activations k / 128
+template <bool Q7>
+int forward_impl(const geo_sc_conv_desc* desc, const void* x, const float* w, int32_t* y, void* workspace,
+                 size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    Geometry g;
+    int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!x || !w || !y) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (!workspace || workspace_bytes < g.ws_bytes || ((uintptr_t)workspace & 255u)) return GEO_SC_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    uint32_t* tables = (uint32_t*)(ws + g.off_tables);
+    uint32_t* wgt = (uint32_t*)(ws + g.off_wgt);
+    uint32_t* act = (uint32_t*)(ws + g.off_act);
+    if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
+    if ((rc = launch_weight_streams(g, w, wgt, tables, s)) != GEO_SC_OK) return rc;
+    rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)x, act, tables, s)
+            : launch_act_streams(g, (const float*)x, act, tables, s);
+    if (rc != GEO_SC_OK) return rc;
+    return launch_conv_forward(g, act, wgt, y, s);
+}
+}  // namespace
+
 extern "C" {
 
 int geo_sc_version(void) { return GEO_SC_VERSION; }
@@ -188,20 +213,14 @@ int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const u
 int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
                                       void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
 {
-    Geometry g;
-    int rc = make_geometry(desc, &g);
-    if (rc != GEO_SC_OK) return rc;
-    if (!x || !w || !y) return GEO_SC_ERR_INVALID_ARGUMENT;
-    if (!workspace || workspace_bytes < g.ws_bytes || ((uintptr_t)workspace & 255u)) return GEO_SC_ERR_WORKSPACE;
-    hipStream_t s = (hipStream_t)stream;
-    char* ws = (char*)workspace;
-    uint32_t* tables = (uint32_t*)(ws + g.off_tables);
-    uint32_t* wgt = (uint32_t*)(ws + g.off_wgt);
-    uint32_t* act = (uint32_t*)(ws + g.off_act);
-    if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
-    if ((rc = launch_weight_streams(g, w, wgt, tables, s)) != GEO_SC_OK) return rc;
-    if ((rc = launch_act_streams(g, x, act, tables, s)) != GEO_SC_OK) return rc;
-    return launch_conv_forward(g, act, wgt, y, s);
+    return forward_impl<false>(desc, x, w, y, workspace, workspace_bytes, stream);
+}
+
+int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, const float* w,
+                                         int32_t* y, void* workspace, size_t workspace_bytes,
+                                         geo_sc_stream_t stream)
+{
+    return forward_impl<true>(desc, x_q7, w, y, workspace, workspace_bytes, stream);
 }
 
 int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes)

@@ -58,6 +58,8 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g);
 // launchers (each returns a geo_sc_status)
 int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s);
 int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s);
+int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* streams, const uint32_t* tables,
+                          hipStream_t s);
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);

@@ -111,8 +111,9 @@ __device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, const uint32_t
 // Activation streams from the unpadded fp32 input; padding positions produce zero words but
 // keep their place in the seed numbering (sc.cpp:409-413).  Layout [n][P][c_in][Wi][Hi], or
 // with ITEM_INNER [P][c_in][Wi][Hi][n]; threads run along the innermost axis of the output.
-template <bool ITEM_INNER>
-__global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __restrict__ x,
+// XT: float (the activation itself) or uint8_t (the 7-bit integer k, activation k / 128).
+template <bool ITEM_INNER, typename XT>
+__global__ __launch_bounds__(kGenThreads) void k_act_streams(const XT* __restrict__ x,
                                                             uint32_t* __restrict__ streams,
                                                             const uint32_t* __restrict__ tables, GenParams gp, int n,
                                                             int c_in, int w_in, int h_in, int pad_w, int pad_h,
@@ -142,7 +143,8 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const float* __rest
         const int ps = (int)p - pad_w, qs = (int)q - pad_h;
         int code = 0;
         if (ps >= 0 && ps < w_in && qs >= 0 && qs < h_in) {
-            const float v = x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs];
+            const float v = sizeof(XT) == 1 ? (float)x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs] * 0.0078125f
+                                            : (float)x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs];
             // ceil(clamp(x*L, 0, L-1))  (sc.cpp:301)
             code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
         }
@@ -287,18 +289,31 @@ int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s)
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
-int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s)
+template <typename XT>
+static int launch_act_streams_t(const Geometry& g, const XT* x, uint32_t* streams, const uint32_t* tables,
+                                hipStream_t s)
 {
     const GenParams gp = gen_params(g, g.load_wait_a);
     const size_t total = (size_t)g.n * g.act_plane;
     const uint32_t wrap = (uint32_t)g.seed_wrap;
     if (g.act_item_inner)
-        hipLaunchKernelGGL(k_act_streams<true>, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
+        hipLaunchKernelGGL((k_act_streams<true, XT>), dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
                            streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     else
-        hipLaunchKernelGGL(k_act_streams<false>, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
-                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
+        hipLaunchKernelGGL((k_act_streams<false, XT>), dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s,
+                           x, streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s)
+{
+    return launch_act_streams_t(g, x, streams, tables, s);
+}
+
+int launch_act_streams_q7(const Geometry& g, const uint8_t* x, uint32_t* streams, const uint32_t* tables,
+                          hipStream_t s)
+{
+    return launch_act_streams_t(g, x, streams, tables, s);
 }
 
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,

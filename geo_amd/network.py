@@ -72,6 +72,35 @@ class CONV_tiny_add_partial(nn.Module):
         return self.bn4(x.view(-1, self.num_classes))
 
 
+    @torch.no_grad()
+    def forward_fused(self, x_in):
+        """Inference forward with one fused epilogue kernel per layer in place of the element-wise
+        op chain (fixed batch norm on the running statistics, relu, AvgPool2, Hardtanh, the next
+        layer's 7-bit quantisation): layers hand each other uint8 7-bit integers, which the
+        activation stream generator reads directly.  Same logits, bit for bit, as ``forward`` in
+        eval mode."""
+        if self.training:
+            raise RuntimeError("forward_fused is the inference path: call model.eval() first")
+        if self.legacy or self.generator != "lfsr":
+            raise NotImplementedError("forward_fused runs the LFSR kernels only")
+        from . import capi, utils_functional as uf
+        layers = [(self.conv1, self.bn1, 0, 0), (self.conv2, self.bn2, 1, 1), (self.conv3, self.bn3, 2, 2),
+                  (self.fc1, self.bn4, 3, 2)]  # (conv, bn, layer index, index of its weight wait)
+        x = uf.quantize(x_in.detach().float(), prec=7)
+        for conv, bn, i, j in layers:
+            conv.weight.data = uf.quantize(conv.weight_org, prec=7)
+            L = 2 ** self.err[i]
+            counts = uf.sc_counts(x, conv.weight.data, L, conv.padding, forward=self.compute,
+                                  load_unit=self.load_unit[i], load_wait_w=self.load_wait[j],
+                                  load_wait_a=self.load_wait[i], z_unit=2 ** self.z_unit[i])
+            w_n, b_n = utils_class._fixed_affine(bn, None, bn.running_mean, bn.running_var)
+            if bn is self.bn4:
+                logits, _ = capi.layer_epilogue(counts, L, w_n, b_n, relu=False, pool=False, hardtanh=False,
+                                                quant7=False)
+                return logits.view(-1, self.num_classes)
+            _, x = capi.layer_epilogue(counts, L, w_n, b_n, relu=self.relu, want_act=False, want_q7=True)
+
+
 def make_param_copies(model):
     """Full-precision master copies the optimiser updates (main_conv.py:203-213)."""
     return [p.detach().clone().float().requires_grad_(True) for p in model.parameters()]

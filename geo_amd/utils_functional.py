@@ -171,6 +171,24 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), load_unit, load_wait_w)
 
 
+def sc_counts(activation, weight, bit_length, padding, forward="1d_bin", load_unit=8, load_wait_w=1, load_wait_a=1,
+              z_unit=1024):
+    """int32 SC counts of one layer without autograd (inference).  ``activation`` is fp32, or
+    uint8 holding the 7-bit integers round(x * 128) that the fused layer epilogue emits.  Same
+    argument meaning as ``conv2d_generic``'s keywords (utils_functional.py:406-510)."""
+    if forward not in ("1d_bin", "z_bin", "yz_bin"):
+        raise NotImplementedError(f"sc_counts(forward={forward!r})")
+    mode = {"1d_bin": "y", "z_bin": "z", "yz_bin": "yz"}[forward]
+    wait_a = load_wait_a if mode == "yz" else load_wait_w
+    kw = dict(total_width=prec_default, load_width=int(load_unit), load_wait_w=int(load_wait_w),
+              load_wait_a=int(wait_a), accumulate=mode, z_unit=max(1, min(int(z_unit), activation.shape[1])))
+    pad = (int(padding[0]), int(padding[1]))
+    w = weight.detach().float().contiguous()
+    if activation.dtype == torch.uint8:
+        return capi.conv2d_add_partial_forward_q7(activation.contiguous(), w, int(bit_length), pad, **kw)
+    return capi.conv2d_add_partial_forward(activation.detach().float().contiguous(), w, int(bit_length), pad, **kw)
+
+
 def smoke_layer_step():
     """One SC layer forward + backward on cuda:0 against the torch surrogate (used by the
     smoke check)."""

@@ -177,6 +177,41 @@ GEO_SC_API int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, 
                                                   void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
 
 /*
+ * Layer epilogue fused into one pass over the convolution's int32 counts.  Replaces the chain of
+ * PyTorch element-wise ops between two SC layers of the reference's networks
+ * (network.py:165-170): count / L (utils_functional.py:632) -> value of BatchNorm2d_fixed /
+ * BatchNorm1d_fixed, x * w_n[c] + b_n[c] with the caller's quantised per-channel w_n, b_n
+ * (utils_class.py:52-64) -> optional relu (network.py:167) -> optional AvgPool2d(2) (:169) ->
+ * optional Hardtanh(0, 1) (:170) -> optional round(v * 128).clamp(-127, 127) / 128, the next
+ * layer's input quantisation (utils_class.py:32, utils_functional.py:33-39).  Same operation order
+ * and rounding as the op chain: the fp32 result is identical.
+ *   counts            int32 (n, c, w, h)
+ *   act_out           fp32 (n, c, wo, ho), wo = w/2, ho = h/2 with GEO_SC_EPI_POOL2 (floor), else w, h;
+ *                     may be NULL when q7_out is given
+ *   q7_out            uint8 (n, c, wo, ho): the integer round(v * 128) in [0, 127]; may be NULL; needs
+ *                     GEO_SC_EPI_HARDTANH01 | GEO_SC_EPI_QUANT7
+ */
+enum geo_sc_epilogue_flags {
+    GEO_SC_EPI_RELU = 1,
+    GEO_SC_EPI_POOL2 = 2,
+    GEO_SC_EPI_HARDTANH01 = 4,
+    GEO_SC_EPI_QUANT7 = 8
+};
+GEO_SC_API int geo_sc_layer_epilogue(const int32_t* counts, int n, int c, int w, int h, int bit_length,
+                                     const float* w_n, const float* b_n, int flags, float* act_out,
+                                     uint8_t* q7_out, geo_sc_stream_t stream);
+
+/*
+ * geo_sc_conv2d_add_partial_forward for activations given as the 7-bit integers k = round(x * 128)
+ * that geo_sc_layer_epilogue emits (uint8 (n, c_in, w_in, h_in), k <= 127): the activation is
+ * x = k / 128, exactly what the reference's layer computes from after its input quantisation
+ * (utils_class.py:32), so the counts equal those of the fp32 entry point on x.  Same workspace.
+ */
+GEO_SC_API int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7,
+                                                    const float* w, int32_t* y, void* workspace,
+                                                    size_t workspace_bytes, geo_sc_stream_t stream);
+
+/*
  * Measurement aid, no counterpart in the reference: enqueues a loop of `iters` x 64
  * v_and_or_b32 instructions per wave (SGPR weight operand, no memory traffic) on 4 waves per
  * SIMD of 256 CUs and reports in *word_ops how many 32-bit lane operations that is; the

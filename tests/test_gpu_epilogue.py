@@ -1,0 +1,122 @@
+"""GPU parity of the fused layer epilogue and of the 7-bit-integer activation input, through the
+C ABI, against the CPU oracle and against the PyTorch op chain; and of the fused inference
+forward of the 4-layer CNN against its module-by-module forward.  Bit-exact."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from geo_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from geo_amd import capi as m
+    return m
+
+
+def _inputs(seed, shape, L, H=5):
+    g = torch.Generator().manual_seed(seed)
+    counts = torch.randint(-H * L, H * L + 1, shape, generator=g, dtype=torch.int32)
+    w_n = torch.randint(-127, 128, (shape[1],), generator=g).float() / 128 * 4.0
+    b_n = torch.randint(-127, 128, (shape[1],), generator=g).float() / 128 * 4.0
+    return counts, w_n, b_n
+
+
+@pytest.mark.parametrize("shape,L", [((3, 5, 8, 6), 64), ((2, 3, 7, 5), 256), ((4, 32, 32, 32), 128),
+                                     ((70, 10, 1, 1), 64)])
+@pytest.mark.parametrize("relu,pool,hardtanh,quant7", [(False, True, True, True), (True, True, True, True),
+                                                       (False, False, False, False), (False, False, True, True),
+                                                       (True, True, False, True)])
+def test_epilogue_matches_oracle(capi, shape, L, relu, pool, hardtanh, quant7):
+    from oracle import epilogue
+    if pool and min(shape[2:]) < 2:
+        pytest.skip("nothing to pool")
+    counts, w_n, b_n = _inputs(L + shape[0], shape, L)
+    want_q7 = hardtanh and quant7
+    act, q7 = capi.layer_epilogue(counts.cuda(), L, w_n, b_n, relu, pool, hardtanh, quant7, want_q7=want_q7)
+    torch.cuda.synchronize()
+    e_act, e_q7 = epilogue.layer_epilogue(counts.numpy(), L, w_n.numpy(), b_n.numpy(), relu, pool, hardtanh, quant7)
+    assert np.array_equal(act.cpu().numpy(), e_act)
+    if want_q7:
+        assert np.array_equal(q7.cpu().numpy(), e_q7)
+        only_q7 = capi.layer_epilogue(counts.cuda(), L, w_n, b_n, relu, pool, hardtanh, quant7, want_act=False,
+                                      want_q7=True)
+        assert only_q7[0] is None and torch.equal(only_q7[1], q7)
+
+
+def test_epilogue_matches_torch_ops_on_real_counts(capi):
+    """Counts of an SC layer, the affine of a BatchNorm2d_fixed in eval mode, and the op chain
+    as the reference's network runs it (network.py:165-170)."""
+    from geo_amd import utils_class, utils_functional as uf
+    x, w = wl.make_inputs((8, 16, 12, 12), (24, 16, 5, 5), "q7", seed=3)
+    counts = capi.conv2d_add_partial_forward(x.cuda(), w.cuda(), 64, (2, 2))
+    bn = utils_class.BatchNorm2d_fixed(24).cuda().eval()
+    with torch.no_grad():
+        bn.running_mean.uniform_(-0.2, 0.2)
+        bn.running_var.uniform_(0.05, 0.5)
+        bn.weight.uniform_(0.5, 1.5)
+        bn.bias.uniform_(-0.3, 0.3)
+        ref = uf.quantize(F.hardtanh(F.avg_pool2d(bn(counts.float() / 64), 2), 0, 1), prec=7)
+        w_n, b_n = utils_class._fixed_affine(bn, None, bn.running_mean, bn.running_var)
+    act, q7 = capi.layer_epilogue(counts, 64, w_n, b_n, want_q7=True)
+    assert torch.equal(act, ref)
+    assert torch.equal(q7.float() / 128, ref)
+
+
+@pytest.mark.parametrize("L", [8, 64, 128, 256])
+@pytest.mark.parametrize("mode,zu", [("y", 1), ("z", 1), ("yz", 2)])
+def test_q7_activations_give_the_fp32_counts(capi, L, mode, zu):
+    g = torch.Generator().manual_seed(L)
+    k = torch.randint(0, 128, (3, 5, 7, 6), generator=g, dtype=torch.uint8)
+    _, w = wl.make_inputs((3, 5, 7, 6), (19, 5, 3, 3), "prescribed", seed=L)
+    wd = w.cuda()
+    for loading in ((7, 8, 1, 1), (7, 2, 2, 3)):
+        a = capi.conv2d_add_partial_forward_q7(k.cuda(), wd, L, (1, 1), *loading, accumulate=mode, z_unit=zu)
+        b = capi.conv2d_add_partial_forward((k.float() / 128).cuda(), wd, L, (1, 1), *loading, accumulate=mode,
+                                            z_unit=zu)
+        assert torch.equal(a, b)
+    # single-row outputs use the batch-item-innermost stream layout
+    k1 = torch.randint(0, 128, (6, 4, 3, 8), generator=g, dtype=torch.uint8)
+    _, w1 = wl.make_inputs((6, 4, 3, 8), (5, 4, 3, 3), "prescribed", seed=1)
+    assert torch.equal(capi.conv2d_add_partial_forward_q7(k1.cuda(), w1.cuda(), L),
+                       capi.conv2d_add_partial_forward((k1.float() / 128).cuda(), w1.cuda(), L))
+
+
+def test_epilogue_argument_errors(capi):
+    counts, w_n, b_n = _inputs(0, (2, 3, 4, 4), 64)
+    with pytest.raises(capi.GeoScError):
+        capi.layer_epilogue(counts.cuda(), 100, w_n, b_n)
+    with pytest.raises(capi.GeoScError):   # the 7-bit output needs the clamp and the quantisation
+        capi.layer_epilogue(counts.cuda(), 64, w_n, b_n, hardtanh=False, want_q7=True)
+    with pytest.raises(ValueError):
+        capi.layer_epilogue(counts.cuda(), 64, w_n[:2], b_n)
+    with pytest.raises(ValueError):
+        capi.layer_epilogue(counts, 64, w_n, b_n)
+
+
+@pytest.mark.parametrize("compute,relu", [("1d_bin", False), ("1d_bin", True), ("yz_bin", False)])
+def test_fused_inference_forward_equals_module_forward(compute, relu):
+    from geo_amd import network
+    torch.manual_seed(0)
+    model = network.CONV_tiny_add_partial(sc_compute=compute, relu=relu).cuda()
+    model.err = [6, 6, 6, 6]
+    with torch.no_grad():
+        for bn in (model.bn1, model.bn2, model.bn3, model.bn4):
+            bn.running_mean.uniform_(-0.1, 0.3)
+            bn.running_var.uniform_(0.02, 0.3)
+            bn.weight.uniform_(0.5, 1.5)
+            bn.bias.uniform_(-0.2, 0.4)
+    model.eval()
+    x = torch.rand(16, 3, 32, 32, generator=torch.Generator().manual_seed(1)).cuda()
+    with torch.no_grad():
+        ref = model(x.clone())
+    got = model.forward_fused(x.clone())
+    assert got.shape == ref.shape == (16, 10)
+    assert torch.equal(got, ref)
+    model.train()
+    with pytest.raises(RuntimeError):
+        model.forward_fused(x)
