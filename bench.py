@@ -198,6 +198,76 @@ def bench_network_step(args, torch):
     print(json.dumps(result))
 
 
+def bench_network_inference(args, torch):
+    """4-layer SC CNN inference forward at batch 256 (eval mode, running statistics): the fused
+    path (one epilogue kernel per layer, 7-bit integer activations between layers) with the
+    module-by-module forward (PyTorch element-wise ops between the SC kernels) timed beside it."""
+    from geo_amd import network
+    from geo_amd import workloads as wl
+
+    L = args.length or 64
+    torch.manual_seed(0)
+    model = network.CONV_tiny_add_partial().cuda().eval()
+    model.err = [L.bit_length() - 1] * 4
+    model.load_unit = [2] * 4
+    model.load_wait = [2] * 4
+    x = torch.rand((256, 3, 32, 32), generator=torch.Generator().manual_seed(0)).cuda()
+
+    def fused():
+        return model.forward_fused(x)
+
+    def fused_eager():  # second timing loop: the same forward replayed from a HIP graph
+        return model.forward_fused(x, graph=True)
+
+    def modules():
+        with torch.no_grad():
+            return model(x.clone())
+
+    same = bool(torch.equal(fused(), modules()))
+    for _ in range(args.warmup):
+        fused()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fused()
+    torch.cuda.synchronize()
+    ms_fused = (time.perf_counter() - t0) * 1e3 / args.steps
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        modules()
+    torch.cuda.synchronize()
+    ms_modules = (time.perf_counter() - t0) * 1e3 / args.steps
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fused_eager()
+    torch.cuda.synchronize()
+    ms_eager = (time.perf_counter() - t0) * 1e3 / args.steps
+    B_total = sum(wl.bit_macs(sx, sw, pad, L) for _, sx, sw, pad in C2_LAYERS)
+    # the epilogue kernel of the first layer alone, against the bytes it has to move
+    from geo_amd import capi
+    counts = torch.randint(-5 * L, 5 * L, (256, 32, 32, 32), dtype=torch.int32, device="cuda")
+    wn = torch.rand(32, device="cuda")
+    bn = torch.rand(32, device="cuda")
+    e = time_events(lambda: capi.layer_epilogue(counts, L, wn, bn, want_act=False, want_q7=True), args.steps, 2, torch)
+    e_ms = sum(e) / len(e)
+    e_bytes = counts.numel() * 4 + counts.numel() // 4
+    print(json.dumps({
+        "metric": f"SC bit-MACs/sec over one inference forward of the 4-layer SC CNN at stream len {L}",
+        "value": B_total / (ms_fused * 1e-3), "unit": "bit-MAC/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_fused, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u32 bit-packed streams, int32 accumulate; u8 activations between layers",
+        "data": "synthetic (torch.manual_seed(0); images U[0,1))",
+        "config": {"workload": "C2: 4-layer SC CNN inference forward, batch 256, fused layer epilogues, cached weight "
+                               "streams, stream "
+                               f"length {L}, load_unit 2 / load_wait 2", "pass": "fwd", "bit_macs_per_step": B_total},
+        "module_forward_ms": ms_modules, "fused_as_hip_graph_replay_ms": ms_eager, "fused_equals_module_forward": same,
+        "roofline": {"bound": "hbm", "kernel": "k_layer_epilogue on (256, 32, 32, 32) counts", "achieved":
+                     e_bytes / (e_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
+                     "frac": e_bytes / (e_ms * 1e-3) / 8e12, "kernel_ms_avg": e_ms, "algorithmic_bytes": e_bytes,
+                     "traffic": None},
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -211,7 +281,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     if args.workload == "C2":
-        bench_network_step(args, torch)
+        if args.passes == "fwd":
+            bench_network_inference(args, torch)
+        else:
+            bench_network_step(args, torch)
         return
     from geo_amd import capi
     from geo_amd import workloads as wl

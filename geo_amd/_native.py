@@ -38,6 +38,7 @@ C_API = {
     "geo_sc_stream_tables_size": (ctypes.c_int, [ctypes.c_int, _SZ]),
     "geo_sc_act_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
     "geo_sc_weight_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
+    "geo_sc_act_streams_q7": (ctypes.c_int, [_D, _P, _P, _P, _P]),
     "geo_sc_act_stream_words": (ctypes.c_int, [_D, _SZ]),
     "geo_sc_probe_and_or_rate": (ctypes.c_int, [ctypes.c_int, _P, ctypes.c_size_t, ctypes.POINTER(ctypes.c_double), _P]),
     "geo_sc_conv2d_add_partial_backward_workspace_size": (ctypes.c_int, [_D, _SZ]),

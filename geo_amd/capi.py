@@ -147,8 +147,14 @@ def _tables(bit_length, device):
 
 
 def act_streams(x, desc: ConvDesc, stream=None):
-    """int32-typed tensor of stream words [N][P][Cin][Wi][Hi] (reinterpret as uint32)."""
-    _require_gpu_f32(x, "x")
+    """int32-typed tensor of stream words [N][P][Cin][Wi][Hi] (reinterpret as uint32).  ``x`` is
+    fp32, or uint8 holding the 7-bit integers round(x * 128)."""
+    q7 = x.dtype == torch.uint8
+    if q7:
+        if not (x.is_cuda and x.is_contiguous()):
+            raise ValueError("x must be a contiguous GPU tensor")
+    else:
+        _require_gpu_f32(x, "x")
     n = ctypes.c_size_t(0)
     _check(_native.lib().geo_sc_act_stream_words(ctypes.byref(desc), ctypes.byref(n)), "act words")
     packs = (desc.bit_length + 31) // 32
@@ -156,8 +162,8 @@ def act_streams(x, desc: ConvDesc, stream=None):
     out = torch.empty((desc.n, packs, desc.c_in, wi, hi), dtype=torch.int32, device=x.device)
     assert out.numel() == n.value
     tables = _tables(desc.bit_length, x.device)
-    _check(_native.lib().geo_sc_act_streams(ctypes.byref(desc), _ptr(x), _ptr(out), _ptr(tables),
-                                            _stream_ptr(stream)), "geo_sc_act_streams")
+    fn = _native.lib().geo_sc_act_streams_q7 if q7 else _native.lib().geo_sc_act_streams
+    _check(fn(ctypes.byref(desc), _ptr(x), _ptr(out), _ptr(tables), _stream_ptr(stream)), "geo_sc_act_streams")
     return out
 
 

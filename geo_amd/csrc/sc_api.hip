@@ -187,6 +187,19 @@ int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* s
     return launch_act_streams(g, x, streams, (const uint32_t*)tables, s);
 }
 
+int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, uint32_t* streams, void* tables,
+                          geo_sc_stream_t stream)
+{
+    Geometry g;
+    int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!x_q7 || !streams || !tables) return GEO_SC_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    rc = launch_build_tables(g, (uint32_t*)tables, s);
+    if (rc != GEO_SC_OK) return rc;
+    return launch_act_streams_q7(g, x_q7, streams, (const uint32_t*)tables, s);
+}
+
 int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
                           geo_sc_stream_t stream)
 {

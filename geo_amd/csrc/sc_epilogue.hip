@@ -69,6 +69,44 @@ __global__ __launch_bounds__(256) void k_layer_epilogue(EpiParams q)
     }
 }
 
+// AvgPool2 case with h a multiple of 4: a thread produces two adjacent outputs from two 16-byte
+// loads (one per input row), 32-bit index arithmetic; a wave reads two contiguous 1 KB runs.
+__global__ __launch_bounds__(256) void k_layer_epilogue_pool_vec(EpiParams q, unsigned pairs_per_row, unsigned n_pairs)
+{
+    const bool relu = q.flags & GEO_SC_EPI_RELU;
+    for (unsigned e = blockIdx.x * 256 + threadIdx.x; e < n_pairs; e += gridDim.x * 256) {
+        const unsigned b2 = e % pairs_per_row;
+        unsigned t = e / pairs_per_row;
+        const unsigned a = t % (unsigned)q.wo;
+        t /= (unsigned)q.wo;
+        const unsigned ch = t % (unsigned)q.c;
+        const float wn = q.w_n[ch], bn = q.b_n[ch];
+        const int32_t* src = q.counts + ((size_t)t * q.w + 2 * a) * q.h + 4 * b2;
+        const int4 r0 = *reinterpret_cast<const int4*>(src);
+        const int4 r1 = *reinterpret_cast<const int4*>(src + q.h);
+        float v[2];
+        v[0] = __fadd_rn(__fadd_rn(__fadd_rn(affine(r0.x, q.inv_len, wn, bn, relu), affine(r0.y, q.inv_len, wn, bn, relu)),
+                                   affine(r1.x, q.inv_len, wn, bn, relu)),
+                         affine(r1.y, q.inv_len, wn, bn, relu)) / 4.0f;
+        v[1] = __fadd_rn(__fadd_rn(__fadd_rn(affine(r0.z, q.inv_len, wn, bn, relu), affine(r0.w, q.inv_len, wn, bn, relu)),
+                                   affine(r1.z, q.inv_len, wn, bn, relu)),
+                         affine(r1.w, q.inv_len, wn, bn, relu)) / 4.0f;
+        uint8_t k8[2] = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (q.flags & GEO_SC_EPI_HARDTANH01) v[i] = fminf(fmaxf(v[i], 0.0f), 1.0f);
+            if (q.flags & GEO_SC_EPI_QUANT7) {
+                const float k = fminf(fmaxf(rintf(__fmul_rn(v[i], 128.0f)), -127.0f), 127.0f);
+                v[i] = k / 128.0f;
+                k8[i] = (uint8_t)(int)k;
+            }
+        }
+        const size_t o = (size_t)e * 2;
+        if (q.q7) *reinterpret_cast<uchar2*>(q.q7 + o) = make_uchar2(k8[0], k8[1]);
+        if (q.act) *reinterpret_cast<float2*>(q.act + o) = make_float2(v[0], v[1]);
+    }
+}
+
 }  // namespace
 
 }  // namespace geo_sc
@@ -105,6 +143,15 @@ extern "C" int geo_sc_layer_epilogue(const int32_t* counts, int n, int c, int w,
     q.total = (long long)n * c * q.wo * q.ho;
     q.inv_len = 1.0f / (float)bit_length;
     q.flags = flags;
+    const bool aligned = (((uintptr_t)counts & 15) | ((uintptr_t)act_out & 7) | ((uintptr_t)q7_out & 1)) == 0;
+    if ((flags & GEO_SC_EPI_POOL2) && h % 4 == 0 && aligned && q.total < 0xffffffffLL) {
+        const unsigned n_pairs = (unsigned)(q.total / 2);
+        long long vb = ((long long)n_pairs + 255) / 256;
+        if (vb > 256 * 32) vb = 256 * 32;
+        hipLaunchKernelGGL(k_layer_epilogue_pool_vec, dim3((unsigned)vb), dim3(256), 0, (hipStream_t)stream, q,
+                           (unsigned)(q.ho / 2), n_pairs);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
     long long blocks = (q.total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     hipLaunchKernelGGL(k_layer_epilogue, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, q);

@@ -72,33 +72,82 @@ class CONV_tiny_add_partial(nn.Module):
         return self.bn4(x.view(-1, self.num_classes))
 
 
+    # ---------------------------------------------------------------- fused inference path
+    def train(self, mode=True):
+        self._fused = None  # parameters may change: drop the cached inference state
+        return super().train(mode)
+
     @torch.no_grad()
-    def forward_fused(self, x_in):
-        """Inference forward with one fused epilogue kernel per layer in place of the element-wise
-        op chain (fixed batch norm on the running statistics, relu, AvgPool2, Hardtanh, the next
-        layer's 7-bit quantisation): layers hand each other uint8 7-bit integers, which the
-        activation stream generator reads directly.  Same logits, bit for bit, as ``forward`` in
-        eval mode."""
-        if self.training:
-            raise RuntimeError("forward_fused is the inference path: call model.eval() first")
-        if self.legacy or self.generator != "lfsr":
+    def prepare_fused(self):
+        """Cache what an inference forward does not need to recompute: per layer the weight streams
+        of the 7-bit-quantised weights and the quantised per-channel affine of its fixed batch
+        norm on the running statistics.  Call again after changing parameters or settings."""
+        if self.legacy or self.generator != "lfsr" or self.compute not in ("1d_bin", "z_bin", "yz_bin"):
             raise NotImplementedError("forward_fused runs the LFSR kernels only")
         from . import capi, utils_functional as uf
         layers = [(self.conv1, self.bn1, 0, 0), (self.conv2, self.bn2, 1, 1), (self.conv3, self.bn3, 2, 2),
-                  (self.fc1, self.bn4, 3, 2)]  # (conv, bn, layer index, index of its weight wait)
-        x = uf.quantize(x_in.detach().float(), prec=7)
+                  (self.fc1, self.bn4, 3, 2)]  # (conv, bn, layer index, index of its weight wait: network.py:186)
+        mode = {"1d_bin": "y", "z_bin": "z", "yz_bin": "yz"}[self.compute]
+        state = []
         for conv, bn, i, j in layers:
             conv.weight.data = uf.quantize(conv.weight_org, prec=7)
-            L = 2 ** self.err[i]
-            counts = uf.sc_counts(x, conv.weight.data, L, conv.padding, forward=self.compute,
-                                  load_unit=self.load_unit[i], load_wait_w=self.load_wait[j],
-                                  load_wait_a=self.load_wait[i], z_unit=2 ** self.z_unit[i])
+            w = conv.weight.data.float().contiguous()
+            wait_w = self.load_wait[j]
+            kw = dict(bit_length=2 ** self.err[i], padding=(int(conv.padding[0]), int(conv.padding[1])),
+                      total_width=uf.prec_default, load_width=int(self.load_unit[i]), load_wait_w=int(wait_w),
+                      load_wait_a=int(self.load_wait[i] if mode == "yz" else wait_w), accumulate=mode,
+                      z_unit=max(1, min(2 ** self.z_unit[i], w.shape[1])))
+            d = capi.make_desc((2, w.shape[1], w.shape[2], w.shape[3]), w.shape, **kw)  # weights do not depend on n
             w_n, b_n = utils_class._fixed_affine(bn, None, bn.running_mean, bn.running_var)
-            if bn is self.bn4:
-                logits, _ = capi.layer_epilogue(counts, L, w_n, b_n, relu=False, pool=False, hardtanh=False,
-                                                quant7=False)
+            state.append(dict(w_shape=tuple(w.shape), kw=kw, wgt=capi.weight_streams(w, d),
+                              w_n=w_n.float().contiguous(), b_n=b_n.float().contiguous()))
+        self._fused = state
+        self._fused_graph = None
+
+    def _fused_eager(self, x):
+        from . import capi
+        last = len(self._fused) - 1
+        for i, st in enumerate(self._fused):
+            d = capi.make_desc(x.shape, st["w_shape"], **st["kw"])
+            counts = capi.conv2d_add_partial_from_streams(capi.act_streams(x, d), st["wgt"], d)
+            L = st["kw"]["bit_length"]
+            if i == last:
+                logits, _ = capi.layer_epilogue(counts, L, st["w_n"], st["b_n"], relu=False, pool=False,
+                                                hardtanh=False, quant7=False)
                 return logits.view(-1, self.num_classes)
-            _, x = capi.layer_epilogue(counts, L, w_n, b_n, relu=self.relu, want_act=False, want_q7=True)
+            _, x = capi.layer_epilogue(counts, L, st["w_n"], st["b_n"], relu=self.relu, want_act=False, want_q7=True)
+
+    @torch.no_grad()
+    def forward_fused(self, x_in, graph=False):
+        """Inference forward with one fused epilogue kernel per layer in place of the element-wise
+        op chain (fixed batch norm on the running statistics, relu, AvgPool2, Hardtanh, the next
+        layer's 7-bit quantisation): layers hand each other uint8 7-bit integers, which the
+        activation stream generator reads directly, and weight streams come from the cache of
+        ``prepare_fused``.  Same logits, bit for bit, as ``forward`` in eval mode.  ``graph=True``
+        records the launches of one forward into a HIP graph per input shape and replays it."""
+        if self.training:
+            raise RuntimeError("forward_fused is the inference path: call model.eval() first")
+        from . import utils_functional as uf
+        if getattr(self, "_fused", None) is None:
+            self.prepare_fused()
+        x = uf.quantize(x_in.detach().float(), prec=7).contiguous()
+        if not graph:
+            return self._fused_eager(x)
+        g = self._fused_graph
+        if g is None or g["x"].shape != x.shape:
+            static_x = x.clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):  # warm the allocator and the kernels outside the capture
+                self._fused_eager(static_x)
+            torch.cuda.current_stream().wait_stream(side)
+            cg = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(cg):
+                out = self._fused_eager(static_x)
+            g = self._fused_graph = dict(x=static_x, out=out, graph=cg)
+        g["x"].copy_(x)
+        g["graph"].replay()
+        return g["out"].clone()
 
 
 def make_param_copies(model):

@@ -211,6 +211,12 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc
                                                     const float* w, int32_t* y, void* workspace,
                                                     size_t workspace_bytes, geo_sc_stream_t stream);
 
+/* geo_sc_act_streams for the uint8 7-bit integer activations of geo_sc_conv2d_add_partial_forward_q7:
+ * with weight streams generated once by geo_sc_weight_streams, an inference loop runs this, then
+ * geo_sc_conv2d_add_partial_from_streams, then geo_sc_layer_epilogue per layer. */
+GEO_SC_API int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, uint32_t* streams,
+                                     void* tables, geo_sc_stream_t stream);
+
 /*
  * Measurement aid, no counterpart in the reference: enqueues a loop of `iters` x 64
  * v_and_or_b32 instructions per wave (SGPR weight operand, no memory traffic) on 4 waves per

@@ -117,6 +117,27 @@ def test_fused_inference_forward_equals_module_forward(compute, relu):
     got = model.forward_fused(x.clone())
     assert got.shape == ref.shape == (16, 10)
     assert torch.equal(got, ref)
+    # HIP-graph replays, with eager work and synchronisations between them, against eager results
+    for seed in (2, 3, 4):
+        xs = torch.rand(16, 3, 32, 32, generator=torch.Generator().manual_seed(seed)).cuda()
+        with torch.no_grad():
+            ref_s = model(xs.clone())
+        torch.cuda.synchronize()
+        assert torch.equal(model.forward_fused(xs, graph=True), ref_s), seed
+    # another batch size records another graph
+    xb = torch.rand(5, 3, 32, 32, generator=torch.Generator().manual_seed(9)).cuda()
+    with torch.no_grad():
+        ref_b = model(xb.clone())
+    assert torch.equal(model.forward_fused(xb, graph=True), ref_b)
+    # parameters changed: the cache is rebuilt after train()/eval()
+    model.train()
+    with torch.no_grad():
+        model.conv2.weight_org.mul_(0.5)
+    model.eval()
+    with torch.no_grad():
+        ref2 = model(x.clone())
+    assert not torch.equal(ref2, ref)
+    assert torch.equal(model.forward_fused(x.clone()), ref2)
     model.train()
     with pytest.raises(RuntimeError):
         model.forward_fused(x)
