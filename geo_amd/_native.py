@@ -22,7 +22,7 @@ class ConvDesc(ctypes.Structure):
     """geo_sc_conv_desc of include/geo_sc.h"""
     _fields_ = [(n, ctypes.c_int32) for n in (
         "n", "c_in", "w_in", "h_in", "c_out", "w_k", "h_k", "pad_w", "pad_h", "bit_length",
-        "total_width", "load_width", "load_wait_w", "load_wait_a", "accumulate", "z_unit")]
+        "total_width", "load_width", "load_wait_w", "load_wait_a", "accumulate", "z_unit", "generator", "seed")]
 
 
 # every symbol include/geo_sc.h declares: name -> (restype, argtypes)

@@ -28,11 +28,13 @@ def _check(status: int, what: str):
 
 
 # enum geo_sc_accumulate
-ACCUMULATE = {"y": 0, "z": 1, "yz": 2}
+ACCUMULATE = {"y": 0, "z": 1, "yz": 2, "full": 3}
+# enum geo_sc_generator
+GENERATOR = {"lfsr": 0, "acc": 1, "rand": 2}
 
 
 def make_desc(x_shape, w_shape, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
-              load_wait_a=1, accumulate="y", z_unit=1) -> ConvDesc:
+              load_wait_a=1, accumulate="y", z_unit=1, generator="lfsr", seed=0) -> ConvDesc:
     """``padding=(p0, p1)`` follows the reference: p0 pads the last dim, p1 the one before.
     ``accumulate``: "y" (OR over c_in and w_k, add over h_k), "z" (OR over the kernel window, add
     over c_in) or "yz" (OR over ``z_unit`` channels and w_k, add over h_k and channel groups)."""
@@ -42,7 +44,9 @@ def make_desc(x_shape, w_shape, bit_length, padding=(0, 0), total_width=7, load_
         raise ValueError(f"channel mismatch: {c_in} vs {c_in2}")
     return ConvDesc(n, c_in, w_in, h_in, c_out, w_k, h_k, int(padding[1]), int(padding[0]), int(bit_length),
                     int(total_width), int(load_width), int(load_wait_w), int(load_wait_a),
-                    ACCUMULATE[accumulate] if isinstance(accumulate, str) else int(accumulate), int(z_unit))
+                    ACCUMULATE[accumulate] if isinstance(accumulate, str) else int(accumulate), int(z_unit),
+                    GENERATOR[generator] if isinstance(generator, str) else int(generator),
+                    ctypes.c_int32(int(seed) & 0xffffffff).value)
 
 
 def _stream_ptr(stream=None):
@@ -76,13 +80,13 @@ def _require_gpu_f32(t, name):
 
 def conv2d_add_partial_forward(x, w, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
                                load_wait_a=1, out=None, workspace=None, stream=None, desc=None, accumulate="y",
-                               z_unit=1):
+                               z_unit=1, generator="lfsr", seed=0):
     """int32 (N, Cout, Wo, Ho) GPU tensor via geo_sc_conv2d_add_partial_forward."""
     _require_gpu_f32(x, "x")
     _require_gpu_f32(w, "w")
     if desc is None:
         desc = make_desc(x.shape, w.shape, bit_length, padding, total_width, load_width, load_wait_w, load_wait_a,
-                         accumulate, z_unit)
+                         accumulate, z_unit, generator, seed)
     ws_bytes = workspace_size(desc)
     if workspace is None:
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)

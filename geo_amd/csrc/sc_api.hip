@@ -44,7 +44,13 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     g->load_width = d->load_width > g->total_width + 1 ? g->total_width + 1 : d->load_width;
     g->load_wait_w = d->load_wait_w;
     g->load_wait_a = d->load_wait_a;
-    if (d->accumulate < GEO_SC_ACC_Y || d->accumulate > GEO_SC_ACC_YZ) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (d->accumulate < GEO_SC_ACC_Y || d->accumulate > GEO_SC_ACC_FULL) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (d->generator < GEO_SC_GEN_LFSR || d->generator > GEO_SC_GEN_RAND) return GEO_SC_ERR_INVALID_ARGUMENT;
+    // the random generators exist for the Y and FULL accumulations only (sc_cuda.cpp:21-32, :65-76)
+    if (d->generator != GEO_SC_GEN_LFSR && d->accumulate != GEO_SC_ACC_Y && d->accumulate != GEO_SC_ACC_FULL)
+        return GEO_SC_ERR_INVALID_ARGUMENT;
+    g->generator = d->generator;
+    g->seed = (uint32_t)d->seed;
     if (d->accumulate == GEO_SC_ACC_YZ && d->z_unit < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
     g->mode = d->accumulate;
     g->z_unit = (d->accumulate == GEO_SC_ACC_YZ && d->z_unit < d->c_in) ? d->z_unit : d->c_in;
@@ -65,11 +71,18 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     g->n_cotile = (d->c_out + kCoTile - 1) / kCoTile;
     g->act_plane = (size_t)plane;
     g->act_words = (size_t)d->n * g->packs * g->act_plane;
+    g->or_rows = 1;
     if (g->mode == GEO_SC_ACC_Z) {
         g->add_outer = 1;
         g->add_inner = d->c_in;
         g->or_ch_total = d->h_k;
         g->or_ch_per_group = d->h_k;
+    } else if (g->mode == GEO_SC_ACC_FULL) {
+        g->add_outer = 1;
+        g->add_inner = 1;
+        g->or_ch_total = d->c_in;
+        g->or_ch_per_group = d->c_in;
+        g->or_rows = d->h_k;
     } else {
         g->add_outer = (d->c_in + g->z_unit - 1) / g->z_unit;
         g->add_inner = d->h_k;
@@ -77,7 +90,7 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
         g->or_ch_per_group = g->z_unit;
     }
     g->seed_wrap = g->mode == GEO_SC_ACC_YZ ? (size_t)g->z_unit * wi * hi : (size_t)plane;
-    g->act_item_inner = g->mode == GEO_SC_ACC_Y && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
+    g->act_item_inner = g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
     g->wgt_words = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile * 2 * kCoTile;
     g->off_tables = 0;

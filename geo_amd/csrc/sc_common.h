@@ -25,7 +25,11 @@ struct Geometry {
     //   Y : add_outer 1,              add_inner h_k,  OR channels = input channels
     //   YZ: add_outer channel groups, add_inner h_k,  OR channels = the group's input channels
     //   Z : add_outer 1,              add_inner c_in, OR channels = kernel rows (h_k)
-    int add_outer, add_inner, or_ch_total, or_ch_per_group;
+    //   FULL: add_outer 1,            add_inner 1,    OR channels = input channels, and the OR also
+    //         runs over or_rows = h_k kernel rows before the popcount (Y-mode weight line order)
+    int add_outer, add_inner, or_ch_total, or_ch_per_group, or_rows;
+    int generator;       // geo_sc_generator
+    uint32_t seed;       // random generators
     size_t seed_wrap;    // activation seed index is (flat index % seed_wrap)
     int wi, hi;          // padded activation dims 2 / 3
     int wo, ho;          // output dims 2 / 3

@@ -25,6 +25,7 @@
 //     Y : g = v,                      k = ci*w_k + u                       (conv2d_or_bin_1d)
 //     Z : g = ci,                     k = u*h_k + v                        (conv2d_or_bin_z)
 //     YZ: g = (ci / z_unit)*h_k + v,  k = (ci % z_unit)*w_k + u            (conv2d_or_bin_yz)
+//     FULL: g = 0,                    k = (ci*w_k + u)*h_k + v             (conv2d_or_approx, :189-210)
 // Members of a ragged last channel block that do not exist carry zero weights.
 #include "sc_common.h"
 
@@ -255,6 +256,12 @@ __host__ __device__ inline Member member_of(const Groups& G, int g, int k)
         e.u = k / G.h_k;
         e.v = k - e.u * G.h_k;
         e.ok = true;
+    } else if (G.mode == GEO_SC_ACC_FULL) {
+        const int t = k / G.h_k;
+        e.v = k - t * G.h_k;
+        e.ci = t / G.w_k;
+        e.u = t - e.ci * G.w_k;
+        e.ok = true;
     } else if (G.mode == GEO_SC_ACC_YZ) {
         const int blk = g / G.h_k;
         const int cl = k / G.w_k;
@@ -279,6 +286,14 @@ __host__ __device__ inline void next_member(const Groups& G, Member& e)
             e.v = 0;
             ++e.u;
         }
+    } else if (G.mode == GEO_SC_ACC_FULL) {
+        if (++e.v == G.h_k) {
+            e.v = 0;
+            if (++e.u == G.w_k) {
+                e.u = 0;
+                ++e.ci;
+            }
+        }
     } else if (++e.u == G.w_k) {
         e.u = 0;
         ++e.ci;
@@ -291,6 +306,9 @@ __host__ __device__ inline void group_of(const Groups& G, int ci, int u, int v, 
     if (G.mode == GEO_SC_ACC_Z) {
         g = ci;
         k = u * G.h_k + v;
+    } else if (G.mode == GEO_SC_ACC_FULL) {
+        g = 0;
+        k = (ci * G.w_k + u) * G.h_k + v;
     } else if (G.mode == GEO_SC_ACC_YZ) {
         const int blk = ci / G.zu;
         g = blk * G.h_k + v;
@@ -405,7 +423,7 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
                                                      int h_in, int pad_w, int pad_h, int wo, int ho, size_t g_stride)
 {
     const int plane = w_in * h_in;
-    const int k_step = G.mode == GEO_SC_ACC_Z ? G.h_k : 1;
+    const int k_step = (G.mode == GEO_SC_ACC_Z || G.mode == GEO_SC_ACC_FULL) ? G.h_k : 1;
     for (int nc = blockIdx.x; nc < n_planes; nc += gridDim.x) {
         const int n = nc / G.c_in, ci = nc - n * G.c_in;
         float* dst = gx + (size_t)nc * plane;
@@ -474,6 +492,9 @@ BwdLayout bwd_layout(const Geometry& g)
     if (g.mode == GEO_SC_ACC_Z) {
         b.G.n_groups = g.c_in;
         b.G.n_members = g.w_k * g.h_k;
+    } else if (g.mode == GEO_SC_ACC_FULL) {
+        b.G.n_groups = 1;
+        b.G.n_members = g.k_or * g.h_k;
     } else if (g.mode == GEO_SC_ACC_YZ) {
         b.G.n_groups = g.add_outer * g.h_k;
         b.G.n_members = g.z_unit * g.w_k;

@@ -32,6 +32,7 @@ struct FwdParams {
     // per outer group, and the activation strides of an inner add step / an OR channel step
     int add_outer, add_inner, or_ch_total, or_ch_per_group;
     unsigned add_stride, or_stride;
+    int or_rows;  // kernel rows OR-ed together before the popcount (1, or h_k for the full OR)
 };
 
 // acc |= a & w with w wave-uniform: a single v_and_or_b32 whose first source is the SGPR.
@@ -206,7 +207,8 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
 //   Y : outer 1,              inner kernel rows,     OR channels = input channels
 //   YZ: outer channel groups, inner kernel rows,     OR channels = the group's input channels
 //   Z : outer 1,              inner input channels,  OR channels = kernel rows
-// (sc_cuda_kernel.cu:176-349), expressed through the two activation strides in FwdParams; the
+//   FULL: one group per pack; the OR runs over the input channels of or_rows = h_k kernel rows
+// (sc_cuda_kernel.cu:176-349, :1351-1366), expressed through the two activation strides in FwdParams; the
 // weight lines arrive in exactly the order the loop consumes them.
 // Template parameters:
 //   R   rows of accumulators per lane.  ROWS_IN_N == false: R consecutive output rows a
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
     const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
     const unsigned add_stride = ROWS_IN_N ? v_stride : q.add_stride;
     const unsigned or_stride = ROWS_IN_N ? ch_stride : q.or_stride;
-    const size_t lines_per_pack = (size_t)q.add_inner * q.or_ch_total * q.w_k;
+    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
     {
         for (int pv = pv_begin; pv < pv_end; pv++) {
             const int p = pv / groups, g = pv - p * groups;
@@ -285,34 +287,37 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
 #pragma unroll
                 for (int c = 0; c < C; c++) orp[r][c] = orn[r][c] = 0u;
 
-            const uint32_t* ap = act_n + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
+            const uint32_t* ap0 = act_n + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
             const size_t line = p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k + (size_t)gi * chs * q.w_k;
             const uint32_t* wp = q.wgt + (line * q.n_cotile + cot) * (2 * C);
 
-            if constexpr (WK > 0) {
-                int ci = 0;
-                for (; ci + CU <= chs; ci += CU)
-                    or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
-                if constexpr (CU > 1)
-                    for (; ci < chs; ci++)
-                        or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
-            } else {
-                for (int ci = 0; ci < chs; ci++) {
-                    for (int u = 0; u < q.w_k; u++) {
-                        uint32_t wv[2 * C];
+            for (int row = 0; row < q.or_rows; row++) {
+                const uint32_t* ap = ap0 + row;  // next kernel row: one word further (never with ROWS_IN_N)
+                if constexpr (WK > 0) {
+                    int ci = 0;
+                    for (; ci + CU <= chs; ci += CU)
+                        or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
+                    if constexpr (CU > 1)
+                        for (; ci < chs; ci++)
+                            or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
+                } else {
+                    for (int ci = 0; ci < chs; ci++) {
+                        for (int u = 0; u < q.w_k; u++) {
+                            uint32_t wv[2 * C];
 #pragma unroll
-                        for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
-                        int row = a0 + u;
-                        row = row < q.wi ? row : q.wi - 1;
-                        const uint32_t aw = ap[(unsigned)row * q.hi];
+                            for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
+                            int arow = a0 + u;
+                            arow = arow < q.wi ? arow : q.wi - 1;
+                            const uint32_t aw = ap[(unsigned)arow * q.hi];
 #pragma unroll
-                        for (int c = 0; c < C; c++) {
-                            and_or(orp[0][c], aw, wv[c]);
-                            and_or(orn[0][c], aw, wv[C + c]);
+                            for (int c = 0; c < C; c++) {
+                                and_or(orp[0][c], aw, wv[c]);
+                                and_or(orn[0][c], aw, wv[C + c]);
+                            }
+                            wp += k_stride;
                         }
-                        wp += k_stride;
+                        ap += or_stride;
                     }
-                    ap += or_stride;
                 }
             }
             // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
@@ -412,6 +417,7 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     const unsigned ch_plane = (unsigned)g.wi * g.hi;
     q.add_stride = g.mode == GEO_SC_ACC_Z ? ch_plane : 1u;
     q.or_stride = g.mode == GEO_SC_ACC_Z ? 1u : ch_plane;
+    q.or_rows = g.or_rows;
     // Two accumulator rows per lane halve the weight traffic per instruction.  Outputs with
     // several rows take them along dim 2 (sliding-window reuse of activation words); outputs
     // with a single row (the SC-linear mapping, classifier layers) take two batch items.

@@ -34,19 +34,30 @@ at::Tensor conv2d_add_yz_variable_acc(torch::Tensor input, torch::Tensor weight,
     return forward_on_device(input, weight, d);
 }
 
-at::Tensor conv2d_add_partial_acc_acc(torch::Tensor, torch::Tensor, int64_t, at::IntArrayRef, at::IntArrayRef, bool,
-                                      int64_t)
+// sc_cuda.cpp:65-76: y-dimension accumulation with the "accurate random" generator (streams with
+// exactly `code` ones).  The reference seeds its generators with constants (37 for the weights, 0
+// for the activations, sc_cuda_kernel.cu:1885, :1957), so it returns the same result on every call;
+// so does this, with its own counter-based generator: same distribution, other bits.
+at::Tensor conv2d_add_partial_acc_acc(torch::Tensor input, torch::Tensor weight, int64_t bit_length,
+                                      at::IntArrayRef padding, at::IntArrayRef stride, bool share, int64_t dim)
 {
-    TORCH_CHECK(false, "sc_extension_cuda.conv2d_add_partial_acc_acc: the random-number stream generators are not "
-                       "implemented by this library (LFSR generators only)");
-    return at::Tensor();
+    (void)stride;
+    (void)share;  // forced off inside the reference's kernels (sc_cuda_kernel.cu:372, :495)
+    (void)dim;    // unused by the reference (sc_cuda.cpp:75)
+    const geo_sc_conv_desc d = make_desc(input, weight, bit_length, padding, 7, 8, 1, 1, GEO_SC_ACC_Y, 1,
+                                         GEO_SC_GEN_ACC, 37);
+    return forward_on_device(input, weight, d);
 }
 
-at::Tensor conv2d_or_acc(torch::Tensor, torch::Tensor, int64_t, at::IntArrayRef, at::IntArrayRef, bool)
+// sc_cuda.cpp:21-32: OR over the whole kernel window and all input channels, Bernoulli random streams.
+at::Tensor conv2d_or_acc(torch::Tensor input, torch::Tensor weight, int64_t bit_length, at::IntArrayRef padding,
+                         at::IntArrayRef stride, bool im2col)
 {
-    TORCH_CHECK(false, "sc_extension_cuda.conv2d_or_acc: the random-number stream generators are not implemented "
-                       "by this library (LFSR generators only)");
-    return at::Tensor();
+    (void)stride;
+    (void)im2col;  // selects where the reference generates its streams; same distribution either way
+    const geo_sc_conv_desc d = make_desc(input, weight, bit_length, padding, 7, 8, 1, 1, GEO_SC_ACC_FULL, 1,
+                                         GEO_SC_GEN_RAND, 0);
+    return forward_on_device(input, weight, d);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
@@ -55,6 +66,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           "SC forward conv2d partial (y or z dimension) bin add, variable load, lfsr generator");
     m.def("conv2d_add_yz_variable_acc", &conv2d_add_yz_variable_acc,
           "SC forward conv2d partial (yz dimension) bin add, variable load, lfsr generator");
-    m.def("conv2d_add_partial_acc_acc", &conv2d_add_partial_acc_acc, "not implemented: raises");
-    m.def("conv2d_or_acc", &conv2d_or_acc, "not implemented: raises");
+    m.def("conv2d_add_partial_acc_acc", &conv2d_add_partial_acc_acc,
+          "SC forward conv2d partial bin add, accurate random generator");
+    m.def("conv2d_or_acc", &conv2d_or_acc, "SC forward conv2d or add, random generator");
 }

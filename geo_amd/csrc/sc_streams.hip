@@ -253,6 +253,150 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams_grouped(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Random stream generators (the reference's "acc" and "rand" generators, sc_cuda_kernel.cu:354-469,
+// :524-545, :1319-1333, which draw from cuRAND per-thread states).  Here every element owns a
+// counter-based Philox4x32-10 sequence: counter (block, index_lo, index_hi, tag), key (seed, 0);
+// word j of the element is output j % 4 of block j / 4.  Results do not depend on the launch shape.
+//   GEO_SC_GEN_RAND: bit t = [code > field (t % cpw) of word t / cpw], n_bits-wide fields from the
+//                    least significant end, cpw = 32 / n_bits: independent Bernoulli(code / L) bits
+//   GEO_SC_GEN_ACC : bit t = [r16 * left_total < left_ones * 65536] with the 16-bit halves of word
+//                    t / 2; left_ones -= bit, left_total -= 1: exactly `code` ones
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                              uint32_t k1, uint32_t (&out)[4])
+{
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        const uint32_t h0 = __umulhi(0xD2511F53u, c0), l0 = 0xD2511F53u * c0;
+        const uint32_t h1 = __umulhi(0xCD9E8D57u, c2), l1 = 0xCD9E8D57u * c2;
+        const uint32_t n0 = h1 ^ c1 ^ k0, n2 = h0 ^ c3 ^ k1;
+        c0 = n0;
+        c1 = l1;
+        c2 = n2;
+        c3 = l0;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0;
+    out[1] = c1;
+    out[2] = c2;
+    out[3] = c3;
+}
+
+struct RandParams {
+    int L, n_bits, packs, bit_unit;
+    int generator;  // GEO_SC_GEN_ACC or GEO_SC_GEN_RAND
+    uint32_t seed;
+};
+
+// The P stream words of one element, handed to put(pack, word).
+template <typename Put>
+__device__ __forceinline__ void random_stream(const RandParams& rp, int code, uint32_t tag, uint64_t index, Put put)
+{
+    uint32_t r[4] = {0, 0, 0, 0};
+    int have_block = -1;
+    const int cpw = rp.generator == GEO_SC_GEN_RAND ? 32 / rp.n_bits : 2;
+    int left_ones = code, left_total = rp.L;
+    for (int p = 0; p < rp.packs; p++) {
+        uint32_t word = 0;
+        if (code != 0) {
+            for (int b = 0; b < rp.bit_unit; b++) {
+                const int t = p * rp.bit_unit + b;
+                const int j = t / cpw, f = t - j * cpw;
+                if ((j >> 2) != have_block) {
+                    have_block = j >> 2;
+                    philox4x32_10((uint32_t)have_block, (uint32_t)index, (uint32_t)(index >> 32), tag, rp.seed, 0u, r);
+                }
+                const uint32_t rw = (j & 3) == 0 ? r[0] : (j & 3) == 1 ? r[1] : (j & 3) == 2 ? r[2] : r[3];
+                uint32_t bit;
+                if (rp.generator == GEO_SC_GEN_RAND) {
+                    bit = (uint32_t)code > ((rw >> (f * rp.n_bits)) & (uint32_t)(rp.L - 1));
+                } else {
+                    const uint32_t r16 = (rw >> (16 * f)) & 0xffffu;
+                    bit = r16 * (uint32_t)left_total < (uint32_t)left_ones * 65536u;
+                    left_ones -= (int)bit;
+                    left_total -= 1;
+                }
+                word = word * 2u + bit;
+            }
+        }
+        put(p, word);
+    }
+}
+
+// Activation streams [n][P][c_in][Wi][Hi] of the random generators; element index = flat index in
+// the padded tensor (n, c_in, Wi, Hi).  Padding positions give zero words.
+__global__ __launch_bounds__(kGenThreads) void k_act_streams_random(const float* __restrict__ x,
+                                                                   uint32_t* __restrict__ streams, RandParams rp, int n,
+                                                                   int c_in, int w_in, int h_in, int pad_w, int pad_h)
+{
+    const int wi = w_in + 2 * pad_w, hi = h_in + 2 * pad_h;
+    const uint32_t plane = (uint32_t)c_in * wi * hi;
+    const size_t total = (size_t)n * plane;
+    const float Lf = (float)rp.L, top = (float)(rp.L - 1);
+    for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
+        const uint32_t item = (uint32_t)(e / plane);
+        const uint32_t i = (uint32_t)(e - (size_t)item * plane);
+        const uint32_t q = i % (uint32_t)hi;
+        const uint32_t r = i / (uint32_t)hi;
+        const uint32_t p = r % (uint32_t)wi;
+        const uint32_t c = r / (uint32_t)wi;
+        const int ps = (int)p - pad_w, qs = (int)q - pad_h;
+        int code = 0;
+        if (ps >= 0 && ps < w_in && qs >= 0 && qs < h_in) {
+            const float v = x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs];
+            code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
+        }
+        uint32_t* dst = streams + (size_t)item * rp.packs * plane + i;
+        random_stream(rp, code, 0u, (uint64_t)e, [&](int pk, uint32_t word) { dst[(size_t)pk * plane] = word; });
+    }
+}
+
+// Weight streams of the random generators in the tiled layout [P][h_k][k][cotile][rail][16];
+// every weight element (also across c_out) has its own sequence; element index = flat index in
+// (c_out, c_in, w_k, h_k), tag 1 for the positive rail and 2 for the negative rail.
+__global__ __launch_bounds__(kGenThreads) void k_weight_streams_random(const float* __restrict__ w,
+                                                                      uint32_t* __restrict__ streams, RandParams rp,
+                                                                      int c_out, int c_in, int w_k, int h_k,
+                                                                      int n_cotile)
+{
+    const int k_or = c_in * w_k;
+    const int co_pad = n_cotile * kCoTile;
+    const size_t total = (size_t)h_k * k_or * co_pad;
+    const size_t pack_stride = (size_t)h_k * k_or * n_cotile * 2 * kCoTile;
+    const float Lf = (float)rp.L, top = (float)(rp.L - 1);
+    for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
+        const int co = (int)(e % co_pad);
+        const size_t r = e / co_pad;
+        const int k = (int)(r % k_or);
+        const int v = (int)(r / k_or);
+        const int ci = k / w_k, u = k % w_k;
+        int cp = 0, cn = 0;
+        uint64_t widx = 0;
+        if (co < c_out) {
+            widx = (((uint64_t)co * c_in + ci) * w_k + u) * h_k + v;
+            const float t = w[widx] * Lf;
+            cp = (int)ceilf(fminf(fmaxf(t, 0.0f), top));
+            cn = (int)ceilf(-fminf(fmaxf(t, -top), 0.0f));
+        }
+        uint32_t* dst = streams + (((size_t)v * k_or + k) * n_cotile + co / kCoTile) * (2 * kCoTile) + (co % kCoTile);
+        random_stream(rp, cp, 1u, widx, [&](int pk, uint32_t word) { dst[pk * pack_stride] = word; });
+        random_stream(rp, cn, 2u, widx, [&](int pk, uint32_t word) { dst[pk * pack_stride + kCoTile] = word; });
+    }
+}
+
+RandParams rand_params(const Geometry& g)
+{
+    RandParams rp;
+    rp.L = g.L;
+    rp.n_bits = g.n_bits;
+    rp.packs = g.packs;
+    rp.bit_unit = g.bit_unit;
+    rp.generator = g.generator;
+    rp.seed = g.seed;
+    return rp;
+}
+
 GenParams gen_params(const Geometry& g, int load_wait)
 {
     GenParams gp;
@@ -293,6 +437,13 @@ template <typename XT>
 static int launch_act_streams_t(const Geometry& g, const XT* x, uint32_t* streams, const uint32_t* tables,
                                 hipStream_t s)
 {
+    if (g.generator != GEO_SC_GEN_LFSR) {
+        if (sizeof(XT) != sizeof(float)) return GEO_SC_ERR_UNSUPPORTED;  // fp32 activations only
+        const size_t n_el = (size_t)g.n * g.act_plane;
+        hipLaunchKernelGGL(k_act_streams_random, dim3(grid_for(n_el)), dim3(kGenThreads), 0, s, (const float*)x,
+                           streams, rand_params(g), g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
     const GenParams gp = gen_params(g, g.load_wait_a);
     const size_t total = (size_t)g.n * g.act_plane;
     const uint32_t wrap = (uint32_t)g.seed_wrap;
@@ -319,8 +470,14 @@ int launch_act_streams_q7(const Geometry& g, const uint8_t* x, uint32_t* streams
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s)
 {
+    if (g.generator != GEO_SC_GEN_LFSR) {
+        const size_t n_el = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
+        hipLaunchKernelGGL(k_weight_streams_random, dim3(grid_for(n_el)), dim3(kGenThreads), 0, s, w, streams,
+                           rand_params(g), g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
     const GenParams gp = gen_params(g, g.load_wait_w);
-    if (g.mode != GEO_SC_ACC_Y) {
+    if (g.mode != GEO_SC_ACC_Y && g.mode != GEO_SC_ACC_FULL) {
         const size_t padded =
             (size_t)g.add_outer * g.add_inner * g.or_ch_per_group * g.w_k * g.n_cotile * kCoTile;
         hipLaunchKernelGGL(k_weight_streams_grouped, dim3(grid_for(padded)), dim3(kGenThreads), table_bytes(g.L), s,

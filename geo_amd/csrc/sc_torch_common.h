@@ -21,7 +21,7 @@ inline void check_status(int rc, const char* what)
 inline geo_sc_conv_desc make_desc(const at::Tensor& input, const at::Tensor& weight, int64_t bit_length,
                                   at::IntArrayRef padding, int64_t total_width, int64_t load_width,
                                   int64_t load_wait_w, int64_t load_wait_a, int accumulate = GEO_SC_ACC_Y,
-                                  int64_t z_unit = 1)
+                                  int64_t z_unit = 1, int generator = GEO_SC_GEN_LFSR, int32_t seed = 0)
 {
     TORCH_CHECK(input.dim() == 4, "input must be (N, C_in, W, H), got ", input.dim(), " dims");
     TORCH_CHECK(weight.dim() == 4, "weight must be (C_out, C_in, W, H), got ", weight.dim(), " dims");
@@ -53,6 +53,8 @@ inline geo_sc_conv_desc make_desc(const at::Tensor& input, const at::Tensor& wei
     TORCH_CHECK(z_unit >= 1, "z_units must be >= 1, got ", z_unit);
     d.accumulate = (int32_t)accumulate;
     d.z_unit = (int32_t)(z_unit > input.size(1) ? input.size(1) : z_unit);
+    d.generator = (int32_t)generator;
+    d.seed = seed;
     return d;
 }
 

@@ -54,6 +54,11 @@ def conv2d_or_bin_1d(activation, w_pos, w_neg, padding, stride):
     return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
 
 
+def conv2d_or_approx(activation, weight, padding, stride):
+    """Surrogate of full OR accumulation (utils_functional.py:189-210, its default branch)."""
+    return 1 - torch.exp(-F.conv2d(activation, weight, padding=padding, stride=stride))
+
+
 def conv2d_or_bin_z(activation, w_pos, w_neg, padding, stride):
     """Surrogate of z-dimension accumulation (utils_functional.py:254-270): one single-channel
     convolution per input channel and rail, 1 - exp(-z), summed over channels."""
@@ -86,7 +91,7 @@ class _SCConv2dAddPartial(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, activation, weight, bit_length, padding, load_unit, load_wait, accumulate="y", z_unit=1,
-                load_wait_a=None):
+                load_wait_a=None, generator="lfsr", seed=0):
         origin = activation.device
         dev = origin if activation.is_cuda else torch.device("cuda", torch.cuda.current_device())
         x = activation.detach().to(dev, torch.float32).contiguous()
@@ -103,8 +108,10 @@ class _SCConv2dAddPartial(torch.autograd.Function):
             # loading (utils_functional.py:493)
             loading = dict(capi.NEUTRAL_LOADING)
         z_unit = max(1, min(int(z_unit), x.shape[1]))
+        if generator != "lfsr":
+            loading = dict(capi.NEUTRAL_LOADING)  # the random generators have no progressive loading
         counts = capi.conv2d_add_partial_forward(x, w, int(bit_length), pad, accumulate=accumulate, z_unit=z_unit,
-                                                 **loading)
+                                                 generator=generator, seed=seed, **loading)
         ctx.save_for_backward(x, w)
         ctx.accumulate = accumulate
         ctx.z_unit = z_unit
@@ -129,7 +136,7 @@ class _SCConv2dAddPartial(torch.autograd.Function):
             gx = gx.to(ctx.origin, ctx.act_dtype)
         if gw is not None:
             gw = gw.to(ctx.w_device, ctx.w_dtype)
-        return gx, gw, None, None, None, None, None, None, None
+        return gx, gw, None, None, None, None, None, None, None, None, None
 
 
 def conv2d_generic(activation, weight, padding, stride, **kwargs):
@@ -137,10 +144,11 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
 
     Keyword arguments read: bit_length (128), generator (None), forward ('full_or'), legacy
     (False), load_unit (8), load_wait_w (1), load_wait_a (1), z_unit (1024); prec/acc/share are
-    accepted and unused on these paths.  Implemented: forward='1d_bin' with generator='lfsr', and
-    forward='z_bin' / 'yz_bin' on GPU tensors (the reference sends those to its LFSR GPU ops
-    whatever the generator, utils_functional.py:503-510), all with legacy=False; anything else
-    raises NotImplementedError.
+    accepted and unused on these paths.  Implemented: forward='1d_bin' with generator='lfsr' or,
+    on GPU tensors, 'acc'; forward='z_bin' / 'yz_bin' on GPU tensors (the reference sends those to
+    its LFSR GPU ops whatever the generator, utils_functional.py:503-510); forward='full_or' on GPU
+    tensors (random Bernoulli streams, :511-514); all with legacy=False; anything else raises
+    NotImplementedError.
     """
     bit_length = kwargs.get("bit_length", 128)
     generator = kwargs.get("generator", None)
@@ -150,19 +158,27 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     load_wait_w = kwargs.get("load_wait_w", 1)
     load_wait_a = kwargs.get("load_wait_a", 1)
     z_unit = kwargs.get("z_unit", 1024)
-    ok_1d = forward == "1d_bin" and generator == "lfsr"
-    ok_zyz = forward in ("z_bin", "yz_bin") and activation.is_cuda
+    ok_1d = forward == "1d_bin" and (generator == "lfsr" or (generator == "acc" and activation.is_cuda))
+    ok_zyz = forward in ("z_bin", "yz_bin", "full_or") and activation.is_cuda
     if legacy or not (ok_1d or ok_zyz):
         raise NotImplementedError(
             f"conv2d_generic(forward={forward!r}, generator={generator!r}, legacy={legacy}, "
             f"cuda={activation.is_cuda}): this build implements forward='1d_bin' with generator='lfsr' and "
-            "forward='z_bin'/'yz_bin' on GPU tensors, legacy=False")
+            "(on GPU tensors also 'acc'), and forward='z_bin'/'yz_bin'/'full_or' on GPU tensors, legacy=False")
     if isinstance(stride, int):
         stride = (stride, stride)
     if tuple(stride) != (1, 1):
         raise NotImplementedError("the SC kernels compute stride 1 only (the reference's native code ignores stride)")
     if isinstance(padding, int):
         padding = (padding, padding)
+    if forward == "full_or":
+        # sc_extension_cuda.conv2d_or_acc: Bernoulli random streams, OR over everything
+        # (utils_functional.py:511-514); surrogate conv2d_or_approx (:616-617)
+        return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), 8, 1, "full", 1, None, "rand",
+                                         0)
+    if forward == "1d_bin" and generator == "acc":
+        # sc_extension_cuda.conv2d_add_partial_acc_acc (utils_functional.py:499-502)
+        return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), 8, 1, "y", 1, None, "acc", 37)
     if forward == "z_bin":
         return _SCConv2dAddPartial.apply(activation, weight, bit_length, tuple(padding), load_unit, load_wait_w, "z")
     if forward == "yz_bin":

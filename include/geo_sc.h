@@ -44,21 +44,38 @@ enum geo_sc_status {
 };
 
 /*
- * Partial binary accumulation modes of the reference's LFSR ops.  Products of one OR group
- * are OR-ed, groups (and stream packs) are added with binary adders.
- *   GEO_SC_ACC_Y   OR over (c_in, w_k), add over h_k: conv2d_add_partial_new (sc.cpp:292) and
- *                  conv2d_add_partial_variable_acc with dim != 0 (sc_cuda.cpp:47-63)
- *   GEO_SC_ACC_Z   OR over (w_k, h_k), add over c_in: conv2d_add_partial_variable_acc with
- *                  dim == 0 (sc_cuda.cpp:57-59, sc_cuda_kernel.cu:2119-2285)
- *   GEO_SC_ACC_YZ  OR over (z_unit consecutive input channels, w_k), add over h_k and over the
- *                  ceil(c_in / z_unit) channel groups: conv2d_add_yz_variable_acc
- *                  (sc_cuda.cpp:34-45, sc_cuda_kernel.cu:1971-2116)
- * Seeds.  Weights use (67+s) % (L-1) + 1 / (37+s) % (L-1) + 1 with s = c_in_index*w_k + w_index
- * (Y), w_index*h_k + h_index (Z, sc_cuda_kernel.cu:322-324) or (c_in_index % z_unit)*w_k +
- * w_index (YZ, :232).  Activations use i % (L-1) + 1 with i the flat index in the padded item
- * (Y, Z) or that index taken inside the channel group, i % (z_unit*Wi*Hi) (YZ, :1080).
+ * Accumulation modes.  Products of one OR group are OR-ed, groups (and stream packs) are added
+ * with binary adders.
+ *   GEO_SC_ACC_Y    OR over (c_in, w_k), add over h_k: conv2d_add_partial_new (sc.cpp:292) and
+ *                   conv2d_add_partial_variable_acc with dim != 0 (sc_cuda.cpp:47-63)
+ *   GEO_SC_ACC_Z    OR over (w_k, h_k), add over c_in: conv2d_add_partial_variable_acc with
+ *                   dim == 0 (sc_cuda.cpp:57-59, sc_cuda_kernel.cu:2119-2285)
+ *   GEO_SC_ACC_YZ   OR over (z_unit consecutive input channels, w_k), add over h_k and over the
+ *                   ceil(c_in / z_unit) channel groups: conv2d_add_yz_variable_acc
+ *                   (sc_cuda.cpp:34-45, sc_cuda_kernel.cu:1971-2116)
+ *   GEO_SC_ACC_FULL OR over (c_in, w_k, h_k), add over packs only: conv2d_or_acc (sc_cuda.cpp:21-32,
+ *                   sc_cuda_kernel.cu:1274-1366)
+ * LFSR seeds.  Weights use (67+s) % (L-1) + 1 / (37+s) % (L-1) + 1 with s = c_in_index*w_k +
+ * w_index (Y, FULL), w_index*h_k + h_index (Z, sc_cuda_kernel.cu:322-324) or (c_in_index %
+ * z_unit)*w_k + w_index (YZ, :232).  Activations use i % (L-1) + 1 with i the flat index in the
+ * padded item (Y, Z, FULL) or that index taken inside the channel group, i % (z_unit*Wi*Hi)
+ * (YZ, :1080).
  */
-enum geo_sc_accumulate { GEO_SC_ACC_Y = 0, GEO_SC_ACC_Z = 1, GEO_SC_ACC_YZ = 2 };
+enum geo_sc_accumulate { GEO_SC_ACC_Y = 0, GEO_SC_ACC_Z = 1, GEO_SC_ACC_YZ = 2, GEO_SC_ACC_FULL = 3 };
+
+/*
+ * Stream generators.  GEO_SC_GEN_LFSR: the deterministic LFSR / comparator streams.
+ * GEO_SC_GEN_ACC ("accurate random", conv2d_add_partial_acc_acc, sc_cuda_kernel.cu:354-420,
+ * :524-545): every activation and weight element gets a stream with exactly `code` ones at
+ * uniformly random positions.  GEO_SC_GEN_RAND (conv2d_or_acc, :422-469, :1319-1333): independent
+ * Bernoulli(code / L) bits.  The reference draws from cuRAND XORWOW states owned by threads, so
+ * its bit sequences depend on its launch shape; here every element owns a counter-based
+ * Philox4x32-10 sequence (counter: block, element index, tag 0 activation / 1 positive / 2
+ * negative weight rail; key: geo_sc_conv_desc.seed): same distributions, reproducible, not
+ * bit-identical to the reference.  No progressive loading; with GEO_SC_ACC_Y or _FULL only, fp32
+ * activations only.
+ */
+enum geo_sc_generator { GEO_SC_GEN_LFSR = 0, GEO_SC_GEN_ACC = 1, GEO_SC_GEN_RAND = 2 };
 
 /*
  * Problem description shared by all entry points.
@@ -86,6 +103,8 @@ typedef struct geo_sc_conv_desc {
     int32_t load_wait_a;  /* load_wait of the activation generator */
     int32_t accumulate;   /* enum geo_sc_accumulate: which products are OR-ed and which are added */
     int32_t z_unit;       /* GEO_SC_ACC_YZ: input channels per OR group (clamped to c_in); else unused */
+    int32_t generator;    /* enum geo_sc_generator */
+    int32_t seed;         /* key of the random generators (its 32 bits); unused with GEO_SC_GEN_LFSR */
 } geo_sc_conv_desc;
 
 /* Library version (GEO_SC_VERSION of the build). */

@@ -38,6 +38,20 @@
  *                        executable z-mode code outside its CUDA kernels
  *                        (sc_cuda_kernel.cu:270-349); an independent per-bit
  *                        formulation of the same reading agrees.
+ *   sco_philox4x32_10    pinned  - the three known-answer vectors of the
+ *                                  published Philox4x32-10 (Salmon et al., SC'11;
+ *                                  Random123 kat_vectors)
+ *   random generators (sco_random_stream_words, generator 1 "acc", 2 "rand")
+ *                        STATISTICAL PARITY ONLY: the reference draws from
+ *                        cuRAND's XORWOW with per-thread states
+ *                        (sc_cuda_kernel.cu:354-420, :422-469, :524-545,
+ *                        :1319-1333); its bit sequences are a property of that
+ *                        library and its launch shape.  What is restated is the
+ *                        distribution: "acc" = exactly `code` ones per stream,
+ *                        drawn without replacement; "rand" = independent
+ *                        Bernoulli(code / L) bits.  Pinned by the exact-count
+ *                        invariant, by bit frequencies and by the closed-form
+ *                        expectation of the layer output.
  *
  * Conventions (same names as the reference): weight (Cout, Cin, W, H) with
  * W = dim 2 and H = dim 3 (the binary-add dimension); padded activation
@@ -401,12 +415,95 @@ int sco_max_threads(void)
  * for yz the index wraps at z_unit*Wi*Hi (:1080), i.e. it is taken inside the channel group.
  * z_unit is clamped to c_in (:1987).
  * ------------------------------------------------------------------------------------------ */
+/* Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+ * SC'11): ten rounds of two 32x32->64 multiplies, key bumped by the Weyl constants. */
+void sco_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4])
+{
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; r++) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* Random stream of one value: the P words of an L-bit stream, MSB-first like the LFSR streams.
+ * The element's random words are Philox outputs with counter (block, index_lo, index_hi, tag)
+ * and key (seed_lo, seed_hi); word j of the element is output j%4 of block j/4.
+ *   generator 2 "rand": bit t = [code > r], r the (t % cpw)-th n_bits-wide field (from the least
+ *     significant end) of word t / cpw, cpw = 32 / n_bits: independent Bernoulli(code / L) bits,
+ *     the distribution of code > curand() % L (sc_cuda_kernel.cu:459-462, :1329-1330).
+ *   generator 1 "acc": bit t = [r16 * left_total < left_ones * 65536], r16 the (t % 2)-th 16-bit
+ *     half of word t / 2, then left_ones -= bit, left_total -= 1: sampling without replacement,
+ *     exactly `code` ones, the distribution of the reference's code_left / total_left >
+ *     curand_uniform() (sc_cuda_kernel.cu:399-411, :539-545).
+ * tag: 0 activations, 1 positive-rail weights, 2 negative-rail weights. */
+void sco_random_stream_words(int code, int L, int generator, uint32_t tag, uint64_t index, uint64_t seed,
+                             uint32_t* words /* [P] */)
+{
+    int n_bits = sco_nbits_for_length(L);
+    int P = (L + 31) / 32, bit_unit = L < 32 ? L : 32;
+    uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t ctr[4] = {0, (uint32_t)index, (uint32_t)(index >> 32), tag};
+    uint32_t r[4] = {0, 0, 0, 0};
+    int have_block = -1;
+    int cpw = generator == 2 ? 32 / n_bits : 2;
+    int left_ones = code, left_total = L;
+    for (int p = 0; p < P; p++) {
+        uint32_t word = 0;
+        for (int b = 0; b < bit_unit; b++) {
+            int t = p * bit_unit + b;
+            int j = t / cpw, f = t % cpw;
+            if (j / 4 != have_block) {
+                have_block = j / 4;
+                ctr[0] = (uint32_t)have_block;
+                sco_philox4x32_10(ctr, key, r);
+            }
+            uint32_t rw = r[j % 4];
+            uint32_t bit;
+            if (generator == 2) {
+                bit = (uint32_t)code > ((rw >> (f * n_bits)) & (uint32_t)(L - 1));
+            } else {
+                uint32_t r16 = (rw >> (16 * f)) & 0xffffu;
+                bit = r16 * (uint32_t)left_total < (uint32_t)left_ones * 65536u;
+                left_ones -= (int)bit;
+                left_total -= 1;
+            }
+            word = word * 2u + bit;
+        }
+        words[p] = word;
+    }
+}
+
+/* generator: 0 LFSR (the seeds and loading arguments above), 1 "acc", 2 "rand" (random streams of
+ * sco_random_stream_words; element index = flat index in the padded activation tensor
+ * (N, Cin, Wi, Hi) resp. in the weight tensor (Cout, Cin, W, H); no progressive loading).
+ * mode 3: OR over the whole kernel window and all input channels, add over packs only
+ * (conv2d_or_acc: matmul_outer with inner_size = Cin*W*H and pws = packs, sc_cuda_kernel.cu:1351-1366). */
+int sco_conv2d_general(const float* x, const float* w, int32_t* y, int N, int Cin, int Wx, int Hx, int Cout, int W,
+                       int H, int pad_w, int pad_h, int L, int total_width, int load_width, int load_wait_w,
+                       int load_wait_a, int mode, int z_unit, int generator, uint64_t seed);
+
 int sco_conv2d_modes(const float* x, const float* w, int32_t* y, int N, int Cin, int Wx, int Hx, int Cout, int W,
                      int H, int pad_w, int pad_h, int L, int total_width, int load_width, int load_wait_w,
                      int load_wait_a, int mode, int z_unit)
 {
+    if (mode > 2) return -1;
+    return sco_conv2d_general(x, w, y, N, Cin, Wx, Hx, Cout, W, H, pad_w, pad_h, L, total_width, load_width,
+                              load_wait_w, load_wait_a, mode, z_unit, 0, 0);
+}
+
+int sco_conv2d_general(const float* x, const float* w, int32_t* y, int N, int Cin, int Wx, int Hx, int Cout, int W,
+                       int H, int pad_w, int pad_h, int L, int total_width, int load_width, int load_wait_w,
+                       int load_wait_a, int mode, int z_unit, int generator, uint64_t seed)
+{
     int n_bits = sco_nbits_for_length(L);
-    if (n_bits < 0 || load_width < 1 || load_wait_w < 1 || load_wait_a < 1 || mode < 0 || mode > 2) return -1;
+    if (n_bits < 0 || load_width < 1 || load_wait_w < 1 || load_wait_a < 1 || mode < 0 || mode > 3) return -1;
+    if (generator < 0 || generator > 2) return -1;
     if (mode == 2 && z_unit < 1) return -1;
     int Wi = Wx + 2 * pad_w, Hi = Hx + 2 * pad_h;
     int Wo = Wi - W + 1, Ho = Hi - H + 1;
@@ -423,7 +520,12 @@ int sco_conv2d_modes(const float* x, const float* w, int32_t* y, int N, int Cin,
             for (int u = 0; u < W; u++)
                 for (int v = 0; v < H; v++) {
                     size_t e = (((size_t)co * Cin + ci) * W + u) * H + v;
-                    int s = mode == 0 ? ci * W + u : (mode == 1 ? u * H + v : (ci % zu) * W + u);
+                    int s = (mode == 0 || mode == 3) ? ci * W + u : (mode == 1 ? u * H + v : (ci % zu) * W + u);
+                    if (generator != 0) {
+                        sco_random_stream_words(sco_code_wpos(w[e], L), L, generator, 1, e, seed, wp + e * P);
+                        sco_random_stream_words(sco_code_wneg(w[e], L), L, generator, 2, e, seed, wn + e * P);
+                        continue;
+                    }
                     sco_stream_words(sco_code_wpos(w[e], L), (67 + s) % (L - 1) + 1, L, n_bits, total_width,
                                      load_width, load_wait_w, wp + e * P);
                     sco_stream_words(sco_code_wneg(w[e], L), (37 + s) % (L - 1) + 1, L, n_bits, total_width,
@@ -435,23 +537,28 @@ int sco_conv2d_modes(const float* x, const float* w, int32_t* y, int N, int Cin,
     uint32_t* A = (uint32_t*)malloc(sizeof(uint32_t) * plane * P); /* [i][p] */
     for (int n = 0; n < N; n++) {
         sco_pad_item(x + (size_t)n * Cin * Wx * Hx, Cin, Wx, Hx, pad_w, pad_h, xp);
-        for (size_t i = 0; i < plane; i++)
-            sco_stream_words(sco_code_act(xp[i], L), (int)((i % wrap) % (size_t)(L - 1)) + 1, L, n_bits, total_width,
-                             load_width, load_wait_a, A + i * P);
+        for (size_t i = 0; i < plane; i++) {
+            if (generator != 0)
+                sco_random_stream_words(sco_code_act(xp[i], L), L, generator, 0, (uint64_t)n * plane + i, seed,
+                                        A + i * P);
+            else
+                sco_stream_words(sco_code_act(xp[i], L), (int)((i % wrap) % (size_t)(L - 1)) + 1, L, n_bits,
+                                 total_width, load_width, load_wait_a, A + i * P);
+        }
         for (int co = 0; co < Cout; co++)
             for (int a = 0; a < Wo; a++)
                 for (int b = 0; b < Ho; b++) {
                     int32_t acc = 0;
                     /* add-groups: y: v; z: ci; yz: (channel group, v) */
-                    int g_outer = mode == 1 ? Cin : zp_n;
-                    int g_inner = mode == 1 ? 1 : H;
+                    int g_outer = mode == 1 ? Cin : (mode == 3 ? 1 : zp_n);
+                    int g_inner = (mode == 1 || mode == 3) ? 1 : H;
                     for (int go = 0; go < g_outer; go++)
                         for (int gi = 0; gi < g_inner; gi++)
                             for (int p = 0; p < P; p++) {
                                 uint32_t orp = 0, orn = 0;
                                 int c0 = mode == 1 ? go : go * zu;
                                 int c1 = mode == 1 ? go + 1 : (c0 + zu < Cin ? c0 + zu : Cin);
-                                int v0 = mode == 1 ? 0 : gi, v1 = mode == 1 ? H : gi + 1;
+                                int v0 = (mode == 1 || mode == 3) ? 0 : gi, v1 = (mode == 1 || mode == 3) ? H : gi + 1;
                                 for (int ci = c0; ci < c1; ci++)
                                     for (int u = 0; u < W; u++)
                                         for (int v = v0; v < v1; v++) {

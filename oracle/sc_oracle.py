@@ -52,6 +52,12 @@ def lib():
     L.sco_conv2d_add_partial.restype = i
     L.sco_conv2d_modes.argtypes = [fp, fp, ip] + [i] * 16
     L.sco_conv2d_modes.restype = i
+    L.sco_conv2d_general.argtypes = [fp, fp, ip] + [i] * 17 + [ctypes.c_uint64]
+    L.sco_conv2d_general.restype = i
+    L.sco_philox4x32_10.argtypes = [up, up, up]
+    L.sco_philox4x32_10.restype = None
+    L.sco_random_stream_words.argtypes = [i, i, i, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_uint64, up]
+    L.sco_random_stream_words.restype = None
     L.sco_max_threads.argtypes = []
     L.sco_max_threads.restype = i
     _lib = L
@@ -163,6 +169,45 @@ def conv2d_modes(x, w, L: int, padding=(0, 0), mode="y", z_unit=1, total_width=7
     rc = lib().sco_conv2d_modes(_ptr(x, ctypes.c_float), _ptr(w, ctypes.c_float), _ptr(y, ctypes.c_int32), N, Cin, Wx,
                                 Hx, Cout, W, H, pad_w, pad_h, L, total_width, load_width, load_wait_w, load_wait_a,
                                 MODES[mode], int(z_unit))
+    if rc != 0:
+        raise ValueError("unsupported stream length or bad arguments")
+    return y
+
+
+GENERATORS = {"lfsr": 0, "acc": 1, "rand": 2}
+MODES_ALL = {"y": 0, "z": 1, "yz": 2, "full": 3}
+
+
+def philox4x32_10(ctr, key):
+    c = np.asarray(ctr, dtype=np.uint32)
+    k = np.asarray(key, dtype=np.uint32)
+    out = np.zeros(4, dtype=np.uint32)
+    lib().sco_philox4x32_10(_ptr(c, ctypes.c_uint32), _ptr(k, ctypes.c_uint32), _ptr(out, ctypes.c_uint32))
+    return out
+
+
+def random_stream(code: int, L: int, generator: str, tag: int, index: int, seed: int):
+    """words[P] uint32 of one value's random stream (generator "acc" or "rand")."""
+    words = np.zeros((L + 31) // 32, dtype=np.uint32)
+    lib().sco_random_stream_words(int(code), L, GENERATORS[generator], tag, index, seed, _ptr(words, ctypes.c_uint32))
+    return words
+
+
+def conv2d_general(x, w, L: int, padding=(0, 0), mode="y", z_unit=1, generator="lfsr", seed=0, total_width=7,
+                   load_width=8, load_wait_w=1, load_wait_a=1):
+    """int32 (N,Cout,Wo,Ho) for any accumulation mode ("y" | "z" | "yz" | "full") and generator
+    ("lfsr" | "acc" | "rand"); scalar loops, small shapes."""
+    x = _f32(x)
+    w = _f32(w)
+    N, Cin, Wx, Hx = x.shape
+    Cout, _, W, H = w.shape
+    pad_h, pad_w = int(padding[0]), int(padding[1])
+    Wo = Wx + 2 * pad_w - W + 1
+    Ho = Hx + 2 * pad_h - H + 1
+    y = np.zeros((N, Cout, max(Wo, 0), max(Ho, 0)), dtype=np.int32)
+    rc = lib().sco_conv2d_general(_ptr(x, ctypes.c_float), _ptr(w, ctypes.c_float), _ptr(y, ctypes.c_int32), N, Cin,
+                                  Wx, Hx, Cout, W, H, pad_w, pad_h, L, total_width, load_width, load_wait_w,
+                                  load_wait_a, MODES_ALL[mode], int(z_unit), GENERATORS[generator], int(seed))
     if rc != 0:
         raise ValueError("unsupported stream length or bad arguments")
     return y

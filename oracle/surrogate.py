@@ -24,7 +24,9 @@ def _groups(act, w_pos, w_neg, mode, z_unit):
     slices them: conv2d_or_bin_1d (utils_functional.py:235-252), conv2d_or_bin_z (:254-270),
     conv2d_or_bin_yz (:272-299)."""
     c_in, i_y, f_y = act.size(1), act.size(3), w_pos.size(3)
-    if mode == "z":
+    if mode == "full":  # conv2d_or_approx (utils_functional.py:189-210): one group, everything OR-ed
+        yield act, w_pos, w_neg
+    elif mode == "z":
         for c in range(c_in):
             yield act[:, c:c + 1].clone(), w_pos[:, c:c + 1].clone(), w_neg[:, c:c + 1].clone()
     elif mode == "yz":
@@ -85,6 +87,8 @@ def surrogate_closed_form_modes(x, w, grad_out, padding=(0, 0), mode="y", z_unit
         groups = [[(c, u, v) for c in range(Cin) for u in range(W)] for v in range(H)]
     elif mode == "z":
         groups = [[(c, u, v) for u in range(W) for v in range(H)] for c in range(Cin)]
+    elif mode == "full":
+        groups = [[(c, u, v) for c in range(Cin) for u in range(W) for v in range(H)]]
     else:
         groups = [[(c, u, v) for c in range(c0, min(c0 + z_unit, Cin)) for u in range(W)]
                   for c0 in range(0, Cin, z_unit) for v in range(H)]
