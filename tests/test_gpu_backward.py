@@ -107,7 +107,9 @@ def test_autograd_binding_matches_reference_composition(capi):
     yc.backward(g)
     assert rel_err(xc.grad, rx) <= RTOL and rel_err(wc.grad, rw) <= RTOL
     with pytest.raises(NotImplementedError):
-        uf.conv2d_generic(xg, wg, (1, 1), (1, 1), bit_length=64, forward="full_or", generator="lfsr")
+        uf.conv2d_generic(xg, wg, (1, 1), (1, 1), bit_length=64, forward="2d_bin", generator="lfsr")
+    with pytest.raises(NotImplementedError):
+        uf.conv2d_generic(xg, wg, (1, 1), (1, 1), bit_length=64, forward="1d_bin", generator="lfsr", legacy=True)
     with pytest.raises(NotImplementedError):
         uf.conv2d_generic(xg, wg, (1, 1), (2, 2), bit_length=64, forward="1d_bin", generator="lfsr")
 

@@ -238,7 +238,7 @@ def test_torch_modules_with_reference_names(capi, so, fixtures_small):
     with pytest.raises(RuntimeError):
         sc_cuda.conv2d_add_partial_variable_acc(x.cuda(), w.cuda(), 100, (pad, pad), (1, 1), 7, 8, 1, False, 2)
     with pytest.raises(RuntimeError):
-        sc_cuda.conv2d_or_acc(x.cuda(), w.cuda(), 64, (pad, pad), (1, 1), False)
+        sc_cuda.conv2d_or_acc(x.cuda(), w.cuda(), 100, (pad, pad), (1, 1), False)
 
 
 def test_runs_on_the_current_stream_and_single_hip_runtime(capi, fixtures_small):
