@@ -41,6 +41,10 @@ def parse():
     ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"],
                     help="C3 (default): the headline layer; C2: the 4-layer SC CNN training step")
     ap.add_argument("--length", type=int, default=0, help="stream length (default: the workload's)")
+    ap.add_argument("--accumulate", default="y", choices=["y", "z", "yz", "full"],
+                    help="accumulation mode of the single-layer workloads (default y: the headline)")
+    ap.add_argument("--z-unit", type=int, default=32, help="channels per OR group for --accumulate yz")
+    ap.add_argument("--generator", default="lfsr", choices=["lfsr", "acc", "rand"])
     ap.add_argument("--pass", dest="passes", default="fwdbwd", choices=["fwd", "fwdbwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
@@ -293,7 +297,9 @@ def main():
     L = args.length or L0
     x, w = wl.make_inputs(sx, sw, "prescribed", 0, vx, vw)
     xd, wd = x.cuda(), w.cuda()
-    desc = capi.make_desc(xd.shape, wd.shape, L, (pad, pad))
+    desc = capi.make_desc(xd.shape, wd.shape, L, (pad, pad), accumulate=args.accumulate, z_unit=args.z_unit,
+                          generator=args.generator, seed=1)
+    variant = args.accumulate != "y" or args.generator != "lfsr"
     ws = torch.empty(capi.workspace_size(desc), dtype=torch.uint8, device="cuda")
     out = torch.empty(capi.output_shape(desc), dtype=torch.int32, device="cuda")
 
@@ -348,7 +354,7 @@ def main():
     word_ops = 2 * B / 32
     achieved = word_ops / (k_avg * 1e-3)
     probe_rate = capi.probe_and_or_rate()
-    traffic = measured_traffic(args.workload, L)
+    traffic = None if variant else measured_traffic(args.workload, L)
     gen_ms = time_events(lambda: (capi.act_streams(xd, desc), capi.weight_streams(wd, desc)), min(args.steps, 10),
                          2, torch)
     N, Cin, Wx, Hx = xd.shape
@@ -371,7 +377,11 @@ def main():
         "dtype": "u32 bit-packed streams, int32 accumulate",
         "data": "synthetic (torch.manual_seed(0); activations U[0,1), weights U[-1,1))",
         "config": {"workload": f"{args.workload}: SC conv2d {tuple(x.shape)} * {tuple(w.shape)} pad {pad}, "
-                               f"stream length {L}, y-dimension partial binary accumulation, LFSR generators",
+                               f"stream length {L}, " + {
+                                   "y": "y-dimension partial binary accumulation", "z": "z-dimension accumulation",
+                                   "yz": f"yz accumulation with z_unit {args.z_unit}",
+                                   "full": "full OR accumulation"}[args.accumulate]
+                               + f", {args.generator} generators",
                    "pass": args.passes, "bit_macs_per_step": B},
         "layer_ms": {"fwd": fwd_avg, "bwd": bwd_avg, "fwd_bit_macs_per_s": B / (fwd_avg * 1e-3)},
         "roofline": {
@@ -398,7 +408,7 @@ def main():
                                                / (bwd_avg * 1e-3) / 1e12) if bwd_avg else None,
                            "peak_tflops_fp32_mfma": 157.3},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not variant:  # the compiled reference has the y / LFSR op only
         kind, cores, sec, note = cpu_baseline(x, w, L, pad)
         result["cpu_baseline"] = {
             "value": B / sec, "unit": "bit-MAC/s", "cores": cores, "kind": kind,
