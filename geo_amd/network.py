@@ -1,7 +1,8 @@
-"""The 4-layer SC CNN of the reference's training script (network.py:126-190,
-``CONV_tiny_add_partial``), restated on this build's layer modules, and the bookkeeping of
-one training step (utils_own.py:81-114).  Only what the 4-layer training-step workload
-needs; datasets, checkpointing and the CLI are not part of this build.
+"""The SC networks of the reference's training script restated on this build's layer modules:
+the 4-layer CNN (network.py:126-190, ``CONV_tiny_add_partial``) and VGG-16 (network.py:12-124,
+``VGG16_add_partial``), and the bookkeeping of one training step (utils_own.py:81-114).  The
+reference's LeNet (``CONV_minimal_add_partial``) is not restated: it builds on a layer class that
+does not exist in the reference (``utils_class.Linear_Or``, network.py:204-206).
 """
 from __future__ import annotations
 
@@ -148,6 +149,70 @@ class CONV_tiny_add_partial(nn.Module):
         g["x"].copy_(x)
         g["graph"].replay()
         return g["out"].clone()
+
+
+class VGG16_add_partial(nn.Module):
+    """VGG-16 for SC (network.py:12-124): thirteen 3x3 SC convolutions in five groups
+    (2, 2, 3, 3, 3 layers; AvgPool2 and Dropout2d after each group), a 1x1 SC convolution as the
+    classifier, fixed batch norm + Hardtanh(0,1) after every layer.  err / z_unit / load_unit /
+    load_wait hold one value per group plus one for the classifier; with ``half_pool`` the layer
+    in front of a pooling uses half the group's stream length (not below 2**5).  Same attribute
+    names as the reference, hence the same ``state_dict`` keys."""
+
+    GROUPS = ((1, 2), (3, 4), (5, 6, 7), (8, 9, 10), (11, 12, 13))
+    WIDTHS = (64, 128, 256, 512, 512)
+
+    def __init__(self, uniform=False, sc_compute="1d_bin", generator="lfsr", legacy=False, half_pool=True):
+        super().__init__()
+        c_in = 3
+        for group, width in zip(self.GROUPS, self.WIDTHS):
+            for i in group:
+                setattr(self, f"conv{i}", utils_class.Conv2d_Add_Partial(c_in, width, kernel_size=3, padding=1,
+                                                                         bias=False))
+                c_in = width
+        for g in range(1, 6):
+            setattr(self, f"drop{g}", nn.Dropout2d())
+        self.fc1 = utils_class.Conv2d_Add_Partial(512, 10, kernel_size=1, padding=0, bias=False)
+        self.pool = nn.AvgPool2d(2)
+        for group, width in zip(self.GROUPS, self.WIDTHS):
+            for i in group:
+                setattr(self, f"bn{i}", utils_class.BatchNorm2d_fixed(width))
+        self.bnfc1 = utils_class.BatchNorm1d_fixed(10)
+        self.tanh = nn.Hardtanh(0, 1)
+        self.err = [7, 7, 7, 7, 7, 7]
+        self.z_unit = [5, 5, 5, 5, 5, 5]
+        self.load_unit = [2, 2, 2, 2, 2, 2]
+        self.load_wait = [2, 2, 2, 2, 2, 2]
+        self.generator = generator
+        self.compute = sc_compute
+        self.legacy = legacy
+        self.half_pool = half_pool
+        if min(self.err) < 4:
+            uniform = True
+        if uniform:
+            for mod in self.modules():
+                if isinstance(mod, nn.Conv2d):
+                    mod.weight.data.uniform_()
+                    mod.weight_org.uniform_()
+
+    def _sc(self, conv, x, g, err):
+        return conv(x, err=err, forward=self.compute, generator=self.generator, z_unit=2 ** self.z_unit[g],
+                    legacy=self.legacy, load_unit=self.load_unit[g], load_wait_w=self.load_wait[g],
+                    load_wait_a=self.load_wait[g])
+
+    def forward(self, x):
+        pool_offset = 1 if self.half_pool else 0
+        for g, group in enumerate(self.GROUPS):
+            for i in group:
+                last = i == group[-1]
+                err = max(self.err[g] - pool_offset, 5) if last else self.err[g]
+                x = getattr(self, f"bn{i}")(self._sc(getattr(self, f"conv{i}"), x, g, err))
+                if last:
+                    x = self.pool(x)
+                x = self.tanh(x)
+            x = getattr(self, f"drop{g + 1}")(x)
+        x = self._sc(self.fc1, x, 5, self.err[5]).view(-1, 10)
+        return self.bnfc1(x)
 
 
 def make_param_copies(model):
