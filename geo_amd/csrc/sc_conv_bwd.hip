@@ -66,8 +66,8 @@ struct GemmParams {
 //   K-major operand: element (k, i) at p[k*ld + i]
 //   I-major operand: element (k, i) at p[i*ld + k]
 // VEC: the operand's leading dimension and extent along its contiguous axis are multiples of
-// 4 floats, so full chunks move as two float4 per thread; the last partial chunk and the
-// general case use guarded scalar loads (out-of-range lanes read a valid dummy address and
+// 4 floats, so chunks move as two float4 per thread (K-major: always, with whole rows of a
+// partial last chunk dropped; I-major: full chunks only); otherwise guarded scalar loads (out-of-range lanes read a valid dummy address and
 // are zeroed by a select, no divergent branches).
 template <bool KMAJOR, bool VEC>
 struct Stager {
@@ -105,12 +105,15 @@ struct Stager {
     // k_left = k_end - k0 of the chunk being fetched
     __device__ __forceinline__ void fetch(float (&r)[8], int k_left)
     {
-        if (VEC && k_left >= kChunk) {
-            const float* q0 = i_ok ? p : dummy;
-            const float* q1 = i_ok ? p + (KMAJOR ? 8 * ld : 4) : dummy;
+        if (VEC && (KMAJOR || k_left >= kChunk)) {
+            // K-major: the float4 runs along i, so a partial last chunk only drops whole rows
+            const bool ok0 = i_ok && (!KMAJOR || kk0 < k_left);
+            const bool ok1 = i_ok && (!KMAJOR || kk0 + 8 < k_left);
+            const float* q0 = ok0 ? p : dummy;
+            const float* q1 = ok1 ? p + (KMAJOR ? 8 * ld : 4) : dummy;
             const float4 v0 = *(const float4*)q0, v1 = *(const float4*)q1;
-            r[0] = i_ok ? v0.x : 0.0f; r[1] = i_ok ? v0.y : 0.0f; r[2] = i_ok ? v0.z : 0.0f; r[3] = i_ok ? v0.w : 0.0f;
-            r[4] = i_ok ? v1.x : 0.0f; r[5] = i_ok ? v1.y : 0.0f; r[6] = i_ok ? v1.z : 0.0f; r[7] = i_ok ? v1.w : 0.0f;
+            r[0] = ok0 ? v0.x : 0.0f; r[1] = ok0 ? v0.y : 0.0f; r[2] = ok0 ? v0.z : 0.0f; r[3] = ok0 ? v0.w : 0.0f;
+            r[4] = ok1 ? v1.x : 0.0f; r[5] = ok1 ? v1.y : 0.0f; r[6] = ok1 ? v1.z : 0.0f; r[7] = ok1 ? v1.w : 0.0f;
         } else {
 #pragma unroll
             for (int c = 0; c < 8; c++) {
@@ -146,6 +149,9 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wave's 64x64 corner in the tile
     const int l32 = lane & 31, lk = lane >> 5;
+    // which of this wave's four 32 x 32 blocks lie inside the result
+    const bool x0 = i0 + wi < q.I, x1 = i0 + wi + 32 < q.I, y0 = j0 + wj < q.J, y1 = j0 + wj + 32 < q.J;
+    const bool full = x1 && y1;
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -174,15 +180,29 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
             sa.fetch(ra, k_end - k0 - kChunk);
             sb.fetch(rb, k_end - k0 - kChunk);
         }
+        // v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32]
+        if (full) {
 #pragma unroll
-        for (int kk = 0; kk < kChunk; kk += 2) {
-            // v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32]
-            const float a0 = as[buf][kk + lk][wi + l32], a1 = as[buf][kk + lk][wi + 32 + l32];
-            const float b0 = bs[buf][kk + lk][wj + l32], b1 = bs[buf][kk + lk][wj + 32 + l32];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            for (int kk = 0; kk < kChunk; kk += 2) {
+                const float a0 = as[buf][kk + lk][wi + l32], a1 = as[buf][kk + lk][wi + 32 + l32];
+                const float b0 = bs[buf][kk + lk][wj + l32], b1 = bs[buf][kk + lk][wj + 32 + l32];
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            }
+        } else {
+            // edge tiles and narrow operands (few output channels, small OR groups): only the
+            // 32 x 32 blocks that hold results are computed
+#pragma unroll
+            for (int kk = 0; kk < kChunk; kk += 2) {
+                const float a0 = as[buf][kk + lk][wi + l32], a1 = as[buf][kk + lk][wi + 32 + l32];
+                const float b0 = bs[buf][kk + lk][wj + l32], b1 = bs[buf][kk + lk][wj + 32 + l32];
+                if (x0 && y0) acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+                if (x0 && y1) acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+                if (x1 && y0) acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+                if (x1 && y1) acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            }
         }
         if (more) {
             // the other buffer was last read one trip ago, before that trip's barrier
@@ -462,7 +482,9 @@ int launch_gemm(const GemmParams& q, int batch, hipStream_t s)
     // float4 staging needs every row start and every chunk start on a 16-byte boundary
     const bool a_vec = q.lda % 4 == 0 && ((uintptr_t)q.a & 15) == 0 && q.a_batch_stride % 4 == 0 && (AK ? q.I % 4 == 0 : true);
     const bool b_vec = q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0 && (BK ? q.J % 4 == 0 : true);
-    if (a_vec && b_vec && q.k_per_split % 4 == 0)
+    // an operand stored I-major moves float4 along k: its chunks must start on multiples of 4
+    const bool k_vec = (AK && BK) || q.k_per_split % 4 == 0;
+    if (a_vec && b_vec && k_vec)
         hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
     else
         hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, false>), grid, dim3(256), 0, s, q);
