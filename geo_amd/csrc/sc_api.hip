@@ -90,7 +90,15 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
         g->or_ch_per_group = g->z_unit;
     }
     g->seed_wrap = g->mode == GEO_SC_ACC_YZ ? (size_t)g->z_unit * wi * hi : (size_t)plane;
-    g->act_item_inner = g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
+    {
+        // waves the position-parallel kernel could start at most (one (pack, add group) pair per
+        // wave) against the 1024 SIMDs; members of one OR group against the 64 lanes
+        const long long pos_waves = (((long long)d->n * wo * ho + 63) / 64) * g->n_cotile * g->packs * g->add_outer *
+                                    g->add_inner;
+        const long long members = (long long)g->or_rows * g->or_ch_per_group * d->w_k;
+        g->thin = pos_waves < 2048 && members >= 64;
+    }
+    g->act_item_inner = !g->thin && g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
     g->wgt_words = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile * 2 * kCoTile;
     g->off_tables = 0;

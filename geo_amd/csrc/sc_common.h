@@ -40,6 +40,9 @@ struct Geometry {
     // innermost), used when the output has a single row so that the convolution kernel's lanes,
     // which then run over batch items, read consecutive words.
     bool act_item_inner;
+    // Few output positions but large OR groups (classifier layers): the convolution runs with
+    // lanes over the members of an OR group instead of over output positions.
+    bool thin;
     size_t act_words;    // n * packs * act_plane
     size_t wgt_words;    // packs * h_k * k_or * n_cotile * 2 * kCoTile
     // workspace carve-up (byte offsets, 256-aligned)

@@ -345,6 +345,72 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
     }
 }
 
+// Layers with few output positions and large OR groups (classifier layers: 64 x 4 x 4 -> 10 at
+// batch 256 has 2560 outputs of 1024 products each): one wave per (output position, c_out tile,
+// pack, add group); the lanes run over the members of the OR group, each with its own weight
+// line in VGPRs, and the 2 x 16 partial OR words are combined across the wave with xor shuffles.
+// Results are added into the zeroed y with integer atomics.  Activation layout [n][P][c_in][wi][hi].
+__global__ __launch_bounds__(64) void k_conv_fwd_thin(FwdParams q)
+{
+    constexpr int C = kCoTile;
+    const int lane = threadIdx.x;
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long m = blockIdx.x / q.n_cotile;
+    const int b = (int)(m % q.ho);
+    const long long t = m / q.ho;
+    const int a = (int)(t % q.wo);
+    const long long n = t / q.wo;
+    const int groups = q.add_outer * q.add_inner;
+    const int p = blockIdx.y / groups, g = blockIdx.y - p * groups;
+    const int go = g / q.add_inner, gi = g - go * q.add_inner;
+    const int ch0 = go * q.or_ch_per_group;
+    const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
+    const int members = q.or_rows * chs * q.w_k;
+    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    const size_t line0 = p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k + (size_t)gi * chs * q.w_k;
+    const uint32_t* ap0 = q.act + ((size_t)n * q.packs + p) * q.act_plane + (size_t)gi * q.add_stride +
+                          (size_t)ch0 * q.or_stride + (size_t)a * q.hi + b;
+
+    uint32_t orp[C], orn[C];
+#pragma unroll
+    for (int c = 0; c < C; c++) orp[c] = orn[c] = 0u;
+    for (int j = lane; j < members; j += 64) {
+        // member j = (kernel row of the OR, channel of the group, tap u), u fastest
+        const int u = j % q.w_k, t2 = j / q.w_k;
+        const int ch = t2 % chs, row = t2 / chs;
+        const uint32_t aw = ap0[(size_t)ch * q.or_stride + (size_t)u * q.hi + row];
+        const uint4* wl = reinterpret_cast<const uint4*>(q.wgt + ((line0 + j) * q.n_cotile + cot) * (2 * C));
+        uint32_t wv[2 * C];
+#pragma unroll
+        for (int v4 = 0; v4 < 2 * C / 4; v4++) {
+            const uint4 w4 = wl[v4];
+            wv[4 * v4] = w4.x;
+            wv[4 * v4 + 1] = w4.y;
+            wv[4 * v4 + 2] = w4.z;
+            wv[4 * v4 + 3] = w4.w;
+        }
+#pragma unroll
+        for (int c = 0; c < C; c++) {
+            orp[c] |= aw & wv[c];
+            orn[c] |= aw & wv[C + c];
+        }
+    }
+    int mine = 0;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        uint32_t vp = orp[c], vn = orn[c];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            vp |= (uint32_t)__shfl_xor((int)vp, off);
+            vn |= (uint32_t)__shfl_xor((int)vn, off);
+        }
+        if (lane == c) mine = __popc(vp) - __popc(vn);
+    }
+    const int co = cot * C + lane;
+    if (lane < C && co < q.c_out)
+        atomicAdd(q.y + (((size_t)n * q.c_out + co) * q.wo + a) * q.ho + b, mine);
+}
+
 __global__ __launch_bounds__(256) void k_zero_i32(int32_t* __restrict__ p, size_t n)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0;
@@ -418,6 +484,16 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     q.add_stride = g.mode == GEO_SC_ACC_Z ? ch_plane : 1u;
     q.or_stride = g.mode == GEO_SC_ACC_Z ? 1u : ch_plane;
     q.or_rows = g.or_rows;
+    if (g.thin) {
+        const long long blocks = (long long)g.n * g.wo * g.ho * g.n_cotile;
+        const long long pv = (long long)g.packs * g.add_outer * g.add_inner;
+        if (blocks > 0x7fffffffLL || pv > 65535 || g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
+        const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
+        size_t zb = (n_out + 255) / 256;
+        hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
+        hipLaunchKernelGGL(k_conv_fwd_thin, dim3((unsigned)blocks, (unsigned)pv), dim3(64), 0, s, q);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
     // Two accumulator rows per lane halve the weight traffic per instruction.  Outputs with
     // several rows take them along dim 2 (sliding-window reuse of activation words); outputs
     // with a single row (the SC-linear mapping, classifier layers) take two batch items.

@@ -252,3 +252,34 @@ def test_runs_on_the_current_stream_and_single_hip_runtime(capi, fixtures_small)
     with open("/proc/self/maps") as f:
         hips = {line.split()[-1] for line in f if "libamdhip64" in line}
     assert len(hips) == 1, hips
+
+
+# ------------------------------------------------------------------ classifier-type layers
+THIN_CASES = [
+    # few output positions, OR groups of at least 64 members: the member-parallel kernel
+    ((6, 64, 4, 4), (10, 64, 4, 4), (0, 0)),       # the 4-layer CNN's classifier
+    ((5, 40, 3, 3), (19, 40, 3, 3), (0, 0)),       # 120 members: ragged over the 64 lanes; two c_out tiles
+    ((3, 128, 1, 1), (33, 128, 1, 1), (0, 0)),     # 1x1 classifier, three c_out tiles
+    ((2, 70, 4, 5), (5, 70, 3, 3), (1, 1)),        # several output positions per item, padding
+    ((2, 24, 5, 4), (7, 24, 2, 3), (1, 0)),        # even kernel extent
+]
+
+
+@pytest.mark.parametrize("case", range(len(THIN_CASES)))
+@pytest.mark.parametrize("L", [8, 64, 256])
+def test_classifier_layers_match_oracle(capi, so, case, L):
+    sx, sw, pad = THIN_CASES[case]
+    x, w = wl.make_inputs(sx, sw, "kaiming", seed=700 + case)
+    w = (w * 3).contiguous()
+    print(f"classifier case {sx} {sw} pad {pad} L {L}", flush=True)
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad, 7, 2, 2, 2)
+    assert L < 64 or np.abs(exp).sum() > 0   # short streams of small weights round to nothing
+    assert np.array_equal(gpu_forward(capi, x, w, L, pad, total_width=7, load_width=2, load_wait_w=2, load_wait_a=2),
+                          exp)
+    for mode, zu in (("yz", 32), ("full", 1)):
+        e2 = so.conv2d_general(x.numpy(), w.numpy(), L, pad, mode, zu)
+        assert np.array_equal(gpu_forward(capi, x, w, L, pad, accumulate=mode, z_unit=zu), e2), mode
+    # 7-bit integer activations take the same path
+    k = (x * 128).round().clamp(0, 127).to(torch.uint8)
+    a = capi.conv2d_add_partial_forward_q7(k.cuda(), w.cuda(), L, pad)
+    assert np.array_equal(a.cpu().numpy(), so.conv2d_add_partial((k.float() / 128).numpy(), w.numpy(), L, pad))
