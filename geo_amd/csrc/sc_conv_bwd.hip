@@ -54,9 +54,8 @@ struct GemmParams {
     int k_per_split;
     long long c_split_stride;
     long long a_batch_stride, b_batch_stride, c_batch_stride;
-    // EPI_EXP_TIMES_G: c[i][j] = g[goff[i] + (j % c_out) * npos] * exp(-acc)
+    // EPI_EXP_TIMES_G: c[i][j] = g[i * c_out + (j % c_out)] * exp(-acc), g = upstream gradient stored [m][c_out]
     const float* __restrict__ g;
-    const int* __restrict__ goff;
     int c_out, npos;
 };
 
@@ -228,19 +227,39 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
                 float v = acc[x][y][r];
                 if (EPI == EPI_EXP_TIMES_G) {
                     const int co = j >= q.c_out ? j - q.c_out : j;
-                    v = q.g[q.goff[i] + co * q.npos] * expf(-v);
+                    v = q.g[(long long)i * q.c_out + co] * expf(-v);
                 }
                 c[(long long)i * q.ldc + j] = v;
             }
         }
 }
 
+// gt[n*npos + pos][co] = g[n][co][pos]: the upstream gradient with the channel innermost, so that the
+// first GEMM's epilogue (lanes along the channel) reads it in contiguous runs instead of one
+// cache line per lane.  32 x 32 tiles through LDS; blockIdx.z = n.
+__global__ __launch_bounds__(256) void k_transpose_grad(const float* __restrict__ g, float* __restrict__ gt, int c_out,
+                                                        int npos)
+{
+    __shared__ float tile[32][33];
+    const size_t item = (size_t)blockIdx.z * c_out * npos;
+    const int p0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int r = ty; r < 32; r += 8) {
+        const int c = c0 + r, p = p0 + tx;
+        tile[r][tx] = (c < c_out && p < npos) ? g[item + (size_t)c * npos + p] : 0.0f;
+    }
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8) {
+        const int p = p0 + r, c = c0 + tx;
+        if (p < npos && c < c_out) gt[item + (size_t)p * c_out + c] = tile[tx][r];
+    }
+}
+
 // Per output position m = (n, a, b): where its receptive field starts in the unpadded input.
 //   base[m] = ((n*c_in)*w_in + (a - pad_w))*h_in + (b - pad_h),  arow[m] = a - pad_w,  bcol[m] = b - pad_h
-//   goff[m] = (n*c_out)*npos + (a*ho + b): index of grad_y[n][0][a][b]
 // Built once per call; it keeps integer divisions out of the per-element kernels.
 __global__ __launch_bounds__(256) void k_position_table(int* __restrict__ base, int* __restrict__ arow,
-                                                        int* __restrict__ bcol, int* __restrict__ goff, int m_total,
+                                                        int* __restrict__ bcol, int m_total,
                                                         int c_in, int c_out, int w_in, int h_in, int pad_w, int pad_h,
                                                         int wo, int ho)
 {
@@ -252,7 +271,6 @@ __global__ __launch_bounds__(256) void k_position_table(int* __restrict__ base, 
         base[m] = ((n * c_in) * w_in + (a - pad_w)) * h_in + (b - pad_h);
         arow[m] = a - pad_w;
         bcol[m] = b - pad_h;
-        goff[m] = n * c_out * wo * ho + (m - n * wo * ho);
     }
 }
 
@@ -499,7 +517,7 @@ struct BwdLayout {
     Groups G;
     int rows_per_chunk;  // add groups processed by one round of launches
     size_t col_v, e_v, part_v, w_v;  // floats per add group of each scratch array
-    size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, bytes;
+    size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, off_gt, bytes;
 };
 
 BwdLayout bwd_layout(const Geometry& g)
@@ -554,7 +572,8 @@ BwdLayout bwd_layout(const Geometry& g)
     b.off_part = o; o += align256(sizeof(float) * rows * b.part_v);
     b.off_wcat = o; o += align256(sizeof(float) * rows * b.w_v);
     b.off_wd = o;   o += align256(sizeof(float) * rows * b.w_v);
-    b.off_pos = o;  o += 4 * align256(sizeof(int) * (size_t)b.m_total);
+    b.off_pos = o;  o += 3 * align256(sizeof(int) * (size_t)b.m_total);
+    b.off_gt = o;   o += align256(sizeof(float) * (size_t)b.m_total * g.c_out);
     b.bytes = o;
     return b;
 }
@@ -584,10 +603,16 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     int* pos_base = (int*)(ws + L.off_pos);
     int* pos_arow = pos_base + pos_stride;
     int* pos_bcol = pos_arow + pos_stride;
-    int* pos_goff = pos_bcol + pos_stride;
+    float* gt = (float*)(ws + L.off_gt);
     const int m_blocks = grid1d(M);
-    hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, pos_goff, M,
+    hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
                        g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
+    {
+        const int npos = g.wo * g.ho;
+        if (g.n > 65535) return GEO_SC_ERR_UNSUPPORTED;  // grid.z of the transpose
+        hipLaunchKernelGGL(k_transpose_grad, dim3((npos + 31) / 32, (g.c_out + 31) / 32, g.n), dim3(256), 0, s, gy, gt,
+                           g.c_out, npos);
+    }
     int rc;
     for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
         const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
@@ -607,7 +632,7 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         q1.splits = 1; q1.k_per_split = K; q1.c_split_stride = 0;
         q1.a_batch_stride = (long long)L.col_v; q1.b_batch_stride = (long long)L.w_v;
         q1.c_batch_stride = (long long)L.e_v;
-        q1.g = gy; q1.goff = pos_goff; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
+        q1.g = gt; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
         if ((rc = launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, nv, s)) != GEO_SC_OK) return rc;
         if (gw) {
             // partial Gw[v][s][k][j] = sum_{m in split s} col_v[k][m] * E_v[m][j]
