@@ -289,38 +289,48 @@ struct RandParams {
     uint32_t seed;
 };
 
-// The P stream words of one element, handed to put(pack, word).
+// The P stream words of one element, handed to put(pack, word).  Bits are produced in stream
+// order, one Philox block (four words) at a time: field f of word w of block blk is stream bit
+// (4*blk + w) * cpw + f.
 template <typename Put>
 __device__ __forceinline__ void random_stream(const RandParams& rp, int code, uint32_t tag, uint64_t index, Put put)
 {
-    uint32_t r[4] = {0, 0, 0, 0};
-    int have_block = -1;
-    const int cpw = rp.generator == GEO_SC_GEN_RAND ? 32 / rp.n_bits : 2;
-    int left_ones = code, left_total = rp.L;
-    for (int p = 0; p < rp.packs; p++) {
-        uint32_t word = 0;
-        if (code != 0) {
-            for (int b = 0; b < rp.bit_unit; b++) {
-                const int t = p * rp.bit_unit + b;
-                const int j = t / cpw, f = t - j * cpw;
-                if ((j >> 2) != have_block) {
-                    have_block = j >> 2;
-                    philox4x32_10((uint32_t)have_block, (uint32_t)index, (uint32_t)(index >> 32), tag, rp.seed, 0u, r);
-                }
-                const uint32_t rw = (j & 3) == 0 ? r[0] : (j & 3) == 1 ? r[1] : (j & 3) == 2 ? r[2] : r[3];
+    if (code == 0) {
+        for (int p = 0; p < rp.packs; p++) put(p, 0u);
+        return;
+    }
+    const bool bernoulli = rp.generator == GEO_SC_GEN_RAND;
+    const int cpw = bernoulli ? 32 / rp.n_bits : 2;
+    const int shift = bernoulli ? rp.n_bits : 16;
+    const uint32_t mask = bernoulli ? (uint32_t)(rp.L - 1) : 0xffffu;
+    uint32_t left_ones = (uint32_t)code, left_total = (uint32_t)rp.L;
+    uint32_t word = 0;
+    int t = 0, in_word = 0, p = 0;
+    for (uint32_t blk = 0; t < rp.L; blk++) {
+        uint32_t r[4];
+        philox4x32_10(blk, (uint32_t)index, (uint32_t)(index >> 32), tag, rp.seed, 0u, r);
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            uint32_t rw = r[w];
+            for (int f = 0; f < cpw && t < rp.L; f++, t++) {
+                const uint32_t field = rw & mask;
+                rw >>= shift;
                 uint32_t bit;
-                if (rp.generator == GEO_SC_GEN_RAND) {
-                    bit = (uint32_t)code > ((rw >> (f * rp.n_bits)) & (uint32_t)(rp.L - 1));
+                if (bernoulli) {
+                    bit = (uint32_t)code > field;
                 } else {
-                    const uint32_t r16 = (rw >> (16 * f)) & 0xffffu;
-                    bit = r16 * (uint32_t)left_total < (uint32_t)left_ones * 65536u;
-                    left_ones -= (int)bit;
-                    left_total -= 1;
+                    bit = field * left_total < left_ones * 65536u;
+                    left_ones -= bit;
+                    left_total -= 1u;
                 }
                 word = word * 2u + bit;
+                if (++in_word == rp.bit_unit) {
+                    put(p++, word);
+                    word = 0;
+                    in_word = 0;
+                }
             }
         }
-        put(p, word);
     }
 }
 
