@@ -136,28 +136,33 @@ def bench_network_step(args, torch):
 
     L = args.length or 64
     torch.manual_seed(0)
-    model = network.CONV_tiny_add_partial().cuda().train()
-    model.err = [L.bit_length() - 1] * 4
-    model.load_unit = [2] * 4
-    model.load_wait = [2] * 4
     g = torch.Generator().manual_seed(0)
     x = torch.rand((256, 3, 32, 32), generator=g).cuda()
     t = torch.randint(10, (256,), generator=g).cuda()
-    copies = network.make_param_copies(model)
-    opt = torch.optim.Adam(copies, lr=2e-3)
     crit = torch.nn.CrossEntropyLoss()
 
-    def step():
-        return network.train_step(model, x.clone(), t, crit, opt, copies)
+    def timed_steps(fused_blocks):
+        """ms per training step; fused_blocks: every conv + batch norm + pool + hardtanh block as one
+        autograd node on the fused HIP tail kernels (same values as the module chain)."""
+        torch.manual_seed(0)
+        model = network.CONV_tiny_add_partial().cuda().train()
+        model.err = [L.bit_length() - 1] * 4
+        model.load_unit = [2] * 4
+        model.load_wait = [2] * 4
+        model.fused_blocks = fused_blocks
+        copies = network.make_param_copies(model)
+        opt = torch.optim.Adam(copies, lr=2e-3)
+        for _ in range(args.warmup):
+            network.train_step(model, x.clone(), t, crit, opt, copies)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            network.train_step(model, x.clone(), t, crit, opt, copies)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_module_chain = timed_steps(False)
+    ms_per_step = timed_steps(True)
 
     layers = {}
     B_total = 0
@@ -192,8 +197,10 @@ def bench_network_step(args, torch):
         "vs_baseline": None, "dtype": "u32 bit-packed streams, int32 accumulate; fp32 backward",
         "data": "synthetic (torch.manual_seed(0); images U[0,1), uniform random labels)",
         "config": {"workload": "C2: 4-layer SC CNN (3->32 k5 @32, 32->32 k5 @16, 32->64 k5 @8, 64->10 k4 @4), batch "
-                               f"256, stream length {L}, load_unit 2 / load_wait 2, fwd+bwd+Adam step",
+                               f"256, stream length {L}, load_unit 2 / load_wait 2, fwd+bwd+Adam step, fused "
+                               "conv + batch-norm + pool + hardtanh blocks",
                    "pass": "train step", "bit_macs_per_step": B_total},
+        "module_chain_ms_per_step": ms_module_chain,
         "layers": layers,
         "roofline": {"bound": "valu", "kernel": "k_conv_fwd, the four layers' launches together",
                      "achieved": achieved / 1e12, "peak": PEAK_VALU_WORD_OPS / 1e12, "unit": "T word-op/s",

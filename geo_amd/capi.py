@@ -144,6 +144,52 @@ def layer_epilogue(counts, bit_length, w_n, b_n, relu=False, pool=True, hardtanh
     return act, q7
 
 
+def layer_tail_backward(counts, grad_out, bit_length, w_n, b_n, mean, invstd, gamma=None, relu=False, pool=True,
+                        hardtanh=True, stream=None):
+    """geo_sc_layer_tail_backward: (grad_y, grad_gamma, grad_beta) of the training-mode layer tail
+    (batch norm on the batch statistics, relu, AvgPool2d(2), Hardtanh(0, 1))."""
+    n, c, w, h = counts.shape
+    dev = counts.device
+    f = lambda t: t.to(dev, torch.float32).contiguous()
+    grad_out, w_n, b_n, mean, invstd = f(grad_out), f(w_n), f(b_n), f(mean), f(invstd)
+    gamma = None if gamma is None else f(gamma)
+    exp = (n, c, w // 2, h // 2) if pool else (n, c, w, h)
+    if tuple(grad_out.shape) != exp:
+        raise ValueError(f"grad_out has shape {tuple(grad_out.shape)}, expected {exp}")
+    flags = (EPI_RELU if relu else 0) | (EPI_POOL2 if pool else 0) | (EPI_HARDTANH01 if hardtanh else 0)
+    nbytes = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_layer_tail_backward_workspace_size(n, c, w, h, ctypes.byref(nbytes)), "tail workspace")
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+    grad_y = torch.empty((n, c, w, h), dtype=torch.float32, device=dev)
+    gg = torch.empty(c, dtype=torch.float32, device=dev)
+    gb = torch.empty(c, dtype=torch.float32, device=dev)
+    _check(_native.lib().geo_sc_layer_tail_backward(_ptr(counts), _ptr(grad_out), n, c, w, h, int(bit_length), _ptr(w_n),
+                                                    _ptr(b_n), _ptr(mean), _ptr(invstd), _ptr(gamma), flags,
+                                                    _ptr(grad_y), _ptr(gg), _ptr(gb), _ptr(ws), ws.numel(),
+                                                    _stream_ptr(stream)), "geo_sc_layer_tail_backward")
+    return grad_y, gg, gb
+
+
+def bn_fixed_affine(mean, var, gamma, beta, eps, elements_per_channel, running_mean=None, running_var=None,
+                    eps_grad=1e-5, stream=None):
+    """geo_sc_bn_fixed_affine: (w_n, b_n, invstd, scale) of a fixed-point batch norm from channel
+    statistics; updates running_mean / running_var in place when given."""
+    c = mean.numel()
+    dev = mean.device
+    for t in (mean, var, gamma, beta, running_mean, running_var):
+        if t is not None and not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == c):
+            raise ValueError("statistics and parameters must be contiguous float32 GPU tensors of one size")
+    w_n = torch.empty(c, dtype=torch.float32, device=dev)
+    b_n = torch.empty(c, dtype=torch.float32, device=dev)
+    invstd = torch.empty(c, dtype=torch.float32, device=dev)
+    scale = torch.empty((), dtype=torch.float32, device=dev)
+    _check(_native.lib().geo_sc_bn_fixed_affine(_ptr(mean), _ptr(var), _ptr(gamma), _ptr(beta), c, float(eps),
+                                                float(eps_grad), int(elements_per_channel), _ptr(running_mean),
+                                                _ptr(running_var), _ptr(w_n), _ptr(b_n), _ptr(invstd), _ptr(scale),
+                                                _stream_ptr(stream)), "geo_sc_bn_fixed_affine")
+    return w_n, b_n, invstd, scale
+
+
 def _tables(bit_length, device):
     n = ctypes.c_size_t(0)
     _check(_native.lib().geo_sc_stream_tables_size(int(bit_length), ctypes.byref(n)), "tables size")

@@ -107,6 +107,197 @@ __global__ __launch_bounds__(256) void k_layer_epilogue_pool_vec(EpiParams q, un
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Backward of the layer tail in training mode.  The reference's autograd sees
+//     y = count / L -> F.batch_norm(y, training=True) (its value replaced by y * w_n + b_n,
+//     utils_class.py:49-64) -> relu -> AvgPool2d(2) -> Hardtanh(0, 1)
+// so the gradient is that of an ordinary batch norm on the batch statistics, with the relu and
+// hardtanh masks taken from the fixed-point values that actually flowed forward:
+//     d[n,c,i,j]  = grad_out[n,c,i/2,j/2] * [0 < pooled value < 1] / 4 * [value before relu > 0]
+//     dbeta[c]    = sum d,   dgamma[c] = sum d * xhat,   xhat = (y - mean[c]) * invstd[c]
+//     dy          = gamma[c] * invstd[c] * (d - dbeta[c] / M - xhat * dgamma[c] / M),  M = n*w*h
+// Three kernels: per-channel partial sums (fixed-order tree per block), their sum in split order
+// (deterministic), and the element-wise application.
+struct TailParams {
+    const int32_t* __restrict__ counts;
+    const float* __restrict__ gout;
+    const float* __restrict__ w_n;
+    const float* __restrict__ b_n;
+    const float* __restrict__ mean;
+    const float* __restrict__ invstd;
+    const float* __restrict__ gamma;  // may be null: 1
+    int n, c, w, h, wo, ho;
+    float inv_len;
+    int flags;
+    int splits;
+};
+
+// gradient reaching the batch-norm output at (item-channel plane nc, i, j)
+__device__ __forceinline__ float tail_d(const TailParams& q, long long nc, int i, int j, float wn, float bn, int count_ij)
+{
+    const bool relu = q.flags & GEO_SC_EPI_RELU;
+    float g;
+    if (q.flags & GEO_SC_EPI_POOL2) {
+        if (i >= 2 * q.wo || j >= 2 * q.ho) return 0.0f;
+        const int a = i >> 1, b = j >> 1;
+        const int32_t* src = q.counts + (nc * q.w + 2 * a) * q.h + 2 * b;
+        const float v00 = affine(src[0], q.inv_len, wn, bn, relu), v01 = affine(src[1], q.inv_len, wn, bn, relu);
+        const float v10 = affine(src[q.h], q.inv_len, wn, bn, relu), v11 = affine(src[q.h + 1], q.inv_len, wn, bn, relu);
+        const float pooled = __fadd_rn(__fadd_rn(__fadd_rn(v00, v01), v10), v11) / 4.0f;
+        g = q.gout[(nc * q.wo + a) * q.ho + b];
+        if ((q.flags & GEO_SC_EPI_HARDTANH01) && !(pooled > 0.0f && pooled < 1.0f)) g = 0.0f;
+        g *= 0.25f;
+    } else {
+        const float v = affine(count_ij, q.inv_len, wn, bn, relu);
+        g = q.gout[(nc * q.w + i) * q.h + j];
+        if ((q.flags & GEO_SC_EPI_HARDTANH01) && !(v > 0.0f && v < 1.0f)) g = 0.0f;
+    }
+    if (relu && !(affine(count_ij, q.inv_len, wn, bn, false) > 0.0f)) g = 0.0f;
+    return g;
+}
+
+// partial[ch][split][2]: sums of d and d * xhat over this split's share of the channel's elements
+__global__ __launch_bounds__(256) void k_tail_bwd_partial(TailParams q, float* __restrict__ partial)
+{
+    __shared__ float red[2][256];
+    const int ch = blockIdx.y;
+    const float wn = q.w_n[ch], bn = q.b_n[ch], mu = q.mean[ch], is = q.invstd[ch];
+    const int plane = q.w * q.h;
+    const long long per_channel = (long long)q.n * plane;
+    float s1 = 0.0f, s2 = 0.0f;
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < per_channel; e += (long long)q.splits * 256) {
+        const long long item = e / plane;
+        const int r = (int)(e - item * plane);
+        const int i = r / q.h, j = r - i * q.h;
+        const long long nc = item * q.c + ch;
+        const int cnt = q.counts[nc * plane + r];
+        const float d = tail_d(q, nc, i, j, wn, bn, cnt);
+        const float xhat = ((float)cnt * q.inv_len - mu) * is;
+        s1 += d;
+        s2 += d * xhat;
+    }
+    red[0][threadIdx.x] = s1;
+    red[1][threadIdx.x] = s2;
+    __syncthreads();
+    for (int step = 128; step >= 1; step >>= 1) {
+        if ((int)threadIdx.x < step) {
+            red[0][threadIdx.x] += red[0][threadIdx.x + step];
+            red[1][threadIdx.x] += red[1][threadIdx.x + step];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partial[((size_t)ch * q.splits + blockIdx.x) * 2] = red[0][0];
+        partial[((size_t)ch * q.splits + blockIdx.x) * 2 + 1] = red[1][0];
+    }
+}
+
+__global__ __launch_bounds__(256) void k_tail_bwd_finalize(const float* __restrict__ partial, int c, int splits,
+                                                           float* __restrict__ sums /* [c][2]: dbeta, dgamma */)
+{
+    const int ch = blockIdx.x * 256 + threadIdx.x;
+    if (ch >= c) return;
+    float s1 = 0.0f, s2 = 0.0f;
+    for (int s = 0; s < splits; s++) {
+        s1 += partial[((size_t)ch * splits + s) * 2];
+        s2 += partial[((size_t)ch * splits + s) * 2 + 1];
+    }
+    sums[2 * ch] = s1;
+    sums[2 * ch + 1] = s2;
+}
+
+__global__ __launch_bounds__(256) void k_tail_bwd_apply(TailParams q, const float* __restrict__ sums,
+                                                        float* __restrict__ grad_y, float* __restrict__ grad_gamma,
+                                                        float* __restrict__ grad_beta)
+{
+    const int plane = q.w * q.h;
+    const long long total = (long long)q.n * q.c * plane;
+    const float inv_m = 1.0f / (float)((long long)q.n * plane);
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)gridDim.x * 256) {
+        const long long nc = e / plane;
+        const int r = (int)(e - nc * plane);
+        const int i = r / q.h, j = r - i * q.h;
+        const int ch = (int)(nc % q.c);
+        const float is = q.invstd[ch];
+        const int cnt = q.counts[e];
+        const float d = tail_d(q, nc, i, j, q.w_n[ch], q.b_n[ch], cnt);
+        const float xhat = ((float)cnt * q.inv_len - q.mean[ch]) * is;
+        const float gm = q.gamma ? q.gamma[ch] : 1.0f;
+        grad_y[e] = gm * is * (d - sums[2 * ch] * inv_m - xhat * sums[2 * ch + 1] * inv_m);
+    }
+    if (blockIdx.x == 0)
+        for (int ch = threadIdx.x; ch < q.c; ch += 256) {
+            if (grad_beta) grad_beta[ch] = sums[2 * ch];
+            if (grad_gamma) grad_gamma[ch] = sums[2 * ch + 1];
+        }
+}
+
+// The fixed-point affine of BatchNorm*_fixed from per-channel statistics (utils_class.py:52-62 with
+// quantize_shift, utils_functional.py:41-57), one workgroup:
+//     inv = sqrt(var + eps);  w = gamma / inv;  b = beta - mean * gamma / inv
+//     scale = 2 ** ceil(log2(mean_over_channels(w) * 3))
+//     w_n = round(w / scale * 128).clamp(-127, 127) / 128 * scale,   b_n likewise with the same scale
+// in PyTorch's operation order, one rounding per operation.  Also the running statistics of
+// F.batch_norm(training=True) (momentum 0.1, unbiased variance) and 1 / sqrt(var + eps_grad) for the
+// backward.  The channel mean is accumulated in double precision.
+__global__ __launch_bounds__(256) void k_bn_fixed_affine(const float* __restrict__ mean, const float* __restrict__ var,
+                                                         const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                         int c, float eps, float eps_grad, float unbias,
+                                                         float* __restrict__ running_mean,
+                                                         float* __restrict__ running_var, float* __restrict__ w_n,
+                                                         float* __restrict__ b_n, float* __restrict__ invstd,
+                                                         float* __restrict__ scale_out)
+{
+    __shared__ double red[256];
+    __shared__ float scale_s;
+    double part = 0.0;
+    for (int ch = threadIdx.x; ch < c; ch += 256) {
+        const float inv = __fsqrt_rn(__fadd_rn(var[ch], eps));
+        const float gm = gamma ? gamma[ch] : 1.0f;
+        part += (double)__fdiv_rn(gm, inv);
+    }
+    red[threadIdx.x] = part;
+    __syncthreads();
+    for (int step = 128; step >= 1; step >>= 1) {
+        if ((int)threadIdx.x < step) red[threadIdx.x] += red[threadIdx.x + step];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const float m = (float)(red[0] / (double)c);
+        scale_s = exp2f(ceilf(log2f(__fmul_rn(m, 3.0f))));
+        if (scale_out) *scale_out = scale_s;
+    }
+    __syncthreads();
+    const float scale = scale_s;
+    for (int ch = threadIdx.x; ch < c; ch += 256) {
+        const float mu = mean[ch], vr = var[ch];
+        const float inv = __fsqrt_rn(__fadd_rn(vr, eps));
+        const float gm = gamma ? gamma[ch] : 1.0f, bt = beta ? beta[ch] : 0.0f;
+        const float w = __fdiv_rn(gm, inv);
+        const float b = __fsub_rn(bt, __fdiv_rn(__fmul_rn(mu, gm), inv));
+        const float qw = fminf(fmaxf(rintf(__fmul_rn(__fdiv_rn(w, scale), 128.0f)), -127.0f), 127.0f);
+        const float qb = fminf(fmaxf(rintf(__fmul_rn(__fdiv_rn(b, scale), 128.0f)), -127.0f), 127.0f);
+        w_n[ch] = __fmul_rn(__fdiv_rn(qw, 128.0f), scale);
+        b_n[ch] = __fmul_rn(__fdiv_rn(qb, 128.0f), scale);
+        if (invstd) invstd[ch] = 1.0f / __fsqrt_rn(__fadd_rn(vr, eps_grad));
+        if (running_mean) running_mean[ch] = __fadd_rn(__fmul_rn(running_mean[ch], 0.9f), __fmul_rn(mu, 0.1f));
+        if (running_var)
+            running_var[ch] = __fadd_rn(__fmul_rn(running_var[ch], 0.9f), __fmul_rn(__fmul_rn(vr, unbias), 0.1f));
+    }
+}
+
+int tail_splits(int n, int c, int w, int h)
+{
+    // enough blocks to fill the GPU, not more than the channel has 256-element chunks
+    const long long per_channel = (long long)n * w * h;
+    long long s = (4096 + c - 1) / c;
+    const long long chunks = (per_channel + 255) / 256;
+    if (s > chunks) s = chunks;
+    if (s < 1) s = 1;
+    if (s > 1024) s = 1024;
+    return (int)s;
+}
+
 }  // namespace
 
 }  // namespace geo_sc
@@ -155,5 +346,73 @@ extern "C" int geo_sc_layer_epilogue(const int32_t* counts, int n, int c, int w,
     long long blocks = (q.total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     hipLaunchKernelGGL(k_layer_epilogue, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, q);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_layer_tail_backward_workspace_size(int n, int c, int w, int h, size_t* bytes)
+{
+    if (!bytes || n < 1 || c < 1 || w < 1 || h < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
+    *bytes = sizeof(float) * 2 * ((size_t)c * tail_splits(n, c, w, h) + (size_t)c);
+    return GEO_SC_OK;
+}
+
+extern "C" int geo_sc_layer_tail_backward(const int32_t* counts, const float* grad_out, int n, int c, int w, int h,
+                                          int bit_length, const float* w_n, const float* b_n, const float* mean,
+                                          const float* invstd, const float* gamma, int flags, float* grad_y,
+                                          float* grad_gamma, float* grad_beta, void* workspace,
+                                          size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    if (!counts || !grad_out || !w_n || !b_n || !mean || !invstd || !grad_y) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (n < 1 || c < 1 || w < 1 || h < 1 || c > 65535) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (flags & ~(GEO_SC_EPI_RELU | GEO_SC_EPI_POOL2 | GEO_SC_EPI_HARDTANH01 | GEO_SC_EPI_QUANT7))
+        return GEO_SC_ERR_INVALID_ARGUMENT;
+    switch (bit_length) {
+    case 8: case 16: case 32: case 64: case 128: case 256: break;
+    default: return GEO_SC_ERR_BIT_LENGTH;
+    }
+    size_t need = 0;
+    geo_sc_layer_tail_backward_workspace_size(n, c, w, h, &need);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 3u)) return GEO_SC_ERR_WORKSPACE;
+    TailParams q;
+    q.counts = counts;
+    q.gout = grad_out;
+    q.w_n = w_n;
+    q.b_n = b_n;
+    q.mean = mean;
+    q.invstd = invstd;
+    q.gamma = gamma;
+    q.n = n;
+    q.c = c;
+    q.w = w;
+    q.h = h;
+    q.wo = (flags & GEO_SC_EPI_POOL2) ? w / 2 : w;
+    q.ho = (flags & GEO_SC_EPI_POOL2) ? h / 2 : h;
+    if (q.wo < 1 || q.ho < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
+    q.inv_len = 1.0f / (float)bit_length;
+    q.flags = flags;
+    q.splits = tail_splits(n, c, w, h);
+    hipStream_t s = (hipStream_t)stream;
+    float* partial = (float*)workspace;
+    float* sums = partial + (size_t)2 * c * q.splits;
+    hipLaunchKernelGGL(k_tail_bwd_partial, dim3(q.splits, c), dim3(256), 0, s, q, partial);
+    hipLaunchKernelGGL(k_tail_bwd_finalize, dim3((c + 255) / 256), dim3(256), 0, s, partial, c, q.splits, sums);
+    const long long total = (long long)n * c * w * h;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipLaunchKernelGGL(k_tail_bwd_apply, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma, grad_beta);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_bn_fixed_affine(const float* mean, const float* var, const float* gamma, const float* beta,
+                                      int c, float eps, float eps_grad, long long elements_per_channel,
+                                      float* running_mean, float* running_var, float* w_n, float* b_n, float* invstd,
+                                      float* scale, geo_sc_stream_t stream)
+{
+    if (!mean || !var || !w_n || !b_n || c < 1 || elements_per_channel < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const float unbias = elements_per_channel > 1
+                             ? (float)((double)elements_per_channel / (double)(elements_per_channel - 1))
+                             : 1.0f;
+    hipLaunchKernelGGL(k_bn_fixed_affine, dim3(1), dim3(256), 0, (hipStream_t)stream, mean, var, gamma, beta, c, eps,
+                       eps_grad, unbias, running_mean, running_var, w_n, b_n, invstd, scale);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }

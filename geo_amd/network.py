@@ -46,6 +46,9 @@ class CONV_tiny_add_partial(nn.Module):
         self.compute = sc_compute
         self.legacy = legacy
         self.relu = relu
+        # training mode on the GPU with the LFSR kernels: run every conv + batch norm + pool +
+        # hardtanh block as one fused autograd node (same values; gradients to fp32 rounding)
+        self.fused_blocks = False
         if uniform:
             self.conv1.weight_org *= 2
             self.conv2.weight_org *= 2
@@ -58,7 +61,18 @@ class CONV_tiny_add_partial(nn.Module):
                     legacy=self.legacy, load_unit=self.load_unit[i], load_wait_w=self.load_wait[j],
                     load_wait_a=self.load_wait[i])
 
+    def _fusable(self, x):
+        return (self.fused_blocks and self.training and x.is_cuda and not self.legacy and self.generator == "lfsr"
+                and self.compute in ("1d_bin", "z_bin", "yz_bin"))
+
+    def _fused(self, conv, bn, x, i, j, **tail):
+        return utils_class.sc_conv_block(conv, bn, x, err=self.err[i], forward=self.compute,
+                                         z_unit=2 ** self.z_unit[i], load_unit=self.load_unit[i],
+                                         load_wait_w=self.load_wait[j], load_wait_a=self.load_wait[i], **tail)
+
     def _block(self, conv, bn, x, i):
+        if self._fusable(x):
+            return self._fused(conv, bn, x, i, i, relu=self.relu)
         x = bn(self._sc(conv, x, i))
         if self.relu:
             x = F.relu(x)
@@ -69,13 +83,16 @@ class CONV_tiny_add_partial(nn.Module):
         x = self._block(self.conv2, self.bn2, x, 1)
         x = self._block(self.conv3, self.bn3, x, 2)
         # the classifier layer takes the third layer's weight wait (network.py:186)
+        if self._fusable(x):
+            y = self._fused(self.fc1, self.bn4, x, 3, 2, relu=False, pool=False, hardtanh=False, quant7=False)
+            return y.view(-1, self.num_classes)
         x = self._sc(self.fc1, x, 3, wait_w_index=2)
         return self.bn4(x.view(-1, self.num_classes))
 
 
     # ---------------------------------------------------------------- fused inference path
     def train(self, mode=True):
-        self._fused = None  # parameters may change: drop the cached inference state
+        self._fused_state = None  # parameters may change: drop the cached inference state
         return super().train(mode)
 
     @torch.no_grad()
@@ -102,13 +119,13 @@ class CONV_tiny_add_partial(nn.Module):
             w_n, b_n = utils_class._fixed_affine(bn, None, bn.running_mean, bn.running_var)
             state.append(dict(w_shape=tuple(w.shape), kw=kw, wgt=capi.weight_streams(w, d),
                               w_n=w_n.float().contiguous(), b_n=b_n.float().contiguous()))
-        self._fused = state
+        self._fused_state = state
         self._fused_graph = None
 
     def _fused_eager(self, x):
         from . import capi
-        last = len(self._fused) - 1
-        for i, st in enumerate(self._fused):
+        last = len(self._fused_state) - 1
+        for i, st in enumerate(self._fused_state):
             d = capi.make_desc(x.shape, st["w_shape"], **st["kw"])
             counts = capi.conv2d_add_partial_from_streams(capi.act_streams(x, d), st["wgt"], d)
             L = st["kw"]["bit_length"]
@@ -129,7 +146,7 @@ class CONV_tiny_add_partial(nn.Module):
         if self.training:
             raise RuntimeError("forward_fused is the inference path: call model.eval() first")
         from . import utils_functional as uf
-        if getattr(self, "_fused", None) is None:
+        if getattr(self, "_fused_state", None) is None:
             self.prepare_fused()
         x = uf.quantize(x_in.detach().float(), prec=7).contiguous()
         if not graph:

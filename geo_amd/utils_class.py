@@ -77,3 +77,77 @@ class BatchNorm1d_fixed(nn.BatchNorm1d):
         w_n, b_n = _fixed_affine(self, x, mean, var)
         out.data = (x.data * w_n + b_n).to(out.dtype)
         return out
+
+
+class _SCConvBlock(torch.autograd.Function):
+    """One block of the reference's networks in training mode as a single autograd node:
+    SC convolution -> BatchNorm*_fixed on the batch statistics -> [relu] -> [AvgPool2d(2)] ->
+    [Hardtanh(0, 1)] -> [7-bit quantisation of the next layer's input] (network.py:165-170).
+    Forward: the HIP SC kernels, the batch statistics and the fixed-point affine exactly as
+    BatchNorm*_fixed computes them (utils_class.py:49-62), then one fused epilogue kernel.
+    Backward: the fused tail backward (gradient of an ordinary batch norm, masks from the
+    fixed-point values), then the HIP surrogate backward of the convolution."""
+
+    @staticmethod
+    def forward(ctx, activation, weight, gamma, beta, bn, conv_kw, relu, pool, hardtanh, quant7):
+        from . import capi
+        x = activation.detach().float().contiguous()
+        w = weight.detach().float().contiguous()
+        L = conv_kw["bit_length"]
+        counts = capi.conv2d_add_partial_forward(x, w, **conv_kw)
+        y = counts.float() / L
+        dims = (0, 2, 3)
+        mean, var = y.mean(dim=dims), y.var(dim=dims, unbiased=False)
+        # One launch for what BatchNorm*_fixed computes per channel (utils_class.py:52-62) and for what
+        # its F.batch_norm(x, running_mean, running_var, weight, bias, training=True) call
+        # (utils_class.py:49) does to the running statistics: that function's default momentum 0.1
+        # and, for the gradient, its default eps 1e-5; the batch counter is not touched.
+        w_n, b_n, invstd, bn.scale = capi.bn_fixed_affine(
+            mean, var, gamma.detach().float().contiguous() if gamma is not None else None,
+            beta.detach().float().contiguous() if beta is not None else None, bn.eps, y.numel() // y.shape[1],
+            bn.running_mean, bn.running_var)
+        act, _ = capi.layer_epilogue(counts, L, w_n, b_n, relu=relu, pool=pool, hardtanh=hardtanh, quant7=quant7)
+        ctx.save_for_backward(x, w, counts, w_n, b_n, mean, invstd,
+                              gamma.detach() if gamma is not None else torch.empty(0, device=x.device))
+        ctx.conv_kw, ctx.flags = conv_kw, (relu, pool, hardtanh)
+        ctx.has_gamma = gamma is not None
+        return act
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from . import capi
+        x, w, counts, w_n, b_n, mean, invstd, gamma = ctx.saved_tensors
+        relu, pool, hardtanh = ctx.flags
+        kw = ctx.conv_kw
+        gy, gg, gb = capi.layer_tail_backward(counts, grad_out.detach().float().contiguous(), kw["bit_length"], w_n,
+                                              b_n, mean, invstd, gamma if ctx.has_gamma else None, relu, pool,
+                                              hardtanh)
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        gx = gw = None
+        if need_x or need_w:
+            gx, gw = capi.conv2d_add_partial_backward(x, w, gy, kw["bit_length"], kw["padding"], need_x, need_w,
+                                                      accumulate=kw["accumulate"], z_unit=kw["z_unit"])
+        return (gx, gw, gg if ctx.has_gamma else None, gb if ctx.has_gamma else None, None, None, None, None, None,
+                None)
+
+
+def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_unit=8, load_wait_w=2, load_wait_a=2,
+                  prec=7, relu=False, pool=True, hardtanh=True, quant7=True):
+    """``hardtanh(pool(relu(bn(conv(input)))))`` of a ``Conv2d_Add_Partial`` and a
+    ``BatchNorm2d_fixed`` / ``BatchNorm1d_fixed`` in training mode, fused (LFSR generators, GPU
+    tensors).  Same in-place quantisation of ``input.data`` and ``conv.weight.data`` as
+    ``Conv2d_Add_Partial.forward`` (utils_class.py:32-33).  The output is already quantised to 7
+    bits (the next layer would do that to its input anyway) unless ``quant7=False``."""
+    if forward not in ("1d_bin", "z_bin", "yz_bin") or not input.is_cuda:
+        raise NotImplementedError("sc_conv_block: LFSR modes 1d_bin / z_bin / yz_bin on GPU tensors")
+    if tuple(conv.stride) != (1, 1):
+        raise NotImplementedError("the SC kernels compute stride 1 only")
+    input.data = utils_functional.quantize(input.data, prec=prec)
+    conv.weight.data = utils_functional.quantize(conv.weight_org, prec=prec)
+    mode = {"1d_bin": "y", "z_bin": "z", "yz_bin": "yz"}[forward]
+    kw = dict(bit_length=2 ** err, padding=(int(conv.padding[0]), int(conv.padding[1])),
+              total_width=utils_functional.prec_default, load_width=int(load_unit), load_wait_w=int(load_wait_w),
+              load_wait_a=int(load_wait_a if mode == "yz" else load_wait_w), accumulate=mode,
+              z_unit=max(1, min(int(z_unit), conv.weight.shape[1])))
+    gamma, beta = (bn.weight, bn.bias) if bn.affine else (None, None)
+    return _SCConvBlock.apply(input, conv.weight, gamma, beta, bn, kw, relu, pool, hardtanh, quant7)

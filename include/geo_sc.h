@@ -221,6 +221,42 @@ GEO_SC_API int geo_sc_layer_epilogue(const int32_t* counts, int n, int c, int w,
                                      uint8_t* q7_out, geo_sc_stream_t stream);
 
 /*
+ * Backward of the same tail in training mode, in which the reference's graph is
+ * y = count / L -> F.batch_norm(y, training=True) with its value replaced by y * w_n + b_n
+ * (utils_class.py:49-64) -> relu -> AvgPool2d(2) -> Hardtanh(0, 1) (network.py:165-170): the
+ * gradient of an ordinary batch norm on the batch statistics, with the relu / hardtanh masks taken
+ * from the fixed-point values that flowed forward; the quantisation passes the gradient through.
+ *   counts, w_n, b_n, flags   as given to geo_sc_layer_epilogue in the forward
+ *   grad_out                  fp32 (n, c, wo, ho): gradient with respect to the tail's output
+ *   mean, invstd              per channel: batch mean of y and 1 / sqrt(biased variance + eps)
+ *   gamma                     the batch norm's weight, or NULL for 1
+ *   grad_y                    fp32 (n, c, w, h): gradient with respect to y = count / L
+ *   grad_gamma, grad_beta     per channel, may be NULL
+ * Deterministic (fixed summation order).  Workspace: geo_sc_layer_tail_backward_workspace_size.
+ */
+GEO_SC_API int geo_sc_layer_tail_backward_workspace_size(int n, int c, int w, int h, size_t* bytes);
+GEO_SC_API int geo_sc_layer_tail_backward(const int32_t* counts, const float* grad_out, int n, int c, int w, int h,
+                                          int bit_length, const float* w_n, const float* b_n, const float* mean,
+                                          const float* invstd, const float* gamma, int flags, float* grad_y,
+                                          float* grad_gamma, float* grad_beta, void* workspace,
+                                          size_t workspace_bytes, geo_sc_stream_t stream);
+
+/*
+ * The per-channel fixed-point affine of BatchNorm2d_fixed / BatchNorm1d_fixed from channel statistics
+ * (utils_class.py:52-62, quantize_shift utils_functional.py:41-57) in one launch:
+ * w = gamma / sqrt(var + eps), b = beta - mean * gamma / sqrt(var + eps), both rounded to 8 bits under
+ * the shared power-of-two scale 2 ** ceil(log2(mean(w) * 3)).  gamma / beta may be NULL (1 / 0).
+ * Optional outputs: invstd = 1 / sqrt(var + eps_grad) for geo_sc_layer_tail_backward; the running
+ * statistics updated as F.batch_norm(training=True) does (momentum 0.1, variance unbiased by
+ * elements_per_channel / (elements_per_channel - 1)); scale (one float).  All pointers are device
+ * pointers to c floats.
+ */
+GEO_SC_API int geo_sc_bn_fixed_affine(const float* mean, const float* var, const float* gamma, const float* beta,
+                                      int c, float eps, float eps_grad, long long elements_per_channel,
+                                      float* running_mean, float* running_var, float* w_n, float* b_n, float* invstd,
+                                      float* scale, geo_sc_stream_t stream);
+
+/*
  * geo_sc_conv2d_add_partial_forward for activations given as the 7-bit integers k = round(x * 128)
  * that geo_sc_layer_epilogue emits (uint8 (n, c_in, w_in, h_in), k <= 127): the activation is
  * x = k / 128, exactly what the reference's layer computes from after its input quantisation

@@ -112,3 +112,82 @@ def test_training_step_bookkeeping():
     for master, p in zip(copies, model.parameters()):
         assert torch.equal(master.data, p.data)
     assert losses[-1] < losses[0] * 1.5
+
+
+@pytest.mark.parametrize("compute,relu", [("1d_bin", False), ("1d_bin", True), ("yz_bin", False)])
+def test_fused_training_blocks_match_module_chain(compute, relu):
+    """fused_blocks=True: one autograd node per conv + batch norm + pool + hardtanh block.  Logits
+    and running statistics equal the module-by-module forward; gradients agree to fp32 rounding."""
+    from geo_amd import network
+
+    def make():
+        torch.manual_seed(0)
+        m = network.CONV_tiny_add_partial(sc_compute=compute, relu=relu).cuda().train()
+        m.err = [6, 6, 6, 6]
+        with torch.no_grad():
+            for bn in (m.bn1, m.bn2, m.bn3, m.bn4):
+                bn.weight.uniform_(0.5, 1.5)
+                bn.bias.uniform_(-0.2, 0.4)
+        return m
+
+    ref, fused = make(), make()
+    fused.fused_blocks = True
+    g = torch.Generator().manual_seed(1)
+    x = torch.rand(32, 3, 32, 32, generator=g).cuda()
+    t = torch.randint(10, (32,), generator=g).cuda()
+    crit = torch.nn.CrossEntropyLoss()
+    out_r = ref(x.clone())
+    out_f = fused(x.clone())
+    assert torch.equal(out_r, out_f)
+    (crit(out_r, t) * 128).backward()
+    (crit(out_f, t) * 128).backward()
+    for (name, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        assert pf.grad is not None, name
+        err = (pf.grad - pr.grad).abs().max().item() / max(pr.grad.abs().max().item(), 1e-30)
+        assert err < 5e-5, (name, err)
+    for (name, br), (_, bf) in zip(ref.named_buffers(), fused.named_buffers()):
+        if br is None:
+            continue
+        if br.dtype.is_floating_point:
+            assert torch.allclose(br, bf, rtol=1e-5, atol=1e-7), name
+        else:
+            assert torch.equal(br, bf), name
+    # eval mode takes the module path again
+    fused.eval()
+    ref.eval()
+    with torch.no_grad():
+        assert torch.allclose(fused(x.clone()), ref(x.clone()), atol=1e-5)
+
+
+def test_tail_backward_matches_torch_autograd():
+    """geo_sc_layer_tail_backward against torch autograd over batch_norm(training) -> relu ->
+    avg_pool2d -> hardtanh with the forward values replaced by the fixed-point affine."""
+    from geo_amd import capi, utils_class
+    import torch.nn.functional as F
+    for (shape, relu, pool, hardtanh) in [((8, 6, 8, 6), False, True, True), ((4, 5, 7, 5), True, True, True),
+                                          ((16, 10, 1, 1), False, False, False), ((3, 4, 6, 6), True, False, True)]:
+        L = 64
+        g = torch.Generator().manual_seed(shape[0])
+        counts = torch.randint(-3 * L, 3 * L + 1, shape, generator=g, dtype=torch.int32).cuda()
+        bn = utils_class.BatchNorm2d_fixed(shape[1]).cuda().train()
+        with torch.no_grad():
+            bn.weight.uniform_(0.5, 1.5)
+            bn.bias.uniform_(-0.2, 0.6)
+        y = (counts.float() / L).requires_grad_(True)
+        v = bn(y)
+        if relu:
+            v = F.relu(v)
+        if pool:
+            v = F.avg_pool2d(v, 2)
+        if hardtanh:
+            v = F.hardtanh(v, 0, 1)
+        go = torch.randn(v.shape, generator=g).cuda()
+        v.backward(go)
+        yd = y.detach()
+        mean, var = yd.mean((0, 2, 3)), yd.var((0, 2, 3), unbiased=False)
+        w_n, b_n = utils_class._fixed_affine(bn, None, mean, var)
+        gy, gg, gb = capi.layer_tail_backward(counts, go, L, w_n, b_n, mean, torch.rsqrt(var + 1e-5), bn.weight.detach(),
+                                              relu, pool, hardtanh)
+        for got, ref in ((gy, y.grad), (gg, bn.weight.grad), (gb, bn.bias.grad)):
+            err = (got - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+            assert err < 2e-5, (shape, err)
