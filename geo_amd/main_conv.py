@@ -50,6 +50,9 @@ def build_parser():
     p.add_argument("--epochs", default=1000, type=int)
     p.add_argument("--iterations", default=None, type=int, help="batches per epoch (default: all)")
     p.add_argument("--synthetic_size", default=2048, type=int, help="images in the SYNTHETIC set")
+    p.add_argument("--fused", default=1, type=int,
+                   help="1: conv + batch norm + pool + hardtanh blocks as fused autograd nodes in training (same "
+                        "values as the module chain); 0: module by module")
     return p
 
 
@@ -104,6 +107,7 @@ def build_model(args):
     net.z_unit = digits(args.z_unit)
     net.load_unit = digits(args.load_unit)
     net.load_wait = digits(args.load_wait)
+    net.fused_blocks = args.fused == 1
     return net
 
 

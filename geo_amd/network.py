@@ -204,6 +204,9 @@ class VGG16_add_partial(nn.Module):
         self.compute = sc_compute
         self.legacy = legacy
         self.half_pool = half_pool
+        # training mode on the GPU with the LFSR kernels: every conv + batch norm + [pool] + hardtanh
+        # block as one fused autograd node (same values; gradients to fp32 rounding)
+        self.fused_blocks = False
         if min(self.err) < 4:
             uniform = True
         if uniform:
@@ -217,17 +220,32 @@ class VGG16_add_partial(nn.Module):
                     legacy=self.legacy, load_unit=self.load_unit[g], load_wait_w=self.load_wait[g],
                     load_wait_a=self.load_wait[g])
 
+    def _fused(self, conv, bn, x, g, err, **tail):
+        return utils_class.sc_conv_block(conv, bn, x, err=err, forward=self.compute, z_unit=2 ** self.z_unit[g],
+                                         load_unit=self.load_unit[g], load_wait_w=self.load_wait[g],
+                                         load_wait_a=self.load_wait[g], **tail)
+
     def forward(self, x):
         pool_offset = 1 if self.half_pool else 0
+        fuse = (self.fused_blocks and self.training and x.is_cuda and not self.legacy and self.generator == "lfsr"
+                and self.compute in ("1d_bin", "z_bin", "yz_bin"))
         for g, group in enumerate(self.GROUPS):
             for i in group:
                 last = i == group[-1]
                 err = max(self.err[g] - pool_offset, 5) if last else self.err[g]
-                x = getattr(self, f"bn{i}")(self._sc(getattr(self, f"conv{i}"), x, g, err))
+                conv, bn = getattr(self, f"conv{i}"), getattr(self, f"bn{i}")
+                if fuse:
+                    # a dropout follows the group's last layer: its input must stay unquantised
+                    x = self._fused(conv, bn, x, g, err, pool=last, quant7=not last)
+                    continue
+                x = bn(self._sc(conv, x, g, err))
                 if last:
                     x = self.pool(x)
                 x = self.tanh(x)
             x = getattr(self, f"drop{g + 1}")(x)
+        if fuse:
+            return self._fused(self.fc1, self.bnfc1, x, 5, self.err[5], pool=False, hardtanh=False,
+                               quant7=False).view(-1, 10)
         x = self._sc(self.fc1, x, 5, self.err[5]).view(-1, 10)
         return self.bnfc1(x)
 

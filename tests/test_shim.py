@@ -86,3 +86,29 @@ def test_vgg16_forward_backward():
     with torch.no_grad():
         a, b = net(x.clone()), net(x.clone())
     assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+def test_vgg16_fused_blocks_match_module_chain():
+    from geo_amd import network
+
+    def run(fused):
+        torch.manual_seed(0)
+        net = network.VGG16_add_partial().cuda().train()
+        net.err = [6, 6, 6, 6, 6, 6]
+        net.fused_blocks = fused
+        x = torch.rand(8, 3, 32, 32, generator=torch.Generator().manual_seed(1)).cuda()
+        torch.manual_seed(5)                      # same dropout masks in both runs
+        y = net(x)
+        y.square().mean().backward()
+        return y.detach(), {n: p.grad.clone() for n, p in net.named_parameters()}
+
+    y_ref, g_ref = run(False)
+    y_fused, g_fused = run(True)
+    assert torch.equal(y_ref, y_fused)
+    for name in g_ref:
+        scale = g_ref[name].abs().max().item()
+        if scale == 0.0:
+            assert g_fused[name].abs().max().item() == 0.0, name
+            continue
+        assert (g_fused[name] - g_ref[name]).abs().max().item() / scale < 1e-4, name
