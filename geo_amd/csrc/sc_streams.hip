@@ -202,6 +202,49 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __r
     }
 }
 
+// The same streams for kernels that are long in dim 3 (h_k >= 16, e.g. the SC-linear mapping with
+// h_k = 256): a workgroup takes one (c_out tile, member k) and 16 consecutive kernel rows, so that
+// the 16 rows of one output channel are one 64-byte run of w, shared by the workgroup's four waves
+// through the vector cache (4096 x 4096 linear layer: 1.46 GB fetched -> the 67 MB of the tensor).
+__global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float* __restrict__ w,
+                                                                    uint32_t* __restrict__ streams,
+                                                                    const uint32_t* __restrict__ tables, GenParams gp,
+                                                                    int c_out, int c_in, int w_k, int h_k, int n_cotile,
+                                                                    int v_chunks)
+{
+    extern __shared__ uint32_t lds[];
+    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    const uint32_t* posp1 = lds;
+    const uint32_t* thr = lds + gp.L;
+    const int k_or = c_in * w_k;
+    const size_t pack_stride = (size_t)h_k * k_or * n_cotile * 2 * kCoTile;
+    const float Lf = (float)gp.L, top = (float)(gp.L - 1);
+    const size_t n_blocks = (size_t)v_chunks * k_or * n_cotile;
+    const int co_l = threadIdx.x & 15, v_l = threadIdx.x >> 4;
+    for (size_t blk = blockIdx.x; blk < n_blocks; blk += gridDim.x) {
+        const int cot = (int)(blk % n_cotile);
+        const size_t r = blk / n_cotile;
+        const int k = (int)(r % k_or);
+        const int v = (int)(r / k_or) * 16 + v_l;
+        const int co = cot * kCoTile + co_l;
+        const int ci = k / w_k, u = k % w_k;
+        if (v >= h_k) continue;
+        int cp = 0, cn = 0;
+        if (co < c_out) {
+            const float t = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v] * Lf;
+            cp = (int)ceilf(fminf(fmaxf(t, 0.0f), top));
+            cn = (int)ceilf(-fminf(fmaxf(t, -top), 0.0f));
+        }
+        const int op = (int)posp1[(67 + k) % (gp.L - 1)];
+        const int on = (int)posp1[(37 + k) % (gp.L - 1)];
+        const size_t base = (((size_t)v * k_or + k) * n_cotile + cot) * (2 * kCoTile) + co_l;
+        for (int pk = 0; pk < gp.packs; pk++) {
+            streams[pk * pack_stride + base] = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
+            streams[pk * pack_stride + base + kCoTile] = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+        }
+    }
+}
+
 // Weight streams of the grouped accumulation modes, same line format, lines ordered as the
 // convolution kernel consumes them: [P][outer add group][inner add group][OR channel of the
 // group][w_k].  z_mode: inner group = input channel, OR channel = kernel row, seed index
@@ -493,6 +536,14 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
         hipLaunchKernelGGL(k_weight_streams_grouped, dim3(grid_for(padded)), dim3(kGenThreads), table_bytes(g.L), s,
                            w, streams, tables, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile,
                            g.mode == GEO_SC_ACC_Z ? 1 : 0, g.add_outer, g.add_inner, g.or_ch_total, g.or_ch_per_group);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
+    if (g.h_k >= 16) {
+        const int v_chunks = (g.h_k + 15) / 16;
+        const size_t n_blocks = (size_t)v_chunks * g.k_or * g.n_cotile;
+        hipLaunchKernelGGL(k_weight_streams_rows, dim3((unsigned)(n_blocks > 256 * 8 ? 256 * 8 : n_blocks)),
+                           dim3(kGenThreads), table_bytes(g.L), s, w, streams, tables, gp, g.c_out, g.c_in, g.w_k,
+                           g.h_k, g.n_cotile, v_chunks);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;

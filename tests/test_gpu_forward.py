@@ -283,3 +283,24 @@ def test_classifier_layers_match_oracle(capi, so, case, L):
     k = (x * 128).round().clamp(0, 127).to(torch.uint8)
     a = capi.conv2d_add_partial_forward_q7(k.cuda(), w.cuda(), L, pad)
     assert np.array_equal(a.cpu().numpy(), so.conv2d_add_partial((k.float() / 128).numpy(), w.numpy(), L, pad))
+
+
+@pytest.mark.parametrize("sx,sw,pad", [((4, 8, 1, 40), (21, 8, 1, 40), (0, 0)),     # linear mapping, 40 kernel rows
+                                       ((2, 3, 4, 24), (5, 3, 2, 17), (1, 0)),      # ragged last chunk of 16 rows
+                                       ((3, 2, 3, 16), (33, 2, 3, 16), (0, 0))])    # exactly one chunk, three c_out tiles
+@pytest.mark.parametrize("L", [16, 128])
+def test_long_kernels_use_the_row_chunked_weight_generator(capi, so, sx, sw, pad, L):
+    x, w = wl.make_inputs(sx, sw, "prescribed", seed=900)
+    w.view(-1)[::5] = 0.0
+    d = capi.make_desc(sx, sw, L, pad, 7, 2, 2, 2)
+    got = u32(capi.weight_streams(w.cuda(), d))                       # [P][H][K][cot][2][16]
+    wpos, wneg = so.weight_streams(w.numpy(), L, 7, 2, 2)             # [P][H][Cin][W][Cout]
+    P, H, Cin, W, Cout = wpos.shape
+    ncot = (Cout + 15) // 16
+    padc = ncot * 16 - Cout
+    exp = np.zeros((P, H, Cin * W, ncot, 2, 16), dtype=np.uint32)
+    exp[..., 0, :] = np.pad(wpos.reshape(P, H, Cin * W, Cout), ((0, 0),) * 3 + ((0, padc),)).reshape(P, H, Cin * W, ncot, 16)
+    exp[..., 1, :] = np.pad(wneg.reshape(P, H, Cin * W, Cout), ((0, 0),) * 3 + ((0, padc),)).reshape(P, H, Cin * W, ncot, 16)
+    assert np.array_equal(got, exp)
+    assert np.array_equal(gpu_forward(capi, x, w, L, pad, total_width=7, load_width=2, load_wait_w=2, load_wait_a=2),
+                          so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad, 7, 2, 2, 2))
