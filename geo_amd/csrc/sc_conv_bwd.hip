@@ -486,6 +486,140 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
     }
 }
 
+// Weight gradient of layers with small OR groups (K <= 16 members, 2 * c_out <= 128: first layers,
+// 3 -> 32 channels with 5 x 5 kernels has K = 15) when no input gradient is asked for.  Per tile of
+// 64 output positions the workgroup gathers the im2col columns into LDS, forms Z = col^T wcat with
+// MFMAs, turns it into E = g exp(-Z) in LDS and accumulates Gw += col E in MFMA accumulators that
+// stay live over all tiles of the workgroup; neither col nor E reach memory (at K = 15 they are
+// 80 MB and 335 MB per call).  A workgroup handles tiles s, s + S, ... of group g0 + blockIdx.y
+// and writes one partial sum part[g][s][k][j] for the common split reduction.
+constexpr int kSmallK = 16;
+constexpr int kSmallTile = 64;
+__global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__ x, const float* __restrict__ wcat,
+                                                       const float* __restrict__ gt, const int* __restrict__ base,
+                                                       const int* __restrict__ arow, const int* __restrict__ bcol,
+                                                       float* __restrict__ part, Groups G, int g0, int M, int w_in,
+                                                       int h_in, int c_out, int splits, size_t w_stride,
+                                                       size_t part_stride)
+{
+    __shared__ __attribute__((aligned(16))) float cs[kSmallK][kSmallTile + 4];  // col tile [k][m]
+    __shared__ __attribute__((aligned(16))) float ws[kSmallK][kLd];             // wcat [k][j], zero padded
+    __shared__ __attribute__((aligned(16))) float es[kSmallTile][kLd];          // E tile [m][j]
+    const int K = G.n_members, J = 2 * c_out;
+    const int g = g0 + blockIdx.y;
+    // the wave index as a scalar: everything derived from it (member indices, which MFMA blocks
+    // exist) stays wave-uniform, so no divergent branches are generated around loads and MFMAs
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int i0 = (wave >> 1) * 32, j0 = (wave & 1) * 64;  // first product: this wave's 32 x 64 corner
+    const int jb = (J + 31) / 32;                           // 32-wide column blocks that hold results
+
+    // wcat of this group, once
+    const float* wg = wcat + (size_t)blockIdx.y * w_stride;
+    for (int e = threadIdx.x; e < kSmallK * kTile; e += 256) {
+        const int k = e / kTile, j = e - k * kTile;
+        ws[k][j] = (k < K && j < J) ? wg[(size_t)k * J + j] : 0.0f;
+    }
+    floatx16 gw_acc[4];
+#pragma unroll
+    for (int y = 0; y < 4; y++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) gw_acc[y][r] = 0.0f;
+
+    const int n_tiles = (M + kSmallTile - 1) / kSmallTile;
+    for (int tile = blockIdx.x; tile < n_tiles; tile += splits) {
+        const int m0 = tile * kSmallTile;
+        __syncthreads();  // the previous tile's second product has read cs and es
+        {
+            // im2col gather: thread -> position m0 + (t & 63), members wave, wave + 4, wave + 8, wave + 12.
+            // Loads without branches: lanes outside the image read x[0] and are zeroed by a select.
+            const int ml = threadIdx.x & 63;
+            const bool m_ok = m0 + ml < M;
+            const int mc = m_ok ? m0 + ml : 0;
+            const int r0 = arow[mc], c0 = bcol[mc], b0 = base[mc];
+            float vals[4];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int k = wave + 4 * q4;
+                const Member mb = member_of(G, g, k < K ? k : 0);
+                const int rr = r0 + mb.u, cc = c0 + mb.v;
+                const bool ok = m_ok && k < K && mb.ok && cc >= 0 && cc < h_in && rr >= 0 && rr < w_in;
+                const float v = x[ok ? b0 + (mb.ci * w_in + mb.u) * h_in + mb.v : 0];
+                vals[q4] = ok ? v : 0.0f;
+            }
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) cs[wave + 4 * q4][ml] = vals[q4];
+        }
+        __syncthreads();
+        // Z[m][j] = sum_k col[k][m] * wcat[k][j]
+        floatx16 z[2];
+#pragma unroll
+        for (int y = 0; y < 2; y++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) z[y][r] = 0.0f;
+        const bool y0 = j0 < J, y1 = j0 + 32 < J;  // which of this wave's two column blocks hold results
+#pragma unroll
+        for (int kk = 0; kk < kSmallK; kk += 2) {
+            const float a = cs[kk + lk][i0 + l32];
+            const float b0 = ws[kk + lk][j0 + l32], b1 = ws[kk + lk][j0 + 32 + l32];
+            if (y0) z[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, z[0], 0, 0, 0);
+            if (y1) z[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, z[1], 0, 0, 0);
+        }
+        // E[m][j] = g[m][co] * exp(-Z), zero outside the problem; all loads of g first, no branches
+#pragma unroll
+        for (int y = 0; y < 2; y++) {
+            const int j = j0 + 32 * y + l32;
+            const int co = j >= c_out ? j - c_out : j;
+            const bool j_ok = j < J;
+            if (y == 0 ? y0 : y1) {  // wave-uniform: column blocks outside the result hold zeros
+                float gv[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = m0 + i0 + 8 * (r >> 2) + 4 * lk + (r & 3);
+                    gv[r] = gt[(m < M && j_ok) ? (long long)m * c_out + co : 0];
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int i = i0 + 8 * (r >> 2) + 4 * lk + (r & 3);
+                    es[i][j] = (m0 + i < M && j_ok) ? gv[r] * expf(-z[y][r]) : 0.0f;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) es[i0 + 8 * (r >> 2) + 4 * lk + (r & 3)][j] = 0.0f;
+            }
+        }
+        __syncthreads();
+        // Gw[k][j] += sum_m col[k][m] * E[m][j]: wave w takes positions 16 w .. 16 w + 15 of the tile
+        const int mw = wave * 16;
+#pragma unroll
+        for (int mm = 0; mm < 16; mm += 2) {
+            const float a = l32 < kSmallK ? cs[l32][mw + mm + lk] : 0.0f;
+#pragma unroll
+            for (int y = 0; y < 4; y++)
+                if (y < jb) {
+                    const float b = es[mw + mm + lk][32 * y + l32];
+                    gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, gw_acc[y], 0, 0, 0);
+                }
+        }
+    }
+    // sum the four waves' accumulators in wave order through LDS (es is free after a barrier)
+    __syncthreads();
+    float (*red)[kSmallK][kLd] = reinterpret_cast<float (*)[kSmallK][kLd]>(&es[0][0]);  // [4][16][kLd] = 64 rows of es
+#pragma unroll
+    for (int y = 0; y < 4; y++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int k = 8 * (r >> 2) + 4 * lk + (r & 3);
+            if (k < kSmallK) red[wave][k][32 * y + l32] = gw_acc[y][r];
+        }
+    __syncthreads();
+    float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)blockIdx.x * K * J;
+    for (int e = threadIdx.x; e < K * J; e += 256) {
+        const int k = e / J, j = e - k * J;
+        pg[e] = ((red[0][k][j] + red[1][k][j]) + red[2][k][j]) + red[3][k][j];
+    }
+}
+
 int grid1d(long long total)
 {
     long long blocks = (total + 255) / 256;
@@ -515,6 +649,7 @@ struct BwdLayout {
     long long m_total;
     int splits, m_per_split;
     Groups G;
+    bool small_k;        // OR groups of at most 16 members and 2 * c_out <= 128: fused weight-gradient kernel
     int rows_per_chunk;  // add groups processed by one round of launches
     size_t col_v, e_v, part_v, w_v;  // floats per add group of each scratch array
     size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, off_gt, bytes;
@@ -543,6 +678,7 @@ BwdLayout bwd_layout(const Geometry& g)
         b.G.n_members = g.k_or;
     }
     const int K = b.G.n_members;
+    b.small_k = K <= kSmallK && 2 * g.c_out <= kTile;
     // split the m-reduction of the weight gradient so that the grid covers the GPU
     const long long tiles = (long long)((K + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
     long long want = (1024 + tiles - 1) / tiles;
@@ -614,6 +750,24 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
                            g.c_out, npos);
     }
     int rc;
+    if (!gx && gw && L.small_k) {
+        // first-layer case: fused im2col + both products, no col / E scratch traffic
+        for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
+            const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
+            int wb = grid1d((long long)K * g.c_out);
+            hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
+                               g.c_out, G, L.w_v);
+            // about eight workgroups per CU in all, each looping over its share of the tiles
+            int active = 2048 / nv;
+            if (active > L.splits) active = L.splits;
+            if (active < 1) active = 1;
+            hipLaunchKernelGGL(k_wgrad_small_k, dim3(active, nv), dim3(256), 0, s, x, wcat, gt, pos_base, pos_arow,
+                               pos_bcol, part, G, v0, M, g.w_in, g.h_in, g.c_out, active, L.w_v, L.part_v);
+            hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
+                               active, g.c_out, G, L.part_v);
+        }
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
     for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
         const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
         hipLaunchKernelGGL(k_im2col_rows,

@@ -51,11 +51,12 @@ def test_backward_matches_float64_oracle(capi, shape_x, shape_w, pad, mode, scal
     assert gx.shape == x.shape and gw.shape == w.shape
     assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
     assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
-    # skipping one output leaves the other unchanged
+    # skipping one output leaves the other unchanged (a weight gradient asked for alone may take the
+    # fused kernel for small OR groups: same value up to the summation order)
     gx2, none = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_w=False)
     none2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_x=False)
     assert none is None and none2 is None
-    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)
+    assert torch.equal(gx2, gx) and rel_err(gw2, gw) <= 1e-6 and rel_err(gw2, rw) <= RTOL
 
 
 def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
@@ -128,3 +129,32 @@ def test_layer_module_quantises_in_place_and_trains(capi):
     y.sum().backward()
     assert layer.weight.grad is not None and torch.isfinite(layer.weight.grad).all()
     assert "weight_org" in layer.state_dict()
+
+
+@pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu", [
+    ((6, 3, 12, 12), (32, 3, 5, 5), (2, 2), "y", 1),      # first layer of the 4-layer CNN: K = 15, 2*c_out = 64
+    ((5, 3, 9, 7), (64, 3, 3, 3), (1, 1), "y", 1),        # first layer of VGG-16: K = 9, 2*c_out = 128
+    ((3, 2, 7, 8), (7, 2, 3, 2), (1, 0), "y", 1),         # partial c_out block, 70 positions: ragged tile
+    ((2, 16, 6, 6), (10, 16, 1, 3), (0, 1), "y", 1),      # K = 16 exactly
+    ((4, 5, 8, 8), (12, 5, 3, 3), (1, 1), "z", 1),        # z mode: groups of 9 members
+    ((4, 7, 8, 8), (12, 7, 3, 3), (1, 1), "yz", 3),       # yz mode, ragged last channel block
+])
+def test_weight_gradient_of_small_or_groups(capi, shape_x, shape_w, pad, mode, zu):
+    """No input gradient requested, OR groups of at most 16 members, at most 64 output channels:
+    the fused weight-gradient kernel.  Same answer as the general path and as the float64 oracle."""
+    from oracle import surrogate
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_x[1] + shape_w[0])
+    w = (w * 3).contiguous()
+    w.view(-1)[::7] = 0.0
+    d = capi.make_desc(x.shape, w.shape, 64, pad)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(1))
+    none, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False,
+                                                accumulate=mode, z_unit=zu)
+    assert none is None
+    _, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
+    assert rel_err(gw, rw) <= RTOL, rel_err(gw, rw)
+    _, gw_general = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, accumulate=mode, z_unit=zu)
+    assert rel_err(gw, gw_general) <= RTOL
+    _, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False,
+                                              accumulate=mode, z_unit=zu)
+    assert torch.equal(gw, gw2)   # deterministic

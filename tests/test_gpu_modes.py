@@ -141,7 +141,7 @@ def test_backward_modes_match_float64_oracle(capi, case, mode, zu):
     none2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_x=False,
                                                   accumulate=mode, z_unit=zu)
     assert none is None and none2 is None
-    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)
+    assert torch.equal(gx2, gx) and rel_err(gw2, gw) <= 1e-6 and rel_err(gw2, rw) <= RTOL
 
 
 @pytest.mark.parametrize("forward,kw", [("z_bin", {}), ("yz_bin", {"z_unit": 4, "load_wait_a": 3}),
