@@ -495,6 +495,9 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
 // and writes one partial sum part[g][s][k][j] for the common split reduction.
 constexpr int kSmallK = 16;
 constexpr int kSmallTile = 64;
+// JB: 32-wide column blocks of the result (ceil(2 * c_out / 32), 1..4), a template parameter so
+// that the MFMAs on the long-lived accumulators are unconditional.
+template <int JB>
 __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__ x, const float* __restrict__ wcat,
                                                        const float* __restrict__ gt, const int* __restrict__ base,
                                                        const int* __restrict__ arow, const int* __restrict__ bcol,
@@ -502,27 +505,29 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
                                                        int h_in, int c_out, int splits, size_t w_stride,
                                                        size_t part_stride)
 {
+    constexpr int NB1 = JB <= 2 ? 1 : 2;  // column blocks of the first product per wave
     __shared__ __attribute__((aligned(16))) float cs[kSmallK][kSmallTile + 4];  // col tile [k][m]
-    __shared__ __attribute__((aligned(16))) float ws[kSmallK][kLd];             // wcat [k][j], zero padded
-    __shared__ __attribute__((aligned(16))) float es[kSmallTile][kLd];          // E tile [m][j]
+    __shared__ __attribute__((aligned(16))) float ws[kSmallK][JB * 32 + 4];      // wcat [k][j], zero padded
+    __shared__ __attribute__((aligned(16))) float es[kSmallTile][JB * 32 + 4];   // E tile [m][j]
     const int K = G.n_members, J = 2 * c_out;
     const int g = g0 + blockIdx.y;
     // the wave index as a scalar: everything derived from it (member indices, which MFMA blocks
     // exist) stays wave-uniform, so no divergent branches are generated around loads and MFMAs
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int l32 = lane & 31, lk = lane >> 5;
-    const int i0 = (wave >> 1) * 32, j0 = (wave & 1) * 64;  // first product: this wave's 32 x 64 corner
-    const int jb = (J + 31) / 32;                           // 32-wide column blocks that hold results
+    // first product: 64 positions x JB column blocks; wave w takes row half w / 2 and column
+    // block(s) w % 2 (JB <= 2) or 2 (w % 2), 2 (w % 2) + 1 (JB > 2)
+    const int i0 = (wave >> 1) * 32;
+    const int cb0 = NB1 == 1 ? (wave & 1) : (wave & 1) * 2;
 
-    // wcat of this group, once
     const float* wg = wcat + (size_t)blockIdx.y * w_stride;
-    for (int e = threadIdx.x; e < kSmallK * kTile; e += 256) {
-        const int k = e / kTile, j = e - k * kTile;
+    for (int e = threadIdx.x; e < kSmallK * JB * 32; e += 256) {
+        const int k = e / (JB * 32), j = e - k * (JB * 32);
         ws[k][j] = (k < K && j < J) ? wg[(size_t)k * J + j] : 0.0f;
     }
-    floatx16 gw_acc[4];
+    floatx16 gw_acc[JB];
 #pragma unroll
-    for (int y = 0; y < 4; y++)
+    for (int y = 0; y < JB; y++)
 #pragma unroll
         for (int r = 0; r < 16; r++) gw_acc[y][r] = 0.0f;
 
@@ -551,27 +556,21 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
             for (int q4 = 0; q4 < 4; q4++) cs[wave + 4 * q4][ml] = vals[q4];
         }
         __syncthreads();
-        // Z[m][j] = sum_k col[k][m] * wcat[k][j]
-        floatx16 z[2];
 #pragma unroll
-        for (int y = 0; y < 2; y++)
+        for (int y = 0; y < NB1; y++) {
+            const int cb = cb0 + y;
+            if (cb < JB) {  // wave-uniform
+                // Z[m][j] = sum_k col[k][m] * wcat[k][j] for one 32 x 32 block
+                floatx16 z;
 #pragma unroll
-            for (int r = 0; r < 16; r++) z[y][r] = 0.0f;
-        const bool y0 = j0 < J, y1 = j0 + 32 < J;  // which of this wave's two column blocks hold results
+                for (int r = 0; r < 16; r++) z[r] = 0.0f;
 #pragma unroll
-        for (int kk = 0; kk < kSmallK; kk += 2) {
-            const float a = cs[kk + lk][i0 + l32];
-            const float b0 = ws[kk + lk][j0 + l32], b1 = ws[kk + lk][j0 + 32 + l32];
-            if (y0) z[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, z[0], 0, 0, 0);
-            if (y1) z[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, z[1], 0, 0, 0);
-        }
-        // E[m][j] = g[m][co] * exp(-Z), zero outside the problem; all loads of g first, no branches
-#pragma unroll
-        for (int y = 0; y < 2; y++) {
-            const int j = j0 + 32 * y + l32;
-            const int co = j >= c_out ? j - c_out : j;
-            const bool j_ok = j < J;
-            if (y == 0 ? y0 : y1) {  // wave-uniform: column blocks outside the result hold zeros
+                for (int kk = 0; kk < kSmallK; kk += 2)
+                    z = __builtin_amdgcn_mfma_f32_32x32x2f32(cs[kk + lk][i0 + l32], ws[kk + lk][cb * 32 + l32], z, 0, 0, 0);
+                // E[m][j] = g[m][co] * exp(-Z), zero outside the problem; loads of g first, no branches
+                const int j = cb * 32 + l32;
+                const int co = j >= c_out ? j - c_out : j;
+                const bool j_ok = j < J;
                 float gv[16];
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
@@ -581,11 +580,8 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int i = i0 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                    es[i][j] = (m0 + i < M && j_ok) ? gv[r] * expf(-z[y][r]) : 0.0f;
+                    es[i][j] = (m0 + i < M && j_ok) ? gv[r] * expf(-z[r]) : 0.0f;
                 }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; r++) es[i0 + 8 * (r >> 2) + 4 * lk + (r & 3)][j] = 0.0f;
             }
         }
         __syncthreads();
@@ -595,18 +591,15 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
         for (int mm = 0; mm < 16; mm += 2) {
             const float a = l32 < kSmallK ? cs[l32][mw + mm + lk] : 0.0f;
 #pragma unroll
-            for (int y = 0; y < 4; y++)
-                if (y < jb) {
-                    const float b = es[mw + mm + lk][32 * y + l32];
-                    gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, gw_acc[y], 0, 0, 0);
-                }
+            for (int y = 0; y < JB; y++)
+                gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, es[mw + mm + lk][32 * y + l32], gw_acc[y], 0, 0, 0);
         }
     }
-    // sum the four waves' accumulators in wave order through LDS (es is free after a barrier)
+    // sum the four waves' accumulators in wave order through LDS (cs/es are free after a barrier)
     __syncthreads();
-    float (*red)[kSmallK][kLd] = reinterpret_cast<float (*)[kSmallK][kLd]>(&es[0][0]);  // [4][16][kLd] = 64 rows of es
+    float (*red)[kSmallK][JB * 32 + 4] = reinterpret_cast<float (*)[kSmallK][JB * 32 + 4]>(&es[0][0]);  // 4 x 16 rows of es
 #pragma unroll
-    for (int y = 0; y < 4; y++)
+    for (int y = 0; y < JB; y++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int k = 8 * (r >> 2) + 4 * lk + (r & 3);
@@ -761,8 +754,17 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             int active = 2048 / nv;
             if (active > L.splits) active = L.splits;
             if (active < 1) active = 1;
-            hipLaunchKernelGGL(k_wgrad_small_k, dim3(active, nv), dim3(256), 0, s, x, wcat, gt, pos_base, pos_arow,
-                               pos_bcol, part, G, v0, M, g.w_in, g.h_in, g.c_out, active, L.w_v, L.part_v);
+            const dim3 grid(active, nv);
+#define GEO_SC_SMALL_K(JB)                                                                                          \
+    hipLaunchKernelGGL(k_wgrad_small_k<JB>, grid, dim3(256), 0, s, x, wcat, gt, pos_base, pos_arow, pos_bcol, part, G, \
+                       v0, M, g.w_in, g.h_in, g.c_out, active, L.w_v, L.part_v)
+            switch ((J + 31) / 32) {
+            case 1: GEO_SC_SMALL_K(1); break;
+            case 2: GEO_SC_SMALL_K(2); break;
+            case 3: GEO_SC_SMALL_K(3); break;
+            default: GEO_SC_SMALL_K(4); break;
+            }
+#undef GEO_SC_SMALL_K
             hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
                                active, g.c_out, G, L.part_v);
         }
