@@ -136,6 +136,26 @@ struct Stager {
     }
 };
 
+// One K-chunk of MFMAs on the first NX x NY of a wave's 2 x 2 blocks of 32 x 32.
+// v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32].
+template <int NX, int NY>
+__device__ __forceinline__ void mma_chunk(floatx16 (&acc)[2][2], const float (*as)[kLd], const float (*bs)[kLd], int wi,
+                                          int wj, int l32, int lk)
+{
+#pragma unroll
+    for (int kk = 0; kk < kChunk; kk += 2) {
+        float a[2], b[2];
+#pragma unroll
+        for (int x = 0; x < NX; x++) a[x] = as[kk + lk][wi + 32 * x + l32];
+#pragma unroll
+        for (int y = 0; y < NY; y++) b[y] = bs[kk + lk][wj + 32 * y + l32];
+#pragma unroll
+        for (int x = 0; x < NX; x++)
+#pragma unroll
+            for (int y = 0; y < NY; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x], b[y], acc[x][y], 0, 0, 0);
+    }
+}
+
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC>
 __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
 {
@@ -148,9 +168,10 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wave's 64x64 corner in the tile
     const int l32 = lane & 31, lk = lane >> 5;
-    // which of this wave's four 32 x 32 blocks lie inside the result
+    // which of this wave's four 32 x 32 blocks lie inside the result: 2 * (second row block) +
+    // (second column block), or -1 when even the first block lies outside
     const bool x0 = i0 + wi < q.I, x1 = i0 + wi + 32 < q.I, y0 = j0 + wj < q.J, y1 = j0 + wj + 32 < q.J;
-    const bool full = x1 && y1;
+    const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -179,29 +200,14 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
             sa.fetch(ra, k_end - k0 - kChunk);
             sb.fetch(rb, k_end - k0 - kChunk);
         }
-        // v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32]
-        if (full) {
-#pragma unroll
-            for (int kk = 0; kk < kChunk; kk += 2) {
-                const float a0 = as[buf][kk + lk][wi + l32], a1 = as[buf][kk + lk][wi + 32 + l32];
-                const float b0 = bs[buf][kk + lk][wj + l32], b1 = bs[buf][kk + lk][wj + 32 + l32];
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-            }
-        } else {
-            // edge tiles and narrow operands (few output channels, small OR groups): only the
-            // 32 x 32 blocks that hold results are computed
-#pragma unroll
-            for (int kk = 0; kk < kChunk; kk += 2) {
-                const float a0 = as[buf][kk + lk][wi + l32], a1 = as[buf][kk + lk][wi + 32 + l32];
-                const float b0 = bs[buf][kk + lk][wj + l32], b1 = bs[buf][kk + lk][wj + 32 + l32];
-                if (x0 && y0) acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-                if (x0 && y1) acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-                if (x1 && y0) acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-                if (x1 && y1) acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
-            }
+        // only the 32 x 32 blocks that hold results are computed (edge tiles, narrow operands); the
+        // choice is wave-uniform and each variant issues its MFMAs unconditionally
+        switch (blocks_xy) {
+        case 3: mma_chunk<2, 2>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
+        case 2: mma_chunk<2, 1>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
+        case 1: mma_chunk<1, 2>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
+        case 0: mma_chunk<1, 1>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
+        default: break;  // this wave's corner lies outside the result
         }
         if (more) {
             // the other buffer was last read one trip ago, before that trip's barrier
