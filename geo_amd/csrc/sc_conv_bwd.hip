@@ -136,48 +136,23 @@ struct Stager {
     }
 };
 
-// One K-chunk of MFMAs on the first NX x NY of a wave's 2 x 2 blocks of 32 x 32.
+// The K loop and the epilogue of one wave that owns the first NX x NY of its 2 x 2 blocks of
+// 32 x 32 (edge tiles and narrow operands leave blocks without results; NX = 0: none, the wave only
+// stages).  A function of its own per (NX, NY), entered through a wave-uniform switch: the
+// accumulators then live in one variant from zeroing to store and every MFMA is unconditional.
+// Conditions on single blocks inside one loop make the compiler copy all accumulators between
+// register classes on every trip.
 // v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32].
-template <int NX, int NY>
-__device__ __forceinline__ void mma_chunk(floatx16 (&acc)[2][2], const float (*as)[kLd], const float (*bs)[kLd], int wi,
-                                          int wj, int l32, int lk)
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC, int NX, int NY>
+__device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChunk][kLd], float (*bs)[kChunk][kLd], int i0,
+                                          int j0, int batch, int split, int k_begin, int k_end, int wi, int wj, int l32,
+                                          int lk)
 {
+    floatx16 acc[NX ? NX : 1][NY ? NY : 1];
 #pragma unroll
-    for (int kk = 0; kk < kChunk; kk += 2) {
-        float a[2], b[2];
+    for (int x = 0; x < NX; x++)
 #pragma unroll
-        for (int x = 0; x < NX; x++) a[x] = as[kk + lk][wi + 32 * x + l32];
-#pragma unroll
-        for (int y = 0; y < NY; y++) b[y] = bs[kk + lk][wj + 32 * y + l32];
-#pragma unroll
-        for (int x = 0; x < NX; x++)
-#pragma unroll
-            for (int y = 0; y < NY; y++) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x], b[y], acc[x][y], 0, 0, 0);
-    }
-}
-
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC>
-__global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
-{
-    __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
-    __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
-    const int i0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile;
-    const int batch = blockIdx.z / q.splits, split = blockIdx.z - batch * q.splits;
-    const int k_begin = split * q.k_per_split;
-    const int k_end = min(q.K, k_begin + q.k_per_split);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wave's 64x64 corner in the tile
-    const int l32 = lane & 31, lk = lane >> 5;
-    // which of this wave's four 32 x 32 blocks lie inside the result: 2 * (second row block) +
-    // (second column block), or -1 when even the first block lies outside
-    const bool x0 = i0 + wi < q.I, x1 = i0 + wi + 32 < q.I, y0 = j0 + wj < q.J, y1 = j0 + wj + 32 < q.J;
-    const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
-
-    floatx16 acc[2][2];
-#pragma unroll
-    for (int x = 0; x < 2; x++)
-#pragma unroll
-        for (int y = 0; y < 2; y++)
+        for (int y = 0; y < NY; y++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
 
@@ -200,14 +175,18 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
             sa.fetch(ra, k_end - k0 - kChunk);
             sb.fetch(rb, k_end - k0 - kChunk);
         }
-        // only the 32 x 32 blocks that hold results are computed (edge tiles, narrow operands); the
-        // choice is wave-uniform and each variant issues its MFMAs unconditionally
-        switch (blocks_xy) {
-        case 3: mma_chunk<2, 2>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
-        case 2: mma_chunk<2, 1>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
-        case 1: mma_chunk<1, 2>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
-        case 0: mma_chunk<1, 1>(acc, as[buf], bs[buf], wi, wj, l32, lk); break;
-        default: break;  // this wave's corner lies outside the result
+#pragma unroll
+        for (int kk = 0; kk < kChunk; kk += 2) {
+            float a[NX ? NX : 1], b[NY ? NY : 1];
+#pragma unroll
+            for (int x = 0; x < NX; x++) a[x] = as[buf][kk + lk][wi + 32 * x + l32];
+#pragma unroll
+            for (int y = 0; y < NY; y++) b[y] = bs[buf][kk + lk][wj + 32 * y + l32];
+#pragma unroll
+            for (int x = 0; x < NX; x++)
+#pragma unroll
+                for (int y = 0; y < NY; y++)
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x], b[y], acc[x][y], 0, 0, 0);
         }
         if (more) {
             // the other buffer was last read one trip ago, before that trip's barrier
@@ -221,9 +200,9 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
     // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
     float* c = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
 #pragma unroll
-    for (int x = 0; x < 2; x++)
+    for (int x = 0; x < NX; x++)
 #pragma unroll
-        for (int y = 0; y < 2; y++) {
+        for (int y = 0; y < NY; y++) {
             const int j = j0 + wj + y * 32 + l32;
             if (j >= q.J) continue;
 #pragma unroll
@@ -238,6 +217,36 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
                 c[(long long)i * q.ldc + j] = v;
             }
         }
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC>
+__global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
+{
+    __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
+    __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
+    const int i0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile;
+    const int batch = blockIdx.z / q.splits, split = blockIdx.z - batch * q.splits;
+    const int k_begin = split * q.k_per_split;
+    const int k_end = min(q.K, k_begin + q.k_per_split);
+    // the wave index through readfirstlane: the compiler then knows that everything derived from it
+    // (tile corner, block choice) is uniform and branches on it with scalar instructions
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wave's 64x64 corner in the tile
+    const int l32 = lane & 31, lk = lane >> 5;
+    // which of this wave's four 32 x 32 blocks lie inside the result
+    const bool x0 = i0 + wi < q.I, x1 = i0 + wi + 32 < q.I, y0 = j0 + wj < q.J, y1 = j0 + wj + 32 < q.J;
+    const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
+#define GEO_SC_GEMM_WAVE(NX, NY)                                                                                        \
+    gemm_wave<A_KMAJOR, B_KMAJOR, EPI, VEC, NX, NY>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk)
+    // every variant runs the same staging and the same number of barriers
+    switch (blocks_xy) {
+    case 3: GEO_SC_GEMM_WAVE(2, 2); break;
+    case 2: GEO_SC_GEMM_WAVE(2, 1); break;
+    case 1: GEO_SC_GEMM_WAVE(1, 2); break;
+    case 0: GEO_SC_GEMM_WAVE(1, 1); break;
+    default: GEO_SC_GEMM_WAVE(0, 0); break;
+    }
+#undef GEO_SC_GEMM_WAVE
 }
 
 // gt[n*npos + pos][co] = g[n][co][pos]: the upstream gradient with the channel innermost, so that the
