@@ -75,6 +75,10 @@ struct Stager {
     long long ld;
     int kk0, ii;         // first k (inside the chunk) and first i (inside the tile) of this thread
     bool i_ok;
+    // which elements of the last fetch lie inside the operand: per float4 after a vector fetch
+    // (vec_), else bit c of ok for element c
+    bool vec_, ok0_, ok1_;
+    unsigned ok;
 
     // element c (0..7) of this thread sits at (k, i) = (kk0 + kdelta(c), ii + idelta(c))
     static __device__ __forceinline__ int kdelta(int c) { return KMAJOR ? (VEC ? (c >> 2) * 8 : c * 2) : c; }
@@ -101,7 +105,9 @@ struct Stager {
         }
         i_ok = i0 + ii < I;
     }
-    // k_left = k_end - k0 of the chunk being fetched
+    // k_left = k_end - k0 of the chunk being fetched.  Only the loads are issued here; lanes outside
+    // the operand are zeroed in commit(), after the MFMAs of the chunk in flight, so that nothing
+    // waits for the loads before those MFMAs.
     __device__ __forceinline__ void fetch(float (&r)[8], int k_left)
     {
         if (VEC && (KMAJOR || k_left >= kChunk)) {
@@ -111,21 +117,33 @@ struct Stager {
             const float* q0 = ok0 ? p : dummy;
             const float* q1 = ok1 ? p + (KMAJOR ? 8 * ld : 4) : dummy;
             const float4 v0 = *(const float4*)q0, v1 = *(const float4*)q1;
-            r[0] = ok0 ? v0.x : 0.0f; r[1] = ok0 ? v0.y : 0.0f; r[2] = ok0 ? v0.z : 0.0f; r[3] = ok0 ? v0.w : 0.0f;
-            r[4] = ok1 ? v1.x : 0.0f; r[5] = ok1 ? v1.y : 0.0f; r[6] = ok1 ? v1.z : 0.0f; r[7] = ok1 ? v1.w : 0.0f;
+            r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+            r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+            ok0_ = ok0;
+            ok1_ = ok1;
+            vec_ = true;
         } else {
+            ok = 0;
+            vec_ = false;
 #pragma unroll
             for (int c = 0; c < 8; c++) {
-                const bool ok = i_ok && kk0 + kdelta(c) < k_left;
-                const float* qq = ok ? p + (KMAJOR ? (long long)kdelta(c) * ld + idelta(c) : (long long)c) : dummy;
-                const float v = *qq;
-                r[c] = ok ? v : 0.0f;
+                const bool okc = i_ok && kk0 + kdelta(c) < k_left;
+                const float* qq = okc ? p + (KMAJOR ? (long long)kdelta(c) * ld + idelta(c) : (long long)c) : dummy;
+                r[c] = *qq;
+                ok |= okc ? 1u << c : 0u;
             }
         }
         p += KMAJOR ? (long long)kChunk * ld : (long long)kChunk;
     }
-    __device__ __forceinline__ void commit(float (*s)[kLd], const float (&r)[8]) const
+    __device__ __forceinline__ void commit(float (*s)[kLd], float (&r)[8]) const
     {
+        if (VEC && vec_) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = (c < 4 ? ok0_ : ok1_) ? r[c] : 0.0f;
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = (ok >> c & 1u) ? r[c] : 0.0f;
+        }
         if (KMAJOR && VEC) {
             *(float4*)&s[kk0][ii] = make_float4(r[0], r[1], r[2], r[3]);
             *(float4*)&s[kk0 + 8][ii] = make_float4(r[4], r[5], r[6], r[7]);
@@ -220,7 +238,8 @@ __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChun
 }
 
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC>
-__global__ __launch_bounds__(256) void k_gemm_f32(GemmParams q)
+// four waves per SIMD (at most 128 registers: four workgroups per CU)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_gemm_f32(GemmParams q)
 {
     __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
