@@ -34,6 +34,12 @@ namespace geo_sc {
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// exp(-z) of the surrogate's OR term, z >= 0: one multiply and v_exp_f32 (about 1 ulp of the result plus
+// |z| 2^-24 from the rounded argument), far inside the gradients' 1e-5; the library expf costs five
+// times the instructions and the fused kernels evaluate it once per (position, group, channel, rail)
+__device__ __forceinline__ float exp_neg(float z) { return __expf(-z); }
 
 constexpr int kTile = 128;   // block tile in I and J
 constexpr int kChunk = 16;   // K per LDS stage
@@ -230,7 +236,7 @@ __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChun
                 float v = acc[x][y][r];
                 if (EPI == EPI_EXP_TIMES_G) {
                     const int co = j >= q.c_out ? j - q.c_out : j;
-                    v = q.g[(long long)i * q.c_out + co] * expf(-v);
+                    v = q.g[(long long)i * q.c_out + co] * exp_neg(v);
                 }
                 c[(long long)i * q.ldc + j] = v;
             }
@@ -614,7 +620,7 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int i = i0 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                    es[i][j] = (m0 + i < M && j_ok) ? gv[r] * expf(-z[r]) : 0.0f;
+                    es[i][j] = (m0 + i < M && j_ok) ? gv[r] * exp_neg(z[r]) : 0.0f;
                 }
             }
         }
@@ -644,6 +650,222 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
     for (int e = threadIdx.x; e < K * J; e += 256) {
         const int k = e / J, j = e - k * J;
         pg[e] = ((red[0][k][j] + red[1][k][j]) + red[2][k][j]) + red[3][k][j];
+    }
+}
+
+// Whole backward of layers with small OR groups (K <= 32 members: z accumulation has K = W * H,
+// yz with small channel blocks K = z_unit * W) in one kernel.  With few members per group the
+// general path's scratch array E[g][m][j] is c_in (z) times larger than the problem's tensors and
+// its GEMMs use a fraction of each MFMA; here a workgroup loops over tiles of 32 output positions
+// of one group, gathers the im2col columns into LDS, forms Z = col^T wcat with MFMAs, turns it
+// into E = g exp(-Z) in LDS and feeds both Gw += col E (accumulators live over all tiles) and
+// dcol = wd^T E^T from it; only dcol (the size of col) reaches memory, for the common col2im.
+// The weights of both products sit in registers for the life of the workgroup.
+//   KS: k-steps of the first product (ceil(K / 2), rounded up to 5, 8, 12 or 16)
+//   NB: 32-column blocks of E per wave; a launch covers NB * 128 columns from j_begin, wider
+//       layers take several launches, later ones adding to dcol
+//   DX: the input gradient is wanted
+// A workgroup handles tiles s, s + S, ... of group g0 + blockIdx.y and writes one partial sum
+// part[g][s][k][j] for the common split reduction.
+constexpr int kFusedK = 32;
+constexpr int kFusedTile = 32;
+template <int KS, int NB, bool DX>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_bwd_small_k(const float* __restrict__ x, const float* __restrict__ wcat,
+                                                     const float* __restrict__ wd, const float* __restrict__ gt,
+                                                     const int* __restrict__ base, const int* __restrict__ arow,
+                                                     const int* __restrict__ bcol, float* __restrict__ part,
+                                                     float* __restrict__ dcol, Groups G, int g0, int M, int w_in, int h_in,
+                                                     int c_out, int j_begin, int splits, int store_part, int dcol_add,
+                                                     size_t w_stride, size_t part_stride, size_t dcol_stride)
+{
+    constexpr int KP = KS <= 8 ? 16 : 32;       // member rows held in LDS and in the weight gradient
+    constexpr int TM = kFusedTile;
+    constexpr int JW = NB * 128;                // columns of E per launch
+    constexpr int DPARTS = KP == 16 ? 2 : 1;    // waves that share one 16 x 16 block of dcol and split j
+    constexpr int DSTEPS = JW / DPARTS / 4;     // 16x16x4 MFMAs per wave and tile in the dcol product
+    constexpr int GQ = KP / 8;                  // members gathered per thread
+    __shared__ float cs[KP][TM + 1];            // col tile [k][m]
+    __shared__ float es[TM][JW + 1];            // E tile [m][j]; the odd stride keeps column reads conflict-free
+    __shared__ float red[2][16][17];            // second j-half's partial dcol blocks (KP == 16)
+    const int K = G.n_members, J = 2 * c_out;
+    const int g = g0 + blockIdx.y;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int l32 = lane & 31, lk = lane >> 5, l16 = lane & 15, lq = lane >> 4;
+
+    // weights of the first product, B operand of step t: wcat[k = 2 t + lk][j]
+    const float* wg = wcat + (size_t)blockIdx.y * w_stride;
+    float w_s[NB][KS];
+#pragma unroll
+    for (int y = 0; y < NB; y++)
+#pragma unroll
+        for (int t = 0; t < KS; t++) {
+            const int k = 2 * t + lk, j = j_begin + 32 * (NB * wave + y) + l32;
+            const bool ok = k < K && j < J;
+            const float v = wg[ok ? (size_t)k * J + j : 0];
+            w_s[y][t] = ok ? v : 0.0f;
+        }
+    // dcol: wave -> (member block kb, position block mb, j part); A operand of step t: wd[j][k = 16 kb + l16]
+    const int kb = KP == 32 ? wave >> 1 : 0, mb = wave & 1, jpart = KP == 32 ? 0 : wave >> 1;
+    const int jd0 = jpart * (JW / DPARTS);
+    float w_d[DX ? DSTEPS : 1];
+    if (DX) {
+        const float* wdg = wd + (size_t)blockIdx.y * w_stride;
+#pragma unroll
+        for (int t = 0; t < DSTEPS; t++) {
+            const int j = j_begin + jd0 + 4 * t + lq, k = 16 * kb + l16;
+            const bool ok = k < K && j < J;
+            const float v = wdg[ok ? (size_t)j * K + k : 0];
+            w_d[t] = ok ? v : 0.0f;
+        }
+    }
+    // im2col gather: thread -> position (t & 31) of the tile, members (t >> 5) + 8 q
+    const int ml = threadIdx.x & 31, slot = threadIdx.x >> 5;
+    int g_off[GQ], g_u[GQ], g_v[GQ];
+    bool g_ok[GQ];
+#pragma unroll
+    for (int q4 = 0; q4 < GQ; q4++) {
+        const int k = slot + 8 * q4;
+        const Member e = member_of(G, g, k < K ? k : 0);
+        g_ok[q4] = k < K && e.ok;
+        g_off[q4] = (e.ci * w_in + e.u) * h_in + e.v;
+        g_u[q4] = e.u;
+        g_v[q4] = e.v;
+    }
+
+    // weight-gradient accumulators: 32 x 32 blocks (lane holds rows 8 (r/4) + 4 lk + r%4 of column l32),
+    // or, with at most 16 members, 16 x 16 blocks (rows 4 lq + r of column l16) at half the MFMA time
+    floatx16 gw_acc[KP == 32 ? NB : 1];
+    floatx4 gw_acc4[KP == 16 ? 2 * NB : 1];
+    if constexpr (KP == 32) {
+#pragma unroll
+        for (int y = 0; y < NB; y++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) gw_acc[y][r] = 0.0f;
+    } else {
+#pragma unroll
+        for (int b = 0; b < 2 * NB; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) gw_acc4[b][r] = 0.0f;
+    }
+
+    float* dg = dcol + (size_t)blockIdx.y * dcol_stride;
+    const int n_tiles = (M + TM - 1) / TM;
+    for (int tile = blockIdx.x; tile < n_tiles; tile += splits) {
+        const int m0 = tile * TM;
+        __syncthreads();  // the previous tile's products have read cs, es and red
+        {
+            const bool m_ok = m0 + ml < M;
+            const int mc = m_ok ? m0 + ml : 0;
+            const int r0 = arow[mc], c0 = bcol[mc], b0 = base[mc];
+            float vals[GQ];
+#pragma unroll
+            for (int q4 = 0; q4 < GQ; q4++) {
+                const int rr = r0 + g_u[q4], cc = c0 + g_v[q4];
+                const bool ok = m_ok && g_ok[q4] && cc >= 0 && cc < h_in && rr >= 0 && rr < w_in;
+                const float v = x[ok ? b0 + g_off[q4] : 0];
+                vals[q4] = ok ? v : 0.0f;
+            }
+#pragma unroll
+            for (int q4 = 0; q4 < GQ; q4++) cs[slot + 8 * q4][ml] = vals[q4];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int y = 0; y < NB; y++) {
+            // Z[m][j] = sum_k col[k][m] * wcat[k][j] for one 32 x 32 block
+            floatx16 z;
+#pragma unroll
+            for (int r = 0; r < 16; r++) z[r] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < KS; t++) z = __builtin_amdgcn_mfma_f32_32x32x2f32(cs[2 * t + lk][l32], w_s[y][t], z, 0, 0, 0);
+            // E[m][j] = g[m][co] * exp(-Z), zero outside the problem; loads of g first, no branches
+            const int jl = 32 * (NB * wave + y) + l32, j = j_begin + jl;
+            const int co = j >= c_out ? j - c_out : j;
+            const bool j_ok = j < J;
+            float gv[16];
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + 8 * (r >> 2) + 4 * lk + (r & 3);
+                gv[r] = gt[(m < M && j_ok) ? (long long)m * c_out + co : 0];
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = 8 * (r >> 2) + 4 * lk + (r & 3);
+                es[i][jl] = (m0 + i < M && j_ok) ? gv[r] * exp_neg(z[r]) : 0.0f;
+            }
+        }
+        __syncthreads();
+        // Gw[k][j] += sum_m col[k][m] * E[m][j] on this wave's column blocks
+        if constexpr (KP == 32) {
+#pragma unroll
+            for (int mm = 0; mm < TM; mm += 2) {
+                const float a = cs[l32][mm + lk];
+#pragma unroll
+                for (int y = 0; y < NB; y++)
+                    gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, es[mm + lk][32 * (NB * wave + y) + l32], gw_acc[y], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int mm = 0; mm < TM; mm += 4) {
+                const float a = cs[l16][mm + lq];
+#pragma unroll
+                for (int b = 0; b < 2 * NB; b++)
+                    gw_acc4[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, es[mm + lq][32 * NB * wave + 16 * b + l16], gw_acc4[b], 0, 0, 0);
+            }
+        }
+        if (DX) {
+            // dcol[k][m] = sum_j wd[j][k] * E[m][j]: one 16 x 16 block per wave (v_mfma_f32_16x16x4_f32:
+            // lane l feeds A[i = l%16][k' = l/16] and B[k' = l/16][j = l%16], holds D[4 (l/16) + r][l%16])
+            floatx4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int t = 0; t < DSTEPS; t++)
+                d = __builtin_amdgcn_mfma_f32_16x16x4f32(w_d[t], es[16 * mb + l16][jd0 + 4 * t + lq], d, 0, 0, 0);
+            if (DPARTS == 2) {
+                if (jpart == 1) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) red[mb][4 * lq + r][l16] = d[r];
+                }
+                __syncthreads();
+                if (jpart == 0) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) d[r] += red[mb][4 * lq + r][l16];
+                }
+            }
+            if (jpart == 0) {
+                const int m = m0 + 16 * mb + l16;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int k = 16 * kb + 4 * lq + r;
+                    if (k < K && m < M) {
+                        float* pd = dg + (size_t)k * M + m;
+                        *pd = dcol_add ? *pd + d[r] : d[r];
+                    }
+                }
+            }
+        }
+    }
+    if (store_part) {
+        float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)blockIdx.x * K * J;
+        if constexpr (KP == 32) {
+#pragma unroll
+            for (int y = 0; y < NB; y++) {
+                const int j = j_begin + 32 * (NB * wave + y) + l32;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int k = 8 * (r >> 2) + 4 * lk + (r & 3);
+                    if (k < K && j < J) pg[(size_t)k * J + j] = gw_acc[y][r];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2 * NB; b++) {
+                const int j = j_begin + 32 * NB * wave + 16 * b + l16;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int k = 4 * lq + r;
+                    if (k < K && j < J) pg[(size_t)k * J + j] = gw_acc4[b][r];
+                }
+            }
+        }
     }
 }
 
@@ -677,6 +899,8 @@ struct BwdLayout {
     int splits, m_per_split;
     Groups G;
     bool small_k;        // OR groups of at most 16 members and 2 * c_out <= 128: fused weight-gradient kernel
+    bool fused_k;        // OR groups of at most 32 members: whole backward in one kernel, no col / E scratch
+    int fused_splits;    // its workgroups per add group
     int rows_per_chunk;  // add groups processed by one round of launches
     size_t col_v, e_v, part_v, w_v;  // floats per add group of each scratch array
     size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, off_gt, bytes;
@@ -706,6 +930,15 @@ BwdLayout bwd_layout(const Geometry& g)
     }
     const int K = b.G.n_members;
     b.small_k = K <= kSmallK && 2 * g.c_out <= kTile;
+    b.fused_k = K <= kFusedK;
+    {
+        // about eight workgroups per CU in all, each looping over its share of the tiles
+        const long long n_tiles = (b.m_total + kFusedTile - 1) / kFusedTile;
+        long long want = 2048 / b.G.n_groups;
+        if (want > n_tiles) want = n_tiles;
+        if (want > 65535) want = 65535;
+        b.fused_splits = (int)(want < 1 ? 1 : want);
+    }
     // split the m-reduction of the weight gradient so that the grid covers the GPU
     const long long tiles = (long long)((K + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
     long long want = (1024 + tiles - 1) / tiles;
@@ -718,10 +951,12 @@ BwdLayout bwd_layout(const Geometry& g)
     auto pad64 = [](size_t v) { return (v + 63) & ~(size_t)63; };
     b.col_v = pad64((size_t)b.m_total * K);
     b.e_v = pad64((size_t)b.m_total * 2 * g.c_out);
-    b.part_v = pad64((size_t)b.splits * K * 2 * g.c_out);
+    b.part_v = pad64((size_t)(b.fused_k && b.fused_splits > b.splits ? b.fused_splits : b.splits) * K * 2 * g.c_out);
     b.w_v = pad64((size_t)K * 2 * g.c_out);
+    // the fused kernel needs neither col nor E
+    const size_t col_alloc = b.fused_k ? 0 : b.col_v, e_alloc = b.fused_k ? 0 : b.e_v;
     // all groups in one round of launches unless that needs more than ~3 GB of scratch
-    const size_t per_row = sizeof(float) * (2 * b.col_v + b.e_v + b.part_v + 2 * b.w_v);
+    const size_t per_row = sizeof(float) * (col_alloc + b.col_v + e_alloc + b.part_v + 2 * b.w_v);
     size_t rows = ((size_t)3 << 30) / per_row;
     if (rows < 1) rows = 1;
     if (rows > (size_t)b.G.n_groups) rows = b.G.n_groups;
@@ -729,8 +964,8 @@ BwdLayout bwd_layout(const Geometry& g)
     if (rows < 1) rows = 1;
     b.rows_per_chunk = (int)rows;
     size_t o = 0;
-    b.off_col = o;  o += align256(sizeof(float) * rows * b.col_v);
-    b.off_e = o;    o += align256(sizeof(float) * rows * b.e_v);
+    b.off_col = o;  o += align256(sizeof(float) * rows * col_alloc);
+    b.off_e = o;    o += align256(sizeof(float) * rows * e_alloc);
     b.off_dcol = o; o += align256(sizeof(float) * rows * b.col_v);
     b.off_part = o; o += align256(sizeof(float) * rows * b.part_v);
     b.off_wcat = o; o += align256(sizeof(float) * rows * b.w_v);
@@ -801,6 +1036,49 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
 #undef GEO_SC_SMALL_K
             hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
                                active, g.c_out, G, L.part_v);
+        }
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+    }
+    if (L.fused_k && !(!gx && gw && L.small_k)) {
+        if (!gx && !gw) return GEO_SC_OK;
+        const int plane_blocks = (g.w_in * g.h_in + 255) / 256;
+        const int n_planes = g.n * g.c_in;
+        const int pb = plane_blocks > 64 ? 64 : plane_blocks;
+        const int want = 256 * 16 / pb;
+        const int ks = (K + 1) / 2;
+        const int jw = J <= 128 ? 128 : 256;
+        for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
+            const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
+            int wb = grid1d((long long)K * g.c_out);
+            hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
+                               g.c_out, G, L.w_v);
+            const dim3 grid(L.fused_splits, nv);
+            for (int jb = 0; jb < J; jb += jw) {
+#define GEO_SC_FUSED_K(KS, NB, DX)                                                                                     \
+    hipLaunchKernelGGL((k_bwd_small_k<KS, NB, DX>), grid, dim3(256), 0, s, x, wcat, wd, gt, pos_base, pos_arow,         \
+                       pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, jb, L.fused_splits, gw ? 1 : 0,         \
+                       jb > 0 ? 1 : 0, L.w_v, L.part_v, L.col_v)
+#define GEO_SC_FUSED_NB_DX(KS)                                                                                         \
+    do {                                                                                                               \
+        if (jw == 128) {                                                                                               \
+            if (gx) GEO_SC_FUSED_K(KS, 1, true); else GEO_SC_FUSED_K(KS, 1, false);                                    \
+        } else {                                                                                                       \
+            if (gx) GEO_SC_FUSED_K(KS, 2, true); else GEO_SC_FUSED_K(KS, 2, false);                                    \
+        }                                                                                                              \
+    } while (0)
+                if (ks <= 5) GEO_SC_FUSED_NB_DX(5);
+                else if (ks <= 8) GEO_SC_FUSED_NB_DX(8);
+                else if (ks <= 12) GEO_SC_FUSED_NB_DX(12);
+                else GEO_SC_FUSED_NB_DX(16);
+#undef GEO_SC_FUSED_NB_DX
+#undef GEO_SC_FUSED_K
+            }
+            if (gw)
+                hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
+                                   L.fused_splits, g.c_out, G, L.part_v);
+            if (gx)
+                hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx,
+                                   v0, nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
         }
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }

@@ -158,3 +158,35 @@ def test_weight_gradient_of_small_or_groups(capi, shape_x, shape_w, pad, mode, z
     _, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False,
                                               accumulate=mode, z_unit=zu)
     assert torch.equal(gw, gw2)   # deterministic
+
+
+@pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu", [
+    ((3, 5, 9, 7), (140, 5, 3, 3), (1, 1), "z", 1),      # 9 members; 280 rails: two column launches, the second adds
+    ((2, 4, 8, 8), (70, 4, 5, 5), (2, 2), "z", 1),       # 25 members, 140 rails in one launch
+    ((2, 20, 6, 6), (12, 20, 3, 3), (1, 1), "yz", 8),    # 24 members, ragged last channel block
+    ((2, 10, 6, 5), (40, 10, 3, 2), (1, 0), "yz", 4),    # 12 members
+    ((4, 5, 7, 7), (40, 5, 3, 3), (1, 1), "y", 1),       # 15 members with an input gradient
+    ((2, 6, 5, 5), (9, 6, 1, 1), (0, 0), "z", 1),        # single-member groups
+    ((1, 3, 33, 31), (5, 3, 3, 3), (0, 2), "z", 1),      # 31 * 33 positions: ragged last tile
+])
+def test_whole_backward_of_small_or_groups(capi, shape_x, shape_w, pad, mode, zu):
+    """OR groups of at most 32 members run the whole backward in one fused kernel (no im2col / E
+    arrays in memory): both gradients against the float64 oracle, alone and together."""
+    from oracle import surrogate
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_x[1] + shape_w[0])
+    w = (w * 3).contiguous()
+    w.view(-1)[::7] = 0.0
+    d = capi.make_desc(x.shape, w.shape, 64, pad)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(4))
+    kw = dict(accumulate=mode, z_unit=zu)
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
+    torch.cuda.synchronize()
+    rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
+    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
+    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    gx2, none = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_w=False, **kw)
+    none2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False, **kw)
+    assert none is None and none2 is None
+    assert torch.equal(gx2, gx) and rel_err(gw2, rw) <= RTOL
+    gx3, gw3 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
+    assert torch.equal(gx3, gx) and torch.equal(gw3, gw)   # deterministic
