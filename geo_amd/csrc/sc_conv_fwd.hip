@@ -199,7 +199,153 @@ __global__ __launch_bounds__(64) void k_conv_fwd(FwdParams q)
     }
 }
 
-// OR-accumulate CU channels for the split kernel: activation words are addressed as a
+// The same kernel for launches that are split over blockIdx.y: each workgroup sums a
+// contiguous range of (pack, add group) pairs and adds its partial result to y with integer
+// atomics (y is zeroed first).  Used for small layers that would otherwise leave most of the
+// GPU idle, and for the accumulation modes other than "OR over (c_in, w_k), add over h_k":
+// the add groups are (outer, inner) pairs, an outer group owning a range of OR channels
+//   Y : outer 1,              inner kernel rows,     OR channels = input channels
+//   YZ: outer channel groups, inner kernel rows,     OR channels = the group's input channels
+//   Z : outer 1,              inner input channels,  OR channels = kernel rows
+//   FULL: one group per pack; the OR runs over the input channels of or_rows = h_k kernel rows
+// (sc_cuda_kernel.cu:176-349, :1351-1366), expressed through the two activation strides in FwdParams; the
+// weight lines arrive in exactly the order the loop consumes them.
+// Template parameters:
+//   R   rows of accumulators per lane.  ROWS_IN_N == false: R consecutive output rows a
+//       (dim 2) of one item; the WK kernel taps slide over R+WK-1 activation words, so each
+//       word is loaded once per channel.  ROWS_IN_N == true (outputs with a single row, e.g.
+//       the SC-linear mapping): R consecutive batch items.
+//   WK  kernel extent in dim 2 (0: run-time extent, R == 1).
+//   CU  input channels per loop trip, chosen so that a trip holds ~192 and-or instructions.
+template <int R, int WK, int CU, bool ROWS_IN_N>
+__global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
+{
+    constexpr int C = kCoTile;
+    static_assert(WK > 0 || (R == 1 && !ROWS_IN_N), "run-time kernel extent handles one row per lane");
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long slot0 = (long long)(blockIdx.x / q.n_cotile) * 64 + threadIdx.x;
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : 0;
+    // lane slot -> (first item n, first output row a0, output column b).  With ROWS_IN_N the
+    // R rows of a lane are items n and n + row_groups, consecutive lanes are consecutive
+    // items, and the activation streams are stored item-innermost.
+    const int b = ROWS_IN_N ? (int)(slot / q.row_groups) : (int)(slot % q.ho);
+    const long long t = slot / q.ho;
+    const int a0 = ROWS_IN_N ? 0 : (int)(t % q.row_groups) * R;
+    const long long n = ROWS_IN_N ? slot % q.row_groups : t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
+
+    constexpr int NW = WK == 0 ? 1 : (ROWS_IN_N ? R * WK : R + WK - 1);
+    // word offsets inside one channel plane.  Rows past the end (partial last group) are
+    // clamped to valid ones: they only feed outputs that are never stored.
+    unsigned off[NW];
+    if constexpr (WK > 0) {
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            if (ROWS_IN_N) {
+                const int r = j / WK, u = j % WK;
+                off[j] = (n + (long long)r * q.row_groups < q.n ? (unsigned)r * q.row_groups : 0u) +
+                         (unsigned)u * q.hi * q.n;
+            } else {
+                const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+                off[j] = (unsigned)row * q.hi;
+            }
+        }
+    } else {
+        off[0] = 0;
+    }
+    // strides (words) of one pack, one kernel row step, one channel
+    const size_t pack_stride = ROWS_IN_N ? (size_t)q.act_plane * q.n : (size_t)q.act_plane;
+    const unsigned v_stride = ROWS_IN_N ? (unsigned)q.n : 1u;
+    const unsigned ch_stride = ROWS_IN_N ? (unsigned)q.wi * q.hi * q.n : (unsigned)q.wi * q.hi;
+    const uint32_t* act_n = ROWS_IN_N ? q.act + (size_t)b * q.n + n : q.act + (size_t)n * item_stride + b;
+    const unsigned k_stride = (unsigned)q.n_cotile * 2 * C;
+
+    int sum[R][C];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int c = 0; c < C; c++) sum[r][c] = 0;
+
+    // (pack, add group) pairs are independent partial sums: blockIdx.y takes a contiguous
+    // range of them when the launch is split to fill the GPU
+    const int groups = q.add_outer * q.add_inner;
+    const int pv_begin = blockIdx.y * q.pv_per_block;
+    const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
+    const unsigned add_stride = ROWS_IN_N ? v_stride : q.add_stride;
+    const unsigned or_stride = ROWS_IN_N ? ch_stride : q.or_stride;
+    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    {
+        for (int pv = pv_begin; pv < pv_end; pv++) {
+            const int p = pv / groups, g = pv - p * groups;
+            const int go = g / q.add_inner, gi = g - go * q.add_inner;
+            const int ch0 = go * q.or_ch_per_group;
+            const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
+            uint32_t orp[R][C], orn[R][C];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int c = 0; c < C; c++) orp[r][c] = orn[r][c] = 0u;
+
+            const uint32_t* ap0 = act_n + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
+            const size_t line = p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k + (size_t)gi * chs * q.w_k;
+            const uint32_t* wp = q.wgt + (line * q.n_cotile + cot) * (2 * C);
+
+            for (int row = 0; row < q.or_rows; row++) {
+                const uint32_t* ap = ap0 + row;  // next kernel row: one word further (never with ROWS_IN_N)
+                if constexpr (WK > 0) {
+                    int ci = 0;
+                    for (; ci + CU <= chs; ci += CU)
+                        or_channels<R, WK, CU, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
+                    if constexpr (CU > 1)
+                        for (; ci < chs; ci++)
+                            or_channels<R, WK, 1, NW, ROWS_IN_N>(orp, orn, ap, wp, off, or_stride, k_stride);
+                } else {
+                    for (int ci = 0; ci < chs; ci++) {
+                        for (int u = 0; u < q.w_k; u++) {
+                            uint32_t wv[2 * C];
+#pragma unroll
+                            for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
+                            int arow = a0 + u;
+                            arow = arow < q.wi ? arow : q.wi - 1;
+                            const uint32_t aw = ap[(unsigned)arow * q.hi];
+#pragma unroll
+                            for (int c = 0; c < C; c++) {
+                                and_or(orp[0][c], aw, wv[c]);
+                                and_or(orn[0][c], aw, wv[C + c]);
+                            }
+                            wp += k_stride;
+                        }
+                        ap += or_stride;
+                    }
+                }
+            }
+            // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int c = 0; c < C; c++) sum[r][c] += __popc(orp[r][c]) - __popc(orn[r][c]);
+        }
+    }
+
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const int co = cot * C + c;
+        if (co >= q.c_out) break;
+        int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const bool row_ok = ROWS_IN_N ? n + (long long)r * q.row_groups < q.n : a0 + r < q.wo;
+            int32_t* dst = yo + (ROWS_IN_N ? (size_t)r * q.row_groups * q.c_out * out_plane : (size_t)r * q.ho);
+            if (!row_ok) continue;
+            atomicAdd(dst, sum[r][c]);  // integer adds: order does not matter
+        }
+    }
+}
+
+// OR-accumulate CU channels for the item-innermost split kernel: activation words are addressed as a
 // wave-uniform pointer plus a 32-bit lane offset in bytes (scalar address arithmetic, one VGPR
 // per offset).  With ROWS_IN_N the lane offsets select the R batch items and the kernel taps advance
 // the uniform pointer by tap_stride; otherwise the lane offsets select the R+WK-1 rows.  FIRST:
@@ -247,9 +393,14 @@ __device__ __forceinline__ void or_channels_u(uint32_t (&orp)[R][kCoTile], uint3
     ap_u += (size_t)CU * ch_stride;
 }
 
-// The same computation for launches that are split over blockIdx.y: each workgroup sums a
-// contiguous range of (pack, add group) pairs and adds its partial result to y with integer
-// atomics (y is zeroed first).  Used for small layers that would otherwise leave most of the
+// The split kernel for item-innermost activation streams (outputs with a single row: the SC-linear
+// mapping).  Its OR groups are short (16 members for a 4096-wide linear layer as 16 x 1 x 256), so
+// per-group overhead counts: the first weight line assigns the accumulators instead of OR-ing into
+// zeroed ones, and activation addresses are a wave-uniform base plus one 32-bit byte offset per
+// lane (4096 x 4096 linear at batch 1024: 6.3 -> 5.65 ms).  For position-major streams this
+// form is 5-6 % slower than k_conv_fwd_split, which therefore keeps them.
+// Each workgroup sums a contiguous range of (pack, add group) pairs and adds its partial result to y
+// with integer atomics (y is zeroed first).  Used for small layers that would otherwise leave most of the
 // GPU idle, and for the accumulation modes other than "OR over (c_in, w_k), add over h_k":
 // the add groups are (outer, inner) pairs, an outer group owning a range of OR channels
 //   Y : outer 1,              inner kernel rows,     OR channels = input channels
@@ -260,7 +411,7 @@ __device__ __forceinline__ void or_channels_u(uint32_t (&orp)[R][kCoTile], uint3
 // FwdParams; the weight lines arrive in exactly the order the loop consumes them.
 // Template parameters as for k_conv_fwd.
 template <int R, int WK, int CU, bool ROWS_IN_N>
-__global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
+__global__ __launch_bounds__(64) void k_conv_fwd_split_items(FwdParams q)
 {
     constexpr int C = kCoTile;
     static_assert(WK > 0 || (R == 1 && !ROWS_IN_N), "run-time kernel extent handles one row per lane");
@@ -496,24 +647,23 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     q.pv_per_block = (pv + splits - 1) / splits;
     splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
     const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y;
-    if (!plain) {
-        // the split kernel's lane offsets are 32-bit byte offsets, relative to the first item of a
-        // tile (or, item-innermost, inside one pack of all items)
-        const long long span = 64 / ((long long)q.row_groups * g.ho) + 2;
-        const unsigned long long reach =
-            ROWS_IN_N ? (unsigned long long)g.act_plane * g.n
-                      : (unsigned long long)(span < g.n ? span : g.n) * g.packs * g.act_plane + g.act_plane;
-        if (reach * 4 >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
+    if (!plain && ROWS_IN_N) {
+        // the item-innermost split kernel's lane offsets are 32-bit byte offsets inside one pack of all items
+        if ((unsigned long long)g.act_plane * g.n * 4 >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
     }
     if (!plain) {
         const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
         size_t zb = (n_out + 255) / 256;
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
     }
-    if (!plain)
-        hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
-                           0, s, q);
-    else
+    if (!plain) {
+        if constexpr (ROWS_IN_N)
+            hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>), dim3((unsigned)blocks, (unsigned)splits),
+                               dim3(64), 0, s, q);
+        else
+            hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, false>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
+                               0, s, q);
+    } else
         hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks), dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
