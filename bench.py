@@ -390,7 +390,10 @@ def main():
                                    "full": "full OR accumulation"}[args.accumulate]
                                + f", {args.generator} generators",
                    "pass": args.passes, "bit_macs_per_step": B},
-        "layer_ms": {"fwd": fwd_avg, "bwd": bwd_avg, "fwd_bit_macs_per_s": B / (fwd_avg * 1e-3)},
+        "layer_ms": {"fwd": fwd_avg, "bwd": bwd_avg, "fwd_bit_macs_per_s": B / (fwd_avg * 1e-3),
+                     "fwd_median": statistics.median(fwd_ms), "fwd_min": min(fwd_ms),
+                     "bwd_median": statistics.median(bwd_ms) if with_bwd else None,
+                     "bwd_min": min(bwd_ms) if with_bwd else None},
         "roofline": {
             "bound": "valu",
             "kernel": "k_conv_fwd (v_and_or_b32 / v_bcnt_u32_b32)",

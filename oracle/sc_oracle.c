@@ -30,14 +30,19 @@
  *                                  z_unit (seeds restart per block); one block
  *                                  is y-mode itself (tests/test_oracle.py)
  *   sco_conv2d_modes, mode z
- *                        pinned where the OR window is one-dimensional (H = 1;
- *                        W = 1 on single-row signals; per-channel
- *                        decomposition when seeds restart per channel).  For
- *                        general W x H windows (joint OR over (u,v), seed
- *                        index u*H+v) PARITY UNPINNED: the reference has no
- *                        executable z-mode code outside its CUDA kernels
- *                        (sc_cuda_kernel.cu:270-349); an independent per-bit
- *                        formulation of the same reading agrees.
+ *                        pinned  - one-dimensional windows (H = 1; W = 1 on
+ *                        single-row signals) are y-mode itself; a general
+ *                        W x H window (joint OR over (u,v), weight seed index
+ *                        u*H+v) is y-mode on the restated problem "kernel
+ *                        column u -> input channel u, one kernel row", whose
+ *                        seeds coincide exactly for sizes with
+ *                        Hi = Wo = 1 (mod L-1); the add over input channels by
+ *                        the per-channel decomposition where planes hold a
+ *                        multiple of L-1 words (tests/test_oracle.py).  What
+ *                        stays a reading of the CUDA text
+ *                        (sc_cuda_kernel.cu:270-349) is only that z-mode takes
+ *                        the seed index u*H+v rather than v*W+u; an independent
+ *                        per-bit formulation of the same reading agrees.
  *   sco_philox4x32_10    pinned  - the three known-answer vectors of the
  *                                  published Philox4x32-10 (Salmon et al., SC'11;
  *                                  Random123 kat_vectors)

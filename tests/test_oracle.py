@@ -300,6 +300,46 @@ def test_z_reduces_to_y_mode_where_the_window_is_one_dimensional():
     assert np.array_equal(so.conv2d_modes(x, w, 8, (0, 0), "z"), exp)
 
 
+def _z_window_as_y_mode(x1, w1, L, load):
+    """Single-channel z-mode (joint OR over a W x H window, weight seed index u*H + v) restated as
+    a y-mode problem: kernel column u becomes input channel u, kernel row index v becomes the
+    dim-2 tap, one kernel row: x'[u, p', q'] = x[q' + u, p'], w'[co, u, v, 0] = w[co, 0, u, v].
+    y-mode then ORs over (c' = u, u' = v) with weight seed index c' * W' + u' = u * H + v - z-mode's.
+    The activation seed of x'[u, q, a] is u*Hi*Wo + q*Wo + a, z-mode's is (a + u)*Hi + q: equal
+    modulo L - 1 (all that a seed depends on) when Hi = Wo = 1 (mod L - 1).
+    Returns out[n, co, a, b]."""
+    n, _, wi, hi = x1.shape
+    c_out, _, W, H = w1.shape
+    wo = wi - W + 1
+    assert hi % (L - 1) == 1 and wo % (L - 1) == 1
+    xt = np.empty((n, W, hi, wo), dtype=np.float32)
+    for u in range(W):
+        xt[:, u] = x1[:, 0, u:u + wo, :].transpose(0, 2, 1)
+    wt = np.ascontiguousarray(w1[:, 0, :, :, None])          # (c_out, W, H, 1)
+    yt = so.conv2d_add_partial(xt, wt, L, (0, 0), *load)       # (n, c_out, Ho, Wo)
+    return yt.transpose(0, 1, 3, 2)
+
+
+@pytest.mark.parametrize("L,W,H,k", [(8, 3, 3, 1), (8, 2, 5, 2), (16, 3, 2, 1), (32, 2, 3, 1), (8, 7, 2, 1)])
+def test_z_two_dimensional_windows_reduce_to_y_mode(L, W, H, k):
+    """General W x H windows of z-mode against the y-mode path that the compiled reference pins:
+    sizes with Hi = Wo = 1 (mod L - 1) make the restated problem's seeds coincide exactly.  With
+    W = L - 1 the channel planes hold a multiple of L - 1 words, so several channels decompose too
+    (z adds over input channels; weight seeds do not depend on the channel)."""
+    hi = wo = 1 + k * (L - 1)
+    wi = wo + W - 1
+    c_in = 3 if W == L - 1 else 1
+    x, w = wl.make_inputs((2, c_in, wi, hi), (3, c_in, W, H), "prescribed", seed=80 + L + W)
+    x, w = x.numpy(), (w.numpy() * 0.5).astype(np.float32)
+    for load in [(7, 8, 1, 1), (7, 2, 2, 3)]:
+        got = so.conv2d_modes(x, w, L, (0, 0), "z", 1, *load)
+        exp = 0
+        for c in range(c_in):
+            exp = exp + _z_window_as_y_mode(x[:, c:c + 1], w[:, c:c + 1], L, load)
+        assert got.any()
+        assert np.array_equal(got, exp), (L, W, H, load)
+
+
 @pytest.mark.parametrize("mode,zu", [("z", 1), ("yz", 2), ("yz", 3), ("y", 1)])
 def test_modes_against_independent_per_bit_formulation(mode, zu):
     for (sx, sw, pad, L) in [((2, 3, 4, 5), (2, 3, 3, 2), (1, 0), 8), ((1, 5, 4, 4), (3, 5, 2, 3), (0, 1), 32)]:
