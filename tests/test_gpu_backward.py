@@ -168,6 +168,10 @@ def test_weight_gradient_of_small_or_groups(capi, shape_x, shape_w, pad, mode, z
     ((4, 5, 7, 7), (40, 5, 3, 3), (1, 1), "y", 1),       # 15 members with an input gradient
     ((2, 6, 5, 5), (9, 6, 1, 1), (0, 0), "z", 1),        # single-member groups
     ((1, 3, 33, 31), (5, 3, 3, 3), (0, 2), "z", 1),      # 31 * 33 positions: ragged last tile
+    ((2, 8, 6, 5), (6, 8, 4, 2), (1, 0), "yz", 8),       # exactly 32 members
+    ((2, 3, 5, 5), (1, 3, 3, 3), (1, 1), "z", 1),        # one output channel
+    ((1, 2100, 3, 3), (2, 2100, 2, 2), (0, 0), "z", 1),  # more groups than workgroups wanted: one workgroup each
+    ((1, 2, 3, 4), (3, 2, 3, 3), (0, 0), "z", 1),        # two output positions in all
 ])
 def test_whole_backward_of_small_or_groups(capi, shape_x, shape_w, pad, mode, zu):
     """OR groups of at most 32 members run the whole backward in one fused kernel (no im2col / E
