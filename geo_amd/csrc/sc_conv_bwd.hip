@@ -63,6 +63,9 @@ struct GemmParams {
     // EPI_EXP_TIMES_G: c[i][j] = g[i * c_out + (j % c_out)] * exp(-acc), g = upstream gradient stored [m][c_out]
     const float* __restrict__ g;
     int c_out, npos;
+    // tile extent per workgroup in i and j: kTile, or kTile / 2 in at most one of them (set by
+    // launch_gemm): the four waves then line up along the other dimension
+    int tile_i, tile_j;
 };
 
 // Staging of one kChunk x kTile operand tile, split in two so that the global loads of chunk
@@ -182,8 +185,8 @@ __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChun
 
     Stager<A_KMAJOR, VEC> sa;
     Stager<B_KMAJOR, VEC> sb;
-    sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, q.I);
-    sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, q.J);
+    sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i));
+    sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j));
     float ra[8], rb[8];
     if (k_begin < k_end) {
         sa.fetch(ra, k_end - k_begin);
@@ -249,17 +252,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 {
     __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
-    const int i0 = blockIdx.x * kTile, j0 = blockIdx.y * kTile;
+    const int i0 = blockIdx.x * q.tile_i, j0 = blockIdx.y * q.tile_j;
     const int batch = blockIdx.z / q.splits, split = blockIdx.z - batch * q.splits;
     const int k_begin = split * q.k_per_split;
     const int k_end = min(q.K, k_begin + q.k_per_split);
     // the wave index through readfirstlane: the compiler then knows that everything derived from it
     // (tile corner, block choice) is uniform and branches on it with scalar instructions
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;  // this wave's 64x64 corner in the tile
+    // this wave's corner in the tile: 2 x 2 waves of 64 x 64; with a tile of 64 in one dimension
+    // (results that are narrow there) the four waves line up along the other, 32 x 64 (or 64 x 32) each
+    const bool narrow_j = q.tile_j < kTile, narrow_i = q.tile_i < kTile;
+    const int wi = narrow_j ? wave * 32 : narrow_i ? 0 : (wave >> 1) * 64;
+    const int wj = narrow_j ? 0 : narrow_i ? wave * 32 : (wave & 1) * 64;
     const int l32 = lane & 31, lk = lane >> 5;
-    // which of this wave's four 32 x 32 blocks lie inside the result
-    const bool x0 = i0 + wi < q.I, x1 = i0 + wi + 32 < q.I, y0 = j0 + wj < q.J, y1 = j0 + wj + 32 < q.J;
+    // which of this wave's (up to) four 32 x 32 blocks lie inside the result
+    const bool x0 = i0 + wi < q.I, x1 = !narrow_j && i0 + wi + 32 < q.I;
+    const bool y0 = j0 + wj < q.J, y1 = !narrow_i && j0 + wj + 32 < q.J;
     const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
 #define GEO_SC_GEMM_WAVE(NX, NY)                                                                                        \
     gemm_wave<A_KMAJOR, B_KMAJOR, EPI, VEC, NX, NY>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk)
@@ -877,9 +885,16 @@ int grid1d(long long total)
 }
 
 template <bool AK, bool BK, int EPI>
-int launch_gemm(const GemmParams& q, int batch, hipStream_t s)
+int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
 {
-    dim3 grid((q.I + kTile - 1) / kTile, (q.J + kTile - 1) / kTile, q.splits * batch);
+    GemmParams q = q0;
+    // A dimension of at most 192 whose last (or only) 128-tile would be at most half full takes tiles of
+    // 64: the 2 x 2 wave arrangement would leave half of the waves of such a tile without work (one
+    // dimension only, j first).
+    auto half_tiles = [](int n) { return n <= 3 * kTile / 2 && (n - 1) % kTile < kTile / 2; };
+    q.tile_j = half_tiles(q.J) ? kTile / 2 : kTile;
+    q.tile_i = q.tile_j == kTile && half_tiles(q.I) ? kTile / 2 : kTile;
+    dim3 grid((q.I + q.tile_i - 1) / q.tile_i, (q.J + q.tile_j - 1) / q.tile_j, q.splits * batch);
     // float4 staging needs every row start and every chunk start on a 16-byte boundary
     const bool a_vec = q.lda % 4 == 0 && ((uintptr_t)q.a & 15) == 0 && q.a_batch_stride % 4 == 0 && (AK ? q.I % 4 == 0 : true);
     const bool b_vec = q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0 && (BK ? q.J % 4 == 0 : true);
