@@ -190,6 +190,19 @@ def bn_fixed_affine(mean, var, gamma, beta, eps, elements_per_channel, running_m
     return w_n, b_n, invstd, scale
 
 
+def quantize(x, prec, out=None, stream=None):
+    """geo_sc_quantize: round(x * 2^prec) clamped to +-(2^prec - 1), over 2^prec, in one launch.
+    ``x`` is a contiguous fp32 GPU tensor; ``out`` may be ``x`` itself."""
+    _require_gpu_f32(x, "x")
+    if out is None:
+        out = torch.empty_like(x)
+    elif not (out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and out.shape == x.shape):
+        raise ValueError("out must be a contiguous fp32 GPU tensor of x's shape")
+    _check(_native.lib().geo_sc_quantize(_ptr(x), _ptr(out), x.numel(), int(prec), _stream_ptr(stream)),
+           "geo_sc_quantize")
+    return out
+
+
 def _tables(bit_length, device):
     n = ctypes.c_size_t(0)
     _check(_native.lib().geo_sc_stream_tables_size(int(bit_length), ctypes.byref(n)), "tables size")

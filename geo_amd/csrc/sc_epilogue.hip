@@ -286,6 +286,20 @@ __global__ __launch_bounds__(256) void k_bn_fixed_affine(const float* __restrict
     }
 }
 
+// quantize of the reference (utils_functional.py:33-39), element-wise; comparisons instead of
+// fminf / fmaxf so that a NaN stays a NaN as torch.clamp leaves it
+__global__ __launch_bounds__(256) void k_quantize(const float* __restrict__ src, float* __restrict__ dst, size_t n,
+                                                  float scale, float inv_scale)
+{
+    const float hi = scale - 1.0f;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+        float v = rintf(src[i] * scale);
+        v = v < -hi ? -hi : (v > hi ? hi : v);
+        dst[i] = v * inv_scale;
+    }
+}
+
 int tail_splits(int n, int c, int w, int h)
 {
     // enough blocks to fill the GPU, not more than the channel has 256-element chunks
@@ -414,5 +428,18 @@ extern "C" int geo_sc_bn_fixed_affine(const float* mean, const float* var, const
                              : 1.0f;
     hipLaunchKernelGGL(k_bn_fixed_affine, dim3(1), dim3(256), 0, (hipStream_t)stream, mean, var, gamma, beta, c, eps,
                        eps_grad, unbias, running_mean, running_var, w_n, b_n, invstd, scale);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_quantize(const float* src, float* dst, size_t n, int prec, geo_sc_stream_t stream)
+{
+    if (prec < 1 || prec > 23) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (n == 0) return GEO_SC_OK;
+    if (!src || !dst) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const float scale = (float)(1u << prec);
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    hipLaunchKernelGGL(k_quantize, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, src, dst, n, scale,
+                       1.0f / scale);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }

@@ -257,6 +257,13 @@ GEO_SC_API int geo_sc_bn_fixed_affine(const float* mean, const float* var, const
                                       float* scale, geo_sc_stream_t stream);
 
 /*
+ * quantize (utils_functional.py:33-39) in one pass: dst = clamp(round(src * 2^prec), -(2^prec - 1), 2^prec - 1)
+ * / 2^prec, rounding half to even as torch.round does; prec 1..23.  The layer applies it to its input
+ * and to weight_org on every call (utils_class.py:32-33).  n fp32 elements on the device; dst may be src.
+ */
+GEO_SC_API int geo_sc_quantize(const float* src, float* dst, size_t n, int prec, geo_sc_stream_t stream);
+
+/*
  * geo_sc_conv2d_add_partial_forward for activations given as the 7-bit integers k = round(x * 128)
  * that geo_sc_layer_epilogue emits (uint8 (n, c_in, w_in, h_in), k <= 127): the activation is
  * x = k / 128, exactly what the reference's layer computes from after its input quantisation

@@ -169,3 +169,27 @@ def test_bn_fixed_affine_matches_torch_ops(capi, c, affine):
     assert torch.equal(w_n, exp_w.expand(c)) and torch.equal(b_n, exp_b.expand(c))
     assert torch.allclose(invstd, torch.rsqrt(var + 1e-5), rtol=1e-6)
     assert torch.allclose(rm, exp_rm, rtol=1e-6, atol=1e-7) and torch.allclose(rv, exp_rv, rtol=1e-6, atol=1e-7)
+
+
+def test_quantize_kernel_equals_the_torch_op_chain():
+    """geo_sc_quantize against (x * 2^p).round().clamp(+-(2^p - 1)) / 2^p (utils_functional.py:33-39):
+    bit for bit, including ties (half to even), the clamp ends, zeros' signs aside, and NaN."""
+    from geo_amd import capi, utils_functional as uf
+    g = torch.Generator().manual_seed(5)
+    x = (torch.rand(100003, generator=g) * 4 - 2)
+    x[:16] = torch.tensor([0.5 / 128, 1.5 / 128, 2.5 / 128, -0.5 / 128, -1.5 / 128, 127.5 / 128, 1.0, -1.0, 3.0, -3.0,
+                           0.0, 126.5 / 128, 1e-9, -1e-9, float("inf"), float("-inf")])
+    x[16] = float("nan")
+    xd = x.cuda()
+    for prec in (7, 8, 3):
+        p2 = 2 ** prec
+        ref = (xd * p2).round().clamp(-p2 + 1, p2 - 1) / p2
+        got = capi.quantize(xd, prec)
+        same = (got == ref) | (got.isnan() & ref.isnan())
+        assert bool(same.all()), (prec, x[~same.cpu()][:5])
+        # the functional entry takes the kernel for fp32 GPU tensors and the op chain elsewhere
+        assert torch.equal(torch.nan_to_num(uf.quantize(xd, prec)), torch.nan_to_num(ref))
+        assert torch.equal(torch.nan_to_num(uf.quantize(x, prec)), torch.nan_to_num(ref.cpu()))
+    y = xd.clone()
+    assert capi.quantize(y, 7, out=y) is y and torch.equal(torch.nan_to_num(y), torch.nan_to_num(capi.quantize(xd, 7)))
+    assert capi.quantize(torch.empty(0, device="cuda"), 7).numel() == 0
