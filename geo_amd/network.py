@@ -268,11 +268,17 @@ def train_step(model, inputs, target, criterion, optimizer, param_copy):
         if hasattr(m, "weight_org"):
             m.weight.data.copy_(m.weight_org)
     params = list(model.parameters())
+    # the per-parameter loops of the reference as multi-tensor calls: one kernel for all gradients,
+    # one for all copies
+    with_grad = [(master, p) for master, p in zip(param_copy, params) if p.grad is not None]
     for master, p in zip(param_copy, params):
-        master.grad = None if p.grad is None else (p.grad.data.float() / SCALE_FACTOR)
+        master.grad = None
+    if with_grad:
+        scaled = torch._foreach_div([p.grad.data.float() for _, p in with_grad], SCALE_FACTOR)
+        for (master, _), g in zip(with_grad, scaled):
+            master.grad = g
     optimizer.step()
-    for master, p in zip(param_copy, params):
-        p.data.copy_(master.data)
+    torch._foreach_copy_([p.data for p in params], [master.data for master in param_copy])
     for m in model.modules():
         if hasattr(m, "weight_org"):
             m.weight_org.copy_(m.weight.data.clamp(-1, 0.999))
