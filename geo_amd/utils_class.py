@@ -95,7 +95,7 @@ class _SCConvBlock(torch.autograd.Function):
         w = weight.detach().float().contiguous()
         L = conv_kw["bit_length"]
         counts = capi.conv2d_add_partial_forward(x, w, **conv_kw)
-        y = counts.float() / L
+        y = counts * (1.0 / L)   # one kernel; exact: L is a power of two
         dims = (0, 2, 3)
         mean, var = y.mean(dim=dims), y.var(dim=dims, unbiased=False)
         # One launch for what BatchNorm*_fixed computes per channel (utils_class.py:52-62) and for what
