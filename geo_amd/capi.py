@@ -237,9 +237,13 @@ def weight_streams(w, desc: ConvDesc, stream=None):
     n = ctypes.c_size_t(0)
     _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
     packs = (desc.bit_length + 31) // 32
-    out = torch.empty((packs, desc.h_k, desc.c_in * desc.w_k, (desc.c_out + 15) // 16, 2, 16), dtype=torch.int32,
-                      device=w.device)
-    assert out.numel() == n.value
+    shape = (packs, desc.h_k, desc.c_in * desc.w_k, (desc.c_out + 15) // 16, 2, 16)
+    classic = packs * desc.h_k * desc.c_in * desc.w_k * ((desc.c_out + 15) // 16) * 32
+    # the buffer may continue behind the two-rail lines (rail-packed copy for large y-mode launches);
+    # the returned view shows the lines and keeps the whole buffer alive
+    buf = torch.empty(n.value, dtype=torch.int32, device=w.device)
+    assert n.value >= classic
+    out = buf[:classic].view(shape)
     tables = _tables(desc.bit_length, w.device)
     _check(_native.lib().geo_sc_weight_streams(ctypes.byref(desc), _ptr(w), _ptr(out), _ptr(tables),
                                                _stream_ptr(stream)), "geo_sc_weight_streams")
@@ -250,6 +254,11 @@ def conv2d_add_partial_from_streams(act, wgt, desc: ConvDesc, out=None, stream=N
     """The AND/OR/popcount kernel alone on pre-generated streams (int32-typed words)."""
     if out is None:
         out = torch.empty(output_shape(desc), dtype=torch.int32, device=act.device)
+    n = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
+    if wgt.untyped_storage().nbytes() - wgt.storage_offset() * wgt.element_size() < 4 * n.value:
+        raise ValueError("weight streams: the buffer behind this tensor is smaller than geo_sc_weight_stream_words "
+                         "(take it from weight_streams())")
     _check(_native.lib().geo_sc_conv2d_add_partial_from_streams(ctypes.byref(desc), _ptr(act), _ptr(wgt), _ptr(out),
                                                                 _stream_ptr(stream)),
            "geo_sc_conv2d_add_partial_from_streams")

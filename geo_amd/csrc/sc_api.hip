@@ -100,7 +100,21 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     }
     g->act_item_inner = !g->thin && g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
-    g->wgt_words = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile * 2 * kCoTile;
+    {
+        // the same count of waves launch_conv_forward sees for two output rows per lane
+        const long long row_groups = (wo + 1) / 2;
+        const long long waves = (((long long)d->n * row_groups * ho + 63) / 64) * g->n_cotile;
+        g->rail = g->mode == GEO_SC_ACC_Y && !g->thin && !g->act_item_inner && wo >= 2 &&
+                  (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) && waves >= 4096;
+    }
+    const size_t lines = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile;
+    g->wgt_words = lines * 2 * kCoTile;
+    g->wgt_rail_off = g->wgt_rail_idx_off = 0;
+    if (g->rail) {
+        g->wgt_rail_off = (g->wgt_words + 63) & ~(size_t)63;
+        g->wgt_rail_idx_off = g->wgt_rail_off + lines * kCoTile;
+        g->wgt_words = g->wgt_rail_idx_off + lines * (kCoTile / 4);
+    }
     g->off_tables = 0;
     g->off_wgt = align256(table_bytes(g->L));
     g->off_act = g->off_wgt + align256(g->wgt_words * sizeof(uint32_t));
@@ -130,6 +144,7 @@ int forward_impl(const geo_sc_conv_desc* desc, const void* x, const float* w, in
     uint32_t* act = (uint32_t*)(ws + g.off_act);
     if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
     if ((rc = launch_weight_streams(g, w, wgt, tables, s)) != GEO_SC_OK) return rc;
+    if ((rc = launch_rail_pack(g, wgt, s)) != GEO_SC_OK) return rc;
     rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)x, act, tables, s)
             : launch_act_streams(g, (const float*)x, act, tables, s);
     if (rc != GEO_SC_OK) return rc;
@@ -231,7 +246,9 @@ int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t
     hipStream_t s = (hipStream_t)stream;
     rc = launch_build_tables(g, (uint32_t*)tables, s);
     if (rc != GEO_SC_OK) return rc;
-    return launch_weight_streams(g, w, streams, (const uint32_t*)tables, s);
+    rc = launch_weight_streams(g, w, streams, (const uint32_t*)tables, s);
+    if (rc != GEO_SC_OK) return rc;
+    return launch_rail_pack(g, streams, s);
 }
 
 int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,

@@ -44,7 +44,14 @@ struct Geometry {
     // lanes over the members of an OR group instead of over output positions.
     bool thin;
     size_t act_words;    // n * packs * act_plane
-    size_t wgt_words;    // packs * h_k * k_or * n_cotile * 2 * kCoTile
+    // Weight stream buffer: lines [packs][h_k][k_or][n_cotile] of 2 x kCoTile words (both rails), then,
+    // with rail, the same lines once more in the rail-packed form the plain y-mode kernel reads:
+    // at wgt_rail_off kCoTile words per line (the non-zero rail's word), at wgt_rail_idx_off
+    // kCoTile / 4 words per line (one byte per channel: which rail).
+    size_t wgt_words, wgt_rail_off, wgt_rail_idx_off;
+    // Large y-mode launches run the rail-skipping kernel: per weight at most one rail's stream
+    // is non-zero (codes of clamp(w, 0, .) and -clamp(w, ., 0)), and only that rail is processed.
+    bool rail;
     // workspace carve-up (byte offsets, 256-aligned)
     size_t off_tables, off_wgt, off_act, ws_bytes;
 };
@@ -70,6 +77,8 @@ int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* stre
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
+// fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.rail)
+int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s);
 size_t backward_workspace_bytes(const Geometry& g);
 int launch_conv_backward(const Geometry& g, const float* x, const float* w, const float* gy, float* gx, float* gw,
                          void* workspace, hipStream_t s);

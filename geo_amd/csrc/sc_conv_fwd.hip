@@ -21,6 +21,8 @@ namespace {
 struct FwdParams {
     const uint32_t* __restrict__ act;  // [n][P][c_in][wi][hi], or [P][c_in][wi][hi][n] with ROWS_IN_N
     const uint32_t* __restrict__ wgt;  // [P][h_k][k_or][n_cotile][2][16]
+    const uint32_t* __restrict__ wgt_rail;      // [P][h_k][k_or][n_cotile][16]: the non-zero rail's word per channel
+    const uint32_t* __restrict__ wgt_rail_idx;  // [P][h_k][k_or][n_cotile][4]: one byte per channel, see k_rail_pack
     int32_t* __restrict__ y;           // [n][c_out][wo][ho]
     int n, c_in, wi, hi, c_out, w_k, h_k, packs;
     int wo, ho, n_cotile;
@@ -617,6 +619,166 @@ __global__ __launch_bounds__(64) void k_conv_fwd_thin(FwdParams q)
         atomicAdd(q.y + (((size_t)n * q.c_out + co) * q.wo + a) * q.ho + b, mine);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Rail-skipping kernel for the plain y-mode launches.
+//
+// A weight has at most one non-zero code (wp = code of clamp(w, 0, .), wn = code of -clamp(w, ., 0),
+// sc.cpp:301-304), and a zero code gives an all-zero stream: of the two v_and_or_b32 that
+// k_conv_fwd issues per (activation word, weight), one always ORs zeros.  Which one is uniform
+// over the wave but varies per (member, channel), so it cannot select a register at compile time;
+// gfx9's VGPR index mode can at run time: with s_set_gpr_idx_on(SRC2, DST) the accumulator operand of
+// every following VALU instruction is offset by M0[7:0], one s_set_gpr_idx_idx per (member,
+// channel) points the same two v_and_or_b32 (two rows) at the channel's positive or negative
+// accumulators.  The scalar instructions issue beside the vector ones (measured: one index update
+// per v_and_or_b32 leaves the vector rate unchanged), so the kernel executes half of k_conv_fwd's
+// vector instructions.
+//
+// The 64 OR accumulators sit in fixed registers v[64:127]: P[c][r] = v[64 + 2 c + r],
+// N[c][r] = v[96 + 2 c + r].  The index byte of a channel is 2 c (positive rail or zero weight) or
+// 32 + 2 c (negative rail); the asm blocks name v64 / v65 and the index does the rest.  The
+// compiler sees the four 16-register vectors as read and written by every block and keeps them
+// in place.  Index mode is switched off at the end of every block: compiler-generated vector
+// instructions in between must not be indexed.
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+
+#define GEO_SC_RAIL_PAIR(W, SET)                                                                                       \
+    SET "v_and_or_b32 v64, %[" W "], %[a0], v64\n"                                                                     \
+        "v_and_or_b32 v65, %[" W "], %[a1], v65\n"
+#define GEO_SC_RAIL_IDX0(I) "s_set_gpr_idx_idx %[" I "]\n"
+#define GEO_SC_RAIL_IDXS(I, SH) "s_lshr_b32 %[t], %[" I "], " #SH "\ns_set_gpr_idx_idx %[t]\n"
+
+// one weight line (16 channels) against the two activation words of the lane's two rows
+__device__ __forceinline__ void rail_line(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1, const uint32_t (&w)[kCoTile],
+                                          const uint32_t (&ix)[kCoTile / 4], uint32_t a0, uint32_t a1)
+{
+    uint32_t t;
+    // not volatile: every effect goes through the operands, and a volatile asm would count as a possible
+    // store, after which the compiler no longer reads the weight lines with scalar loads
+    asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n"
+        GEO_SC_RAIL_PAIR("w0", "") GEO_SC_RAIL_PAIR("w1", GEO_SC_RAIL_IDXS("i0", 8))
+        GEO_SC_RAIL_PAIR("w2", GEO_SC_RAIL_IDXS("i0", 16)) GEO_SC_RAIL_PAIR("w3", GEO_SC_RAIL_IDXS("i0", 24))
+        GEO_SC_RAIL_PAIR("w4", GEO_SC_RAIL_IDX0("i1")) GEO_SC_RAIL_PAIR("w5", GEO_SC_RAIL_IDXS("i1", 8))
+        GEO_SC_RAIL_PAIR("w6", GEO_SC_RAIL_IDXS("i1", 16)) GEO_SC_RAIL_PAIR("w7", GEO_SC_RAIL_IDXS("i1", 24))
+        GEO_SC_RAIL_PAIR("w8", GEO_SC_RAIL_IDX0("i2")) GEO_SC_RAIL_PAIR("w9", GEO_SC_RAIL_IDXS("i2", 8))
+        GEO_SC_RAIL_PAIR("w10", GEO_SC_RAIL_IDXS("i2", 16)) GEO_SC_RAIL_PAIR("w11", GEO_SC_RAIL_IDXS("i2", 24))
+        GEO_SC_RAIL_PAIR("w12", GEO_SC_RAIL_IDX0("i3")) GEO_SC_RAIL_PAIR("w13", GEO_SC_RAIL_IDXS("i3", 8))
+        GEO_SC_RAIL_PAIR("w14", GEO_SC_RAIL_IDXS("i3", 16)) GEO_SC_RAIL_PAIR("w15", GEO_SC_RAIL_IDXS("i3", 24))
+        "s_set_gpr_idx_off\n"
+        : "+{v[64:79]}"(p0), "+{v[80:95]}"(p1), "+{v[96:111]}"(n0), "+{v[112:127]}"(n1), [t] "=&s"(t)
+        : [w0] "s"(w[0]), [w1] "s"(w[1]), [w2] "s"(w[2]), [w3] "s"(w[3]), [w4] "s"(w[4]), [w5] "s"(w[5]), [w6] "s"(w[6]),
+          [w7] "s"(w[7]), [w8] "s"(w[8]), [w9] "s"(w[9]), [w10] "s"(w[10]), [w11] "s"(w[11]), [w12] "s"(w[12]),
+          [w13] "s"(w[13]), [w14] "s"(w[14]), [w15] "s"(w[15]), [i0] "s"(ix[0]), [i1] "s"(ix[1]), [i2] "s"(ix[2]),
+          [i3] "s"(ix[3]), [a0] "v"(a0), [a1] "v"(a1)
+        : "m0", "scc");
+}
+#undef GEO_SC_RAIL_PAIR
+#undef GEO_SC_RAIL_IDX0
+#undef GEO_SC_RAIL_IDXS
+static_assert(kCoTile == 16, "rail_line is written for tiles of 16 output channels");
+
+// Two output rows per lane (R = 2), position-major activation streams, kernel extent WK in dim 2.
+// Same lane -> position mapping, grid and result as k_conv_fwd<2, WK, 1, false>.
+template <int WK>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_rail(FwdParams q)
+{
+    constexpr int C = kCoTile, R = 2, NW = R + WK - 1;
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long slot0 = (long long)(blockIdx.x / q.n_cotile) * 64 + threadIdx.x;
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : 0;
+    const int b = (int)(slot % q.ho);
+    const long long t = slot / q.ho;
+    const int a0 = (int)(t % q.row_groups) * R;
+    const long long n = t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
+    // word offsets inside one channel plane; rows past the end (partial last group) are clamped to
+    // valid ones: they only feed outputs that are never stored
+    unsigned off[NW];
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+        const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+        off[j] = (unsigned)row * q.hi;
+    }
+    const unsigned ch_stride = (unsigned)q.wi * q.hi;
+    const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
+    const int k_or = q.c_in * q.w_k;
+    const unsigned k_stride = (unsigned)q.n_cotile * C, ki_stride = (unsigned)q.n_cotile * (C / 4);
+
+    int sum[2 * C];  // [2 c + r]
+#pragma unroll
+    for (int i = 0; i < 2 * C; i++) sum[i] = 0;
+
+    for (int p = 0; p < q.packs; p++) {
+        for (int v = 0; v < q.h_k; v++) {
+            u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
+            const uint32_t* ap = act_n + (size_t)p * q.act_plane + v;
+            const size_t line0 = (size_t)(p * q.h_k + v) * k_or * q.n_cotile + cot;
+            const uint32_t* wp = q.wgt_rail + line0 * C;
+            const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 4);
+            for (int ci = 0; ci < q.c_in; ci++) {
+                uint32_t aw[NW];
+#pragma unroll
+                for (int j = 0; j < NW; j++) aw[j] = ap[off[j]];
+                uint32_t wv[WK][C], iv[WK][C / 4];
+#pragma unroll
+                for (int u = 0; u < WK; u++) {
+#pragma unroll
+                    for (int c = 0; c < C; c++) wv[u][c] = wp[u * k_stride + c];
+#pragma unroll
+                    for (int c = 0; c < C / 4; c++) iv[u][c] = ip[u * ki_stride + c];
+                }
+#pragma unroll
+                for (int u = 0; u < WK; u++) rail_line(p0, p1, n0, n1, wv[u], iv[u], aw[u], aw[u + 1]);
+                wp += WK * k_stride;
+                ip += WK * ki_stride;
+                ap += ch_stride;
+            }
+            // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
+#pragma unroll
+            for (int i = 0; i < C; i++) {
+                sum[i] += __popc(p0[i]) - __popc(n0[i]);
+                sum[C + i] += __popc(p1[i]) - __popc(n1[i]);
+            }
+        }
+    }
+
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const int co = cot * C + c;
+        if (co >= q.c_out) break;
+        int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[2 * c + r];
+    }
+}
+
+// Rail-packed weight lines from the two-rail lines: word = pos | neg (at most one is non-zero),
+// index byte of channel c = 2 c for the positive rail (and for zero weights), 32 + 2 c for the
+// negative one: the register offsets k_conv_fwd_rail feeds to s_set_gpr_idx_idx.  One thread per line.
+__global__ __launch_bounds__(256) void k_rail_pack(const uint32_t* __restrict__ lines2, uint32_t* __restrict__ words,
+                                                   uint32_t* __restrict__ idx, size_t n_lines)
+{
+    constexpr int C = kCoTile;
+    for (size_t l = (size_t)blockIdx.x * 256 + threadIdx.x; l < n_lines; l += (size_t)gridDim.x * 256) {
+        const uint32_t* src = lines2 + l * 2 * C;
+        uint32_t packed[C / 4];
+#pragma unroll
+        for (int c4 = 0; c4 < C / 4; c4++) packed[c4] = 0;
+#pragma unroll
+        for (int c = 0; c < C; c++) {
+            const uint32_t wp = src[c], wn = src[C + c];
+            words[l * C + c] = wp | wn;
+            const uint32_t byte = (wn != 0u ? 2u * C : 0u) + 2u * c;
+            packed[c >> 2] |= byte << (8 * (c & 3));
+        }
+#pragma unroll
+        for (int c4 = 0; c4 < C / 4; c4++) idx[l * (C / 4) + c4] = packed[c4];
+    }
+}
+
 __global__ __launch_bounds__(256) void k_zero_i32(int32_t* __restrict__ p, size_t n)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0;
@@ -663,6 +825,11 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         else
             hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, false>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
                                0, s, q);
+    } else if (g.rail) {
+        if constexpr (R == 2 && !ROWS_IN_N && WK > 0)
+            hipLaunchKernelGGL((k_conv_fwd_rail<WK>), dim3((unsigned)blocks), dim3(64), 0, s, q);
+        else
+            return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail for these launches only
     } else
         hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks), dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
@@ -670,11 +837,23 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
 
 }  // namespace
 
+int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s)
+{
+    if (!g.rail) return GEO_SC_OK;
+    const size_t lines = (size_t)g.packs * g.h_k * g.k_or * g.n_cotile;
+    size_t blocks = (lines + 255) / 256;
+    hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,
+                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s)
 {
     FwdParams q;
     q.act = act;
     q.wgt = wgt;
+    q.wgt_rail = g.rail ? wgt + g.wgt_rail_off : nullptr;
+    q.wgt_rail_idx = g.rail ? wgt + g.wgt_rail_idx_off : nullptr;
     q.y = y;
     q.c_in = g.c_in;
     q.wi = g.wi;

@@ -157,6 +157,11 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, c
  * c_out (sc.cpp:336-388, sc_cuda_kernel.cu:91-170).  Modes Z and YZ keep the line format and
  * order the lines by (pack, add group, OR member): Z [P][c_in][h_k*w_k] with member
  * h_index*w_k + w_index; YZ [P][channel group][h_k][channels of the group * w_k].
+ * A weight has at most one non-zero rail (its codes are those of clamp(w, 0, .) and
+ * -clamp(w, ., 0), sc.cpp:301-304).  For large y-mode layers the buffer continues behind these
+ * lines with a second, rail-packed copy that the convolution kernel reads there (per line 16
+ * words pos | neg, then per line 4 words holding one byte per channel: which rail);
+ * geo_sc_weight_stream_words is the size of the whole buffer, geo_sc_weight_streams fills all of it.
  *
  * `tables` is scratch of geo_sc_stream_tables_size(L) bytes.
  */
@@ -169,6 +174,7 @@ GEO_SC_API int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* 
  * The AND / OR / popcount kernel alone, on streams in the two layouts above (what the
  * forward runs after its generators; the body of stream_compute_add_direct_variable,
  * sc_cuda_kernel.cu:693-1002, and of matmul_outer, sc.cpp:12-259).  y is fully overwritten.
+ * weight_streams is a buffer of geo_sc_weight_stream_words words as geo_sc_weight_streams fills it.
  */
 GEO_SC_API int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,
                                                       const uint32_t* weight_streams, int32_t* y,
