@@ -113,7 +113,7 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     if (g->rail) {
         g->wgt_rail_off = (g->wgt_words + 63) & ~(size_t)63;
         g->wgt_rail_idx_off = g->wgt_rail_off + lines * kCoTile;
-        g->wgt_words = g->wgt_rail_idx_off + lines * (kCoTile / 4);
+        g->wgt_words = g->wgt_rail_idx_off + lines * (kCoTile / 2);
     }
     g->off_tables = 0;
     g->off_wgt = align256(table_bytes(g->L));

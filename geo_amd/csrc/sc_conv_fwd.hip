@@ -21,8 +21,8 @@ namespace {
 struct FwdParams {
     const uint32_t* __restrict__ act;  // [n][P][c_in][wi][hi], or [P][c_in][wi][hi][n] with ROWS_IN_N
     const uint32_t* __restrict__ wgt;  // [P][h_k][k_or][n_cotile][2][16]
-    const uint32_t* __restrict__ wgt_rail;      // [P][h_k][k_or][n_cotile][16]: the non-zero rail's word per channel
-    const uint32_t* __restrict__ wgt_rail_idx;  // [P][h_k][k_or][n_cotile][4]: one byte per channel, see k_rail_pack
+    const uint32_t* __restrict__ wgt_rail;      // [P][h_k][n_cotile][k_or][16]: the non-zero rail's word per channel
+    const uint32_t* __restrict__ wgt_rail_idx;  // [P][h_k][n_cotile][k_or][8]: a 16-bit field per channel, see k_rail_pack
     int32_t* __restrict__ y;           // [n][c_out][wo][ho]
     int n, c_in, wi, hi, c_out, w_k, h_k, packs;
     int wo, ho, n_cotile;
@@ -627,15 +627,18 @@ __global__ __launch_bounds__(64) void k_conv_fwd_thin(FwdParams q)
 // k_conv_fwd issues per (activation word, weight), one always ORs zeros.  Which one is uniform
 // over the wave but varies per (member, channel), so it cannot select a register at compile time;
 // gfx9's VGPR index mode can at run time: with s_set_gpr_idx_on(SRC2, DST) the accumulator operand of
-// every following VALU instruction is offset by M0[7:0], one s_set_gpr_idx_idx per (member,
+// every following VALU instruction is offset by M0[7:0], one M0 update per (member,
 // channel) points the same two v_and_or_b32 (two rows) at the channel's positive or negative
 // accumulators.  The scalar instructions issue beside the vector ones (measured: one index update
 // per v_and_or_b32 leaves the vector rate unchanged), so the kernel executes half of k_conv_fwd's
 // vector instructions.
 //
 // The 64 OR accumulators sit in fixed registers v[64:127]: P[c][r] = v[64 + 2 c + r],
-// N[c][r] = v[96 + 2 c + r].  The index byte of a channel is 2 c (positive rail or zero weight) or
-// 32 + 2 c (negative rail); the asm blocks name v64 / v65 and the index does the rest.  The
+// N[c][r] = v[96 + 2 c + r].  The index of a channel is 2 c (positive rail or zero weight) or
+// 32 + 2 c (negative rail); the asm blocks name v64 / v65 and the index does the rest.  The index
+// arrives as a ready-made 16-bit M0 value per channel (index and the two operand enables), so one
+// scalar instruction per channel moves it into M0 (s_and_b32 / s_lshr_b32 on a word that holds two
+// of them; same effect as s_set_gpr_idx_idx, without a separate shift).  The
 // compiler sees the four 16-register vectors as read and written by every block and keeps them
 // in place.  Index mode is switched off at the end of every block: compiler-generated vector
 // instructions in between must not be indexed.
@@ -644,36 +647,36 @@ typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 #define GEO_SC_RAIL_PAIR(W, SET)                                                                                       \
     SET "v_and_or_b32 v64, %[" W "], %[a0], v64\n"                                                                     \
         "v_and_or_b32 v65, %[" W "], %[a1], v65\n"
-#define GEO_SC_RAIL_IDX0(I) "s_set_gpr_idx_idx %[" I "]\n"
-#define GEO_SC_RAIL_IDXS(I, SH) "s_lshr_b32 %[t], %[" I "], " #SH "\ns_set_gpr_idx_idx %[t]\n"
+// M0 of a channel from its 16-bit field: index in bits 7:0, the SRC2 and DST enables in bits 15:12
+#define GEO_SC_RAIL_LO(I) "s_and_b32 m0, %[" I "], 0xffff\n"
+#define GEO_SC_RAIL_HI(I) "s_lshr_b32 m0, %[" I "], 16\n"
 
 // one weight line (16 channels) against the two activation words of the lane's two rows
 __device__ __forceinline__ void rail_line(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1, const uint32_t (&w)[kCoTile],
-                                          const uint32_t (&ix)[kCoTile / 4], uint32_t a0, uint32_t a1)
+                                          const uint32_t (&ix)[kCoTile / 2], uint32_t a0, uint32_t a1)
 {
-    uint32_t t;
     // not volatile: every effect goes through the operands, and a volatile asm would count as a possible
     // store, after which the compiler no longer reads the weight lines with scalar loads
     asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n"
-        GEO_SC_RAIL_PAIR("w0", "") GEO_SC_RAIL_PAIR("w1", GEO_SC_RAIL_IDXS("i0", 8))
-        GEO_SC_RAIL_PAIR("w2", GEO_SC_RAIL_IDXS("i0", 16)) GEO_SC_RAIL_PAIR("w3", GEO_SC_RAIL_IDXS("i0", 24))
-        GEO_SC_RAIL_PAIR("w4", GEO_SC_RAIL_IDX0("i1")) GEO_SC_RAIL_PAIR("w5", GEO_SC_RAIL_IDXS("i1", 8))
-        GEO_SC_RAIL_PAIR("w6", GEO_SC_RAIL_IDXS("i1", 16)) GEO_SC_RAIL_PAIR("w7", GEO_SC_RAIL_IDXS("i1", 24))
-        GEO_SC_RAIL_PAIR("w8", GEO_SC_RAIL_IDX0("i2")) GEO_SC_RAIL_PAIR("w9", GEO_SC_RAIL_IDXS("i2", 8))
-        GEO_SC_RAIL_PAIR("w10", GEO_SC_RAIL_IDXS("i2", 16)) GEO_SC_RAIL_PAIR("w11", GEO_SC_RAIL_IDXS("i2", 24))
-        GEO_SC_RAIL_PAIR("w12", GEO_SC_RAIL_IDX0("i3")) GEO_SC_RAIL_PAIR("w13", GEO_SC_RAIL_IDXS("i3", 8))
-        GEO_SC_RAIL_PAIR("w14", GEO_SC_RAIL_IDXS("i3", 16)) GEO_SC_RAIL_PAIR("w15", GEO_SC_RAIL_IDXS("i3", 24))
+        GEO_SC_RAIL_PAIR("w0", "") GEO_SC_RAIL_PAIR("w1", GEO_SC_RAIL_HI("i0"))
+        GEO_SC_RAIL_PAIR("w2", GEO_SC_RAIL_LO("i1")) GEO_SC_RAIL_PAIR("w3", GEO_SC_RAIL_HI("i1"))
+        GEO_SC_RAIL_PAIR("w4", GEO_SC_RAIL_LO("i2")) GEO_SC_RAIL_PAIR("w5", GEO_SC_RAIL_HI("i2"))
+        GEO_SC_RAIL_PAIR("w6", GEO_SC_RAIL_LO("i3")) GEO_SC_RAIL_PAIR("w7", GEO_SC_RAIL_HI("i3"))
+        GEO_SC_RAIL_PAIR("w8", GEO_SC_RAIL_LO("i4")) GEO_SC_RAIL_PAIR("w9", GEO_SC_RAIL_HI("i4"))
+        GEO_SC_RAIL_PAIR("w10", GEO_SC_RAIL_LO("i5")) GEO_SC_RAIL_PAIR("w11", GEO_SC_RAIL_HI("i5"))
+        GEO_SC_RAIL_PAIR("w12", GEO_SC_RAIL_LO("i6")) GEO_SC_RAIL_PAIR("w13", GEO_SC_RAIL_HI("i6"))
+        GEO_SC_RAIL_PAIR("w14", GEO_SC_RAIL_LO("i7")) GEO_SC_RAIL_PAIR("w15", GEO_SC_RAIL_HI("i7"))
         "s_set_gpr_idx_off\n"
-        : "+{v[64:79]}"(p0), "+{v[80:95]}"(p1), "+{v[96:111]}"(n0), "+{v[112:127]}"(n1), [t] "=&s"(t)
+        : "+{v[64:79]}"(p0), "+{v[80:95]}"(p1), "+{v[96:111]}"(n0), "+{v[112:127]}"(n1)
         : [w0] "s"(w[0]), [w1] "s"(w[1]), [w2] "s"(w[2]), [w3] "s"(w[3]), [w4] "s"(w[4]), [w5] "s"(w[5]), [w6] "s"(w[6]),
           [w7] "s"(w[7]), [w8] "s"(w[8]), [w9] "s"(w[9]), [w10] "s"(w[10]), [w11] "s"(w[11]), [w12] "s"(w[12]),
           [w13] "s"(w[13]), [w14] "s"(w[14]), [w15] "s"(w[15]), [i0] "s"(ix[0]), [i1] "s"(ix[1]), [i2] "s"(ix[2]),
-          [i3] "s"(ix[3]), [a0] "v"(a0), [a1] "v"(a1)
+          [i3] "s"(ix[3]), [i4] "s"(ix[4]), [i5] "s"(ix[5]), [i6] "s"(ix[6]), [i7] "s"(ix[7]), [a0] "v"(a0), [a1] "v"(a1)
         : "m0", "scc");
 }
 #undef GEO_SC_RAIL_PAIR
-#undef GEO_SC_RAIL_IDX0
-#undef GEO_SC_RAIL_IDXS
+#undef GEO_SC_RAIL_LO
+#undef GEO_SC_RAIL_HI
 static_assert(kCoTile == 16, "rail_line is written for tiles of 16 output channels");
 
 // Two output rows per lane (R = 2), position-major activation streams, kernel extent WK in dim 2.
@@ -702,7 +705,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const unsigned ch_stride = (unsigned)q.wi * q.hi;
     const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
     const int k_or = q.c_in * q.w_k;
-    const unsigned k_stride = (unsigned)q.n_cotile * C, ki_stride = (unsigned)q.n_cotile * (C / 4);
 
     int sum[2 * C];  // [2 c + r]
 #pragma unroll
@@ -712,25 +714,27 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int v = 0; v < q.h_k; v++) {
             u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
             const uint32_t* ap = act_n + (size_t)p * q.act_plane + v;
-            const size_t line0 = (size_t)(p * q.h_k + v) * k_or * q.n_cotile + cot;
+            // rail-packed lines are stored [pack][kernel row][c_out tile][member]: a channel's WK lines
+            // follow each other
+            const size_t line0 = ((size_t)(p * q.h_k + v) * q.n_cotile + cot) * k_or;
             const uint32_t* wp = q.wgt_rail + line0 * C;
-            const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 4);
+            const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
             for (int ci = 0; ci < q.c_in; ci++) {
                 uint32_t aw[NW];
 #pragma unroll
                 for (int j = 0; j < NW; j++) aw[j] = ap[off[j]];
-                uint32_t wv[WK][C], iv[WK][C / 4];
+                uint32_t wv[WK][C], iv[WK][C / 2];
 #pragma unroll
                 for (int u = 0; u < WK; u++) {
 #pragma unroll
-                    for (int c = 0; c < C; c++) wv[u][c] = wp[u * k_stride + c];
+                    for (int c = 0; c < C; c++) wv[u][c] = wp[u * C + c];
 #pragma unroll
-                    for (int c = 0; c < C / 4; c++) iv[u][c] = ip[u * ki_stride + c];
+                    for (int c = 0; c < C / 2; c++) iv[u][c] = ip[u * (C / 2) + c];
                 }
 #pragma unroll
                 for (int u = 0; u < WK; u++) rail_line(p0, p1, n0, n1, wv[u], iv[u], aw[u], aw[u + 1]);
-                wp += WK * k_stride;
-                ip += WK * ki_stride;
+                wp += WK * C;
+                ip += WK * (C / 2);
                 ap += ch_stride;
             }
             // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
@@ -755,27 +759,31 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
 }
 
-// Rail-packed weight lines from the two-rail lines: word = pos | neg (at most one is non-zero),
-// index byte of channel c = 2 c for the positive rail (and for zero weights), 32 + 2 c for the
-// negative one: the register offsets k_conv_fwd_rail feeds to s_set_gpr_idx_idx.  One thread per line.
+// Rail-packed weight lines from the two-rail lines [pv][k][cot][2][16]: word = pos | neg (at most
+// one is non-zero), stored [pv][cot][k][16]; per channel a 16-bit field with what k_conv_fwd_rail
+// moves into M0: bits 7:0 the register offset of the channel's accumulators, 2 c for the positive
+// rail (and for zero weights), 32 + 2 c for the negative one, bits 15:12 the SRC2 and DST enables of
+// the VGPR index mode; stored [pv][cot][k][8].  One thread per line.
 __global__ __launch_bounds__(256) void k_rail_pack(const uint32_t* __restrict__ lines2, uint32_t* __restrict__ words,
-                                                   uint32_t* __restrict__ idx, size_t n_lines)
+                                                   uint32_t* __restrict__ idx, size_t n_lines, int k_or, int n_cotile)
 {
     constexpr int C = kCoTile;
     for (size_t l = (size_t)blockIdx.x * 256 + threadIdx.x; l < n_lines; l += (size_t)gridDim.x * 256) {
+        const size_t cot = l % n_cotile, t = l / n_cotile, k = t % k_or, pv = t / k_or;
+        const size_t dst = (pv * n_cotile + cot) * k_or + k;
         const uint32_t* src = lines2 + l * 2 * C;
-        uint32_t packed[C / 4];
+        uint32_t packed[C / 2];
 #pragma unroll
-        for (int c4 = 0; c4 < C / 4; c4++) packed[c4] = 0;
+        for (int c2 = 0; c2 < C / 2; c2++) packed[c2] = 0;
 #pragma unroll
         for (int c = 0; c < C; c++) {
             const uint32_t wp = src[c], wn = src[C + c];
-            words[l * C + c] = wp | wn;
-            const uint32_t byte = (wn != 0u ? 2u * C : 0u) + 2u * c;
-            packed[c >> 2] |= byte << (8 * (c & 3));
+            words[dst * C + c] = wp | wn;
+            const uint32_t field = 0xC000u | ((wn != 0u ? 2u * C : 0u) + 2u * c);
+            packed[c >> 1] |= field << (16 * (c & 1));
         }
 #pragma unroll
-        for (int c4 = 0; c4 < C / 4; c4++) idx[l * (C / 4) + c4] = packed[c4];
+        for (int c2 = 0; c2 < C / 2; c2++) idx[dst * (C / 2) + c2] = packed[c2];
     }
 }
 
@@ -843,7 +851,7 @@ int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s)
     const size_t lines = (size_t)g.packs * g.h_k * g.k_or * g.n_cotile;
     size_t blocks = (lines + 255) / 256;
     hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,
-                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines);
+                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines, g.k_or, g.n_cotile);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
