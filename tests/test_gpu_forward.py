@@ -1,6 +1,7 @@
 """GPU parity of the HIP forward path, driven through the C ABI (geo_amd.capi) and through
 the PyTorch modules with the reference's names.  Everything is compared bit-for-bit with
 the CPU oracle, the reference-kernel fixtures and the reference-kernel checksums."""
+import ctypes
 import hashlib
 
 import numpy as np
@@ -304,3 +305,44 @@ def test_long_kernels_use_the_row_chunked_weight_generator(capi, so, sx, sw, pad
     assert np.array_equal(got, exp)
     assert np.array_equal(gpu_forward(capi, x, w, L, pad, total_width=7, load_width=2, load_wait_w=2, load_wait_a=2),
                           so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad, 7, 2, 2, 2))
+
+
+# ------------------------------------------------------------------ rail-skipping kernel
+@pytest.mark.parametrize("shape_x,shape_w,pad,L,loading,gen", [
+    ((128, 3, 33, 32), (50, 3, 3, 3), (1, 1), 32, (7, 8, 1, 1), "lfsr"),    # odd row count, partial c_out tile
+    ((128, 3, 32, 32), (50, 3, 3, 3), (1, 1), 64, (7, 2, 2, 2), "lfsr"),    # progressive loading
+    ((136, 2, 32, 31), (64, 2, 5, 5), (2, 2), 16, (7, 8, 1, 1), "lfsr"),    # 5-wide kernel, partly empty last wave
+    ((128, 5, 32, 32), (49, 5, 1, 1), (0, 0), 128, (7, 8, 1, 1), "lfsr"),   # 1 x 1
+    ((128, 4, 32, 32), (65, 4, 3, 2), (1, 0), 8, (7, 8, 1, 1), "lfsr"),     # L = 8, even kernel extent in dim 3
+    ((128, 3, 32, 32), (50, 3, 3, 3), (1, 1), 64, (7, 8, 1, 1), "acc"),     # random generators: same kernel
+])
+def test_large_y_mode_launches_skip_the_zero_rail(capi, so, shape_x, shape_w, pad, L, loading, gen):
+    """Launches of at least 4096 waves in y mode run the kernel that processes only the non-zero rail of
+    every weight (register-indexed accumulators): bit-exact against the oracle, through the whole-op
+    entry point, the uint8 entry point and the stage entry points."""
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_w[0])
+    w = (w * 3).clamp(-1, 1).contiguous()
+    w.view(-1)[::5] = 0.0                                  # zero weights: neither rail
+    tw, lw, ww, wa = loading
+    d = capi.make_desc(x.shape, w.shape, L, pad, tw, lw, ww, wa, generator=gen, seed=11)
+    n_words = ctypes.c_size_t(0)
+    from geo_amd import _native
+    assert _native.lib().geo_sc_weight_stream_words(ctypes.byref(d), ctypes.byref(n_words)) == 0
+    P, (Cout, Cin, W, H) = (L + 31) // 32, w.shape
+    assert n_words.value > P * H * Cin * W * ((Cout + 15) // 16) * 32   # the buffer carries the rail-packed copy
+    if gen == "lfsr":
+        exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad, tw, lw, ww, wa)
+    else:
+        exp = so.conv2d_general(x.numpy(), w.numpy(), L, pad, "y", 1, gen, 11)
+    y = capi.conv2d_add_partial_forward(x.cuda(), w.cuda(), L, pad, tw, lw, ww, wa, generator=gen, seed=11)
+    assert np.array_equal(y.cpu().numpy(), exp)
+    y2 = capi.conv2d_add_partial_from_streams(capi.act_streams(x.cuda(), d), capi.weight_streams(w.cuda(), d), d)
+    assert torch.equal(y2, y)
+    if gen == "lfsr":
+        xq = (x * 128).round().to(torch.uint8).cuda()
+        y3 = capi.conv2d_add_partial_forward_q7(xq, w.cuda(), L, pad, tw, lw, ww, wa)
+        assert torch.equal(y3, y)
+    # a buffer without the rail-packed copy is refused by the Python binding
+    with pytest.raises(ValueError):
+        short = torch.zeros(P * H * Cin * W * ((Cout + 15) // 16) * 32, dtype=torch.int32, device="cuda")
+        capi.conv2d_add_partial_from_streams(capi.act_streams(x.cuda(), d), short, d)
