@@ -52,6 +52,7 @@ C_API = {
                                [_P] * 7),
     "geo_sc_conv2d_add_partial_forward_q7": (ctypes.c_int, [_D, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_quantize": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, _P]),
+    "geo_sc_weight_streams_finish": (ctypes.c_int, [_D, _P, _P]),
 }
 
 _lib = None

@@ -250,6 +250,31 @@ def weight_streams(w, desc: ConvDesc, stream=None):
     return out
 
 
+def weight_streams_from_lines(lines, desc: ConvDesc, stream=None):
+    """A complete weight stream buffer from two-rail lines [P][H][K][ceil(Cout/16)][2][16] written by the
+    caller (int32-typed GPU tensor): copies them into a buffer of geo_sc_weight_stream_words words and
+    lets geo_sc_weight_streams_finish fill the rest.  Returns the view of the lines, as weight_streams()."""
+    n = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
+    if not (lines.is_cuda and lines.dtype == torch.int32 and lines.is_contiguous()) or lines.numel() > n.value:
+        raise ValueError("lines must be a contiguous int32 GPU tensor of the two-rail layout")
+    buf = torch.empty(n.value, dtype=torch.int32, device=lines.device)
+    out = buf[:lines.numel()].view(lines.shape)
+    out.copy_(lines)
+    _check(_native.lib().geo_sc_weight_streams_finish(ctypes.byref(desc), _ptr(out), _stream_ptr(stream)),
+           "geo_sc_weight_streams_finish")
+    return out
+
+
+def skips_zero_rail(desc: ConvDesc) -> bool:
+    """True when the forward of this geometry runs the kernel that processes only the non-zero rail
+    of every weight (its weight stream buffer then carries the rail-packed copy)."""
+    n = ctypes.c_size_t(0)
+    _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
+    packs = (desc.bit_length + 31) // 32
+    return n.value > packs * desc.h_k * desc.c_in * desc.w_k * ((desc.c_out + 15) // 16) * 32
+
+
 def conv2d_add_partial_from_streams(act, wgt, desc: ConvDesc, out=None, stream=None):
     """The AND/OR/popcount kernel alone on pre-generated streams (int32-typed words)."""
     if out is None:

@@ -100,20 +100,17 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     }
     g->act_item_inner = !g->thin && g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
-    {
-        // the same count of waves launch_conv_forward sees for two output rows per lane
-        const long long row_groups = (wo + 1) / 2;
-        const long long waves = (((long long)d->n * row_groups * ho + 63) / 64) * g->n_cotile;
-        g->rail = g->mode == GEO_SC_ACC_Y && !g->thin && !g->act_item_inner && wo >= 2 &&
-                  (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) && waves >= 4096;
-    }
-    const size_t lines = (size_t)g->packs * d->h_k * g->k_or * g->n_cotile;
-    g->wgt_words = lines * 2 * kCoTile;
+    // two output rows per lane, compile-time kernel extent in dim 2, position-major streams: the
+    // launches launch_conv_forward gives to the rail-skipping kernels
+    g->rail = !g->thin && !g->act_item_inner && wo >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5);
+    const size_t lines = (size_t)g->packs * d->h_k * g->k_or;
+    g->wgt_words = lines * g->n_cotile * 2 * kCoTile;
     g->wgt_rail_off = g->wgt_rail_idx_off = 0;
+    g->wgt_rail_lines = lines;
     if (g->rail) {
         g->wgt_rail_off = (g->wgt_words + 63) & ~(size_t)63;
-        g->wgt_rail_idx_off = g->wgt_rail_off + lines * kCoTile;
-        g->wgt_words = g->wgt_rail_idx_off + lines * (kCoTile / 2);
+        g->wgt_rail_idx_off = g->wgt_rail_off + lines * g->n_cotile * kCoTile;
+        g->wgt_words = g->wgt_rail_idx_off + lines * g->n_cotile * (kCoTile / 2);
     }
     g->off_tables = 0;
     g->off_wgt = align256(table_bytes(g->L));
@@ -249,6 +246,15 @@ int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t
     rc = launch_weight_streams(g, w, streams, (const uint32_t*)tables, s);
     if (rc != GEO_SC_OK) return rc;
     return launch_rail_pack(g, streams, s);
+}
+
+int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams, geo_sc_stream_t stream)
+{
+    Geometry g;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!streams) return GEO_SC_ERR_INVALID_ARGUMENT;
+    return launch_rail_pack(g, streams, (hipStream_t)stream);
 }
 
 int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,

@@ -47,11 +47,12 @@ struct Geometry {
     // Weight stream buffer: lines [packs][h_k][k_or][n_cotile] of 2 x kCoTile words (both rails), then,
     // with rail, the same lines once more in the rail-packed form the plain y-mode kernel reads:
     // at wgt_rail_off kCoTile words per line (the non-zero rail's word), at wgt_rail_idx_off
-    // kCoTile / 2 words per line (16 bits per channel: which rail), lines ordered
-    // [packs][h_k][n_cotile][k_or].
-    size_t wgt_words, wgt_rail_off, wgt_rail_idx_off;
-    // Large y-mode launches run the rail-skipping kernel: per weight at most one rail's stream
-    // is non-zero (codes of clamp(w, 0, .) and -clamp(w, ., 0)), and only that rail is processed.
+    // kCoTile / 2 words per line (16 bits per channel: which rail), both ordered [n_cotile][line]
+    // with wgt_rail_lines lines per tile.
+    size_t wgt_words, wgt_rail_off, wgt_rail_idx_off, wgt_rail_lines;
+    // Position-major launches with two output rows per lane run the rail-skipping kernels: per weight
+    // at most one rail's stream is non-zero (codes of clamp(w, 0, .) and -clamp(w, ., 0)), and only
+    // that rail is processed.
     bool rail;
     // workspace carve-up (byte offsets, 256-aligned)
     size_t off_tables, off_wgt, off_act, ws_bytes;

@@ -21,8 +21,9 @@ namespace {
 struct FwdParams {
     const uint32_t* __restrict__ act;  // [n][P][c_in][wi][hi], or [P][c_in][wi][hi][n] with ROWS_IN_N
     const uint32_t* __restrict__ wgt;  // [P][h_k][k_or][n_cotile][2][16]
-    const uint32_t* __restrict__ wgt_rail;      // [P][h_k][n_cotile][k_or][16]: the non-zero rail's word per channel
-    const uint32_t* __restrict__ wgt_rail_idx;  // [P][h_k][n_cotile][k_or][8]: a 16-bit field per channel, see k_rail_pack
+    const uint32_t* __restrict__ wgt_rail;      // [n_cotile][line][16]: the non-zero rail's word per channel
+    const uint32_t* __restrict__ wgt_rail_idx;  // [n_cotile][line][8]: a 16-bit field per channel, see k_rail_pack
+    size_t rail_lines;                          // lines per c_out tile: P * lines per pack
     int32_t* __restrict__ y;           // [n][c_out][wo][ho]
     int n, c_in, wi, hi, c_out, w_k, h_k, packs;
     int wo, ho, n_cotile;
@@ -714,9 +715,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int v = 0; v < q.h_k; v++) {
             u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
             const uint32_t* ap = act_n + (size_t)p * q.act_plane + v;
-            // rail-packed lines are stored [pack][kernel row][c_out tile][member]: a channel's WK lines
-            // follow each other
-            const size_t line0 = ((size_t)(p * q.h_k + v) * q.n_cotile + cot) * k_or;
+            // rail-packed lines are stored [c_out tile][line]: the lines of a tile follow each other in
+            // the order the loops consume them
+            const size_t line0 = (size_t)cot * q.rail_lines + (size_t)(p * q.h_k + v) * k_or;
             const uint32_t* wp = q.wgt_rail + line0 * C;
             const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
             for (int ci = 0; ci < q.c_in; ci++) {
@@ -759,18 +760,103 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
 }
 
-// Rail-packed weight lines from the two-rail lines [pv][k][cot][2][16]: word = pos | neg (at most
-// one is non-zero), stored [pv][cot][k][16]; per channel a 16-bit field with what k_conv_fwd_rail
-// moves into M0: bits 7:0 the register offset of the channel's accumulators, 2 c for the positive
-// rail (and for zero weights), 32 + 2 c for the negative one, bits 15:12 the SRC2 and DST enables of
-// the VGPR index mode; stored [pv][cot][k][8].  One thread per line.
+// The rail-skipping form of k_conv_fwd_split<2, WK, 1, false>: launches split over blockIdx.y and
+// the accumulation modes other than y, position-major activation streams, two output rows per lane.
+// Partial sums are added to the zeroed y with integer atomics.
+template <int WK>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_split_rail(FwdParams q)
+{
+    constexpr int C = kCoTile, R = 2, NW = R + WK - 1;
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long slot0 = (long long)(blockIdx.x / q.n_cotile) * 64 + threadIdx.x;
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : 0;
+    const int b = (int)(slot % q.ho);
+    const long long t = slot / q.ho;
+    const int a0 = (int)(t % q.row_groups) * R;
+    const long long n = t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
+    unsigned off[NW];
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+        const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+        off[j] = (unsigned)row * q.hi;
+    }
+    const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
+
+    int sum[2 * C];  // [2 c + r]
+#pragma unroll
+    for (int i = 0; i < 2 * C; i++) sum[i] = 0;
+
+    const int groups = q.add_outer * q.add_inner;
+    const int pv_begin = blockIdx.y * q.pv_per_block;
+    const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
+    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    for (int pv = pv_begin; pv < pv_end; pv++) {
+        const int p = pv / groups, g = pv - p * groups;
+        const int go = g / q.add_inner, gi = g - go * q.add_inner;
+        const int ch0 = go * q.or_ch_per_group;
+        const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
+        u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
+        const uint32_t* ap0 = act_n + (size_t)p * q.act_plane + (size_t)gi * q.add_stride + (size_t)ch0 * q.or_stride;
+        const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
+                            (size_t)gi * chs * q.w_k;
+        const uint32_t* wp = q.wgt_rail + line * C;
+        const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
+        for (int row = 0; row < q.or_rows; row++) {
+            const uint32_t* ap = ap0 + row;  // next kernel row: one word further
+            for (int ci = 0; ci < chs; ci++) {
+                uint32_t aw[NW];
+#pragma unroll
+                for (int j = 0; j < NW; j++) aw[j] = ap[off[j]];
+                uint32_t wv[WK][C], iv[WK][C / 2];
+#pragma unroll
+                for (int u = 0; u < WK; u++) {
+#pragma unroll
+                    for (int c = 0; c < C; c++) wv[u][c] = wp[u * C + c];
+#pragma unroll
+                    for (int c = 0; c < C / 2; c++) iv[u][c] = ip[u * (C / 2) + c];
+                }
+#pragma unroll
+                for (int u = 0; u < WK; u++) rail_line(p0, p1, n0, n1, wv[u], iv[u], aw[u], aw[u + 1]);
+                wp += WK * C;
+                ip += WK * (C / 2);
+                ap += q.or_stride;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            sum[i] += __popc(p0[i]) - __popc(n0[i]);
+            sum[C + i] += __popc(p1[i]) - __popc(n1[i]);
+        }
+    }
+
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const int co = cot * C + c;
+        if (co >= q.c_out) break;
+        int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (a0 + r < q.wo) atomicAdd(yo + (size_t)r * q.ho, sum[2 * c + r]);  // integer adds: order does not matter
+    }
+}
+
+// Rail-packed weight lines from the two-rail lines [line][cot][2][16]: word = pos | neg (at most one
+// is non-zero), stored [cot][line][16]; per channel a 16-bit field with what the rail kernels move
+// into M0: bits 7:0 the register offset of the channel's accumulators, 2 c for the positive rail
+// (and for zero weights), 32 + 2 c for the negative one, bits 15:12 the SRC2 and DST enables of
+// the VGPR index mode; stored [cot][line][8].  One thread per (line, tile).
 __global__ __launch_bounds__(256) void k_rail_pack(const uint32_t* __restrict__ lines2, uint32_t* __restrict__ words,
-                                                   uint32_t* __restrict__ idx, size_t n_lines, int k_or, int n_cotile)
+                                                   uint32_t* __restrict__ idx, size_t n_lines, int n_cotile)
 {
     constexpr int C = kCoTile;
-    for (size_t l = (size_t)blockIdx.x * 256 + threadIdx.x; l < n_lines; l += (size_t)gridDim.x * 256) {
-        const size_t cot = l % n_cotile, t = l / n_cotile, k = t % k_or, pv = t / k_or;
-        const size_t dst = (pv * n_cotile + cot) * k_or + k;
+    const size_t total = n_lines * n_cotile;
+    for (size_t l = (size_t)blockIdx.x * 256 + threadIdx.x; l < total; l += (size_t)gridDim.x * 256) {
+        const size_t cot = l % n_cotile, line = l / n_cotile;
+        const size_t dst = cot * n_lines + line;
         const uint32_t* src = lines2 + l * 2 * C;
         uint32_t packed[C / 2];
 #pragma unroll
@@ -830,7 +916,13 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         if constexpr (ROWS_IN_N)
             hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>), dim3((unsigned)blocks, (unsigned)splits),
                                dim3(64), 0, s, q);
-        else
+        else if (g.rail) {
+            if constexpr (R == 2 && WK > 0)
+                hipLaunchKernelGGL((k_conv_fwd_split_rail<WK>), dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s,
+                                   q);
+            else
+                return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail for these launches only
+        } else
             hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, false>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
                                0, s, q);
     } else if (g.rail) {
@@ -848,10 +940,10 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s)
 {
     if (!g.rail) return GEO_SC_OK;
-    const size_t lines = (size_t)g.packs * g.h_k * g.k_or * g.n_cotile;
-    size_t blocks = (lines + 255) / 256;
+    const size_t lines = g.wgt_rail_lines;
+    size_t blocks = (lines * g.n_cotile + 255) / 256;
     hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,
-                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines, g.k_or, g.n_cotile);
+                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines, g.n_cotile);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
@@ -862,6 +954,7 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     q.wgt = wgt;
     q.wgt_rail = g.rail ? wgt + g.wgt_rail_off : nullptr;
     q.wgt_rail_idx = g.rail ? wgt + g.wgt_rail_idx_off : nullptr;
+    q.rail_lines = g.wgt_rail_lines;
     q.y = y;
     q.c_in = g.c_in;
     q.wi = g.wi;

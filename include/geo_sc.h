@@ -179,6 +179,13 @@ GEO_SC_API int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* 
 GEO_SC_API int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,
                                                       const uint32_t* weight_streams, int32_t* y,
                                                       geo_sc_stream_t stream);
+/*
+ * For callers that write the two-rail weight lines themselves (layout above) into a buffer of
+ * geo_sc_weight_stream_words words: fills the rest of the buffer (the rail-packed copy) from those
+ * lines.  geo_sc_weight_streams does this itself.  Every (line, channel) must have at most one
+ * non-zero rail, as streams of the reference's codes have.
+ */
+GEO_SC_API int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams, geo_sc_stream_t stream);
 /* Word counts of the two stream buffers above. */
 GEO_SC_API int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
 GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);

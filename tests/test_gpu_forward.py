@@ -102,8 +102,8 @@ def test_conv_kernel_alone_on_oracle_streams(capi, so):
     tiled = np.zeros((P, H, K, ncot, 2, 16), dtype=np.uint32)
     tiled[..., 0, :] = np.pad(wpos.reshape(P, H, K, Cout), ((0, 0),) * 3 + ((0, pad_c),)).reshape(P, H, K, ncot, 16)
     tiled[..., 1, :] = np.pad(wneg.reshape(P, H, K, Cout), ((0, 0),) * 3 + ((0, pad_c),)).reshape(P, H, K, ncot, 16)
-    y = capi.conv2d_add_partial_from_streams(torch.from_numpy(act.view(np.int32)).cuda(),
-                                             torch.from_numpy(tiled.view(np.int32)).cuda(), d)
+    wgt = capi.weight_streams_from_lines(torch.from_numpy(tiled.view(np.int32)).cuda(), d)
+    y = capi.conv2d_add_partial_from_streams(torch.from_numpy(act.view(np.int32)).cuda(), wgt, d)
     exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, (1, 1))
     assert np.array_equal(y.cpu().numpy(), exp)
 
