@@ -115,9 +115,10 @@ class CONV_tiny_add_partial(nn.Module):
                       total_width=uf.prec_default, load_width=int(self.load_unit[i]), load_wait_w=int(wait_w),
                       load_wait_a=int(self.load_wait[i] if mode == "yz" else wait_w), accumulate=mode,
                       z_unit=max(1, min(2 ** self.z_unit[i], w.shape[1])))
-            d = capi.make_desc((2, w.shape[1], w.shape[2], w.shape[3]), w.shape, **kw)  # weights do not depend on n
             w_n, b_n = utils_class._fixed_affine(bn, None, bn.running_mean, bn.running_var)
-            state.append(dict(w_shape=tuple(w.shape), kw=kw, wgt=capi.weight_streams(w, d),
+            # the weight stream buffer is generated at the first forward: its stream words do not
+            # depend on the input, but what else the buffer carries depends on the layer's geometry
+            state.append(dict(w=w, w_shape=tuple(w.shape), kw=kw, wgt=None, wgt_for=None,
                               w_n=w_n.float().contiguous(), b_n=b_n.float().contiguous()))
         self._fused_state = state
         self._fused_graph = None
@@ -127,6 +128,8 @@ class CONV_tiny_add_partial(nn.Module):
         last = len(self._fused_state) - 1
         for i, st in enumerate(self._fused_state):
             d = capi.make_desc(x.shape, st["w_shape"], **st["kw"])
+            if st["wgt_for"] != tuple(x.shape):
+                st["wgt"], st["wgt_for"] = capi.weight_streams(st["w"], d), tuple(x.shape)
             counts = capi.conv2d_add_partial_from_streams(capi.act_streams(x, d), st["wgt"], d)
             L = st["kw"]["bit_length"]
             if i == last:
