@@ -100,9 +100,9 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     }
     g->act_item_inner = !g->thin && g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
-    // two output rows per lane, compile-time kernel extent in dim 2, position-major streams: the
-    // launches launch_conv_forward gives to the rail-skipping kernels
-    g->rail = !g->thin && !g->act_item_inner && wo >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5);
+    // two output rows (or, item-innermost, two batch items) per lane and a compile-time kernel extent
+    // in dim 2: the launches launch_conv_forward gives to the rail-skipping kernels
+    g->rail = !g->thin && (wo >= 2 || g->act_item_inner) && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5);
     const size_t lines = (size_t)g->packs * d->h_k * g->k_or;
     g->wgt_words = lines * g->n_cotile * 2 * kCoTile;
     g->wgt_rail_off = g->wgt_rail_idx_off = 0;

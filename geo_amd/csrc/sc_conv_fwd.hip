@@ -14,6 +14,8 @@
 // Consecutive workgroups take the c_out tiles of the same positions.
 #include "sc_common.h"
 
+#include <type_traits>
+
 namespace geo_sc {
 
 namespace {
@@ -844,6 +846,108 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
 }
 
+// The rail-skipping kernel for item-innermost activation streams (outputs with a single row: the
+// SC-linear mapping).  A lane's two accumulator rows are the batch items n and n + row_groups;
+// consecutive lanes are consecutive items.  Activation addresses are a wave-uniform pointer plus one
+// 32-bit byte offset per lane and item; the kernel taps advance the uniform pointer.  Partial sums
+// over blockIdx.y's (pack, add group) range are added to the zeroed y with integer atomics.
+// CU: input channels per loop trip (their loads are issued together: 3 for 1-wide kernels, so that a
+// trip still holds 96 vector instructions behind one wait).
+template <int WK, int CU>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_items_rail(FwdParams q)
+{
+    constexpr int C = kCoTile, R = 2;
+    const int cot = blockIdx.x % q.n_cotile;
+    const long long slot_first = (long long)(blockIdx.x / q.n_cotile) * 64;  // always a live slot
+    const long long slot0 = slot_first + threadIdx.x;
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : slot_first;
+    const int b = (int)(slot / q.row_groups);
+    const long long n = slot % q.row_groups;
+    // lane offsets (bytes) of the two items; an item past the end is clamped to the first one: it
+    // only feeds an output that is never stored
+    unsigned loff[R];
+#pragma unroll
+    for (int j = 0; j < R; j++)
+        loff[j] = 4u * ((unsigned)b * q.n + (unsigned)n +
+                        (n + (long long)j * q.row_groups < q.n ? (unsigned)j * q.row_groups : 0u));
+    const size_t pack_stride = (size_t)q.act_plane * q.n;
+    const unsigned tap_stride = (unsigned)q.hi * q.n;
+    const unsigned add_stride = (unsigned)q.n;
+    const unsigned or_stride = (unsigned)q.wi * q.hi * q.n;
+
+    int sum[2 * C];  // [2 c + r]
+#pragma unroll
+    for (int i = 0; i < 2 * C; i++) sum[i] = 0;
+
+    const int groups = q.add_outer * q.add_inner;
+    const int pv_begin = blockIdx.y * q.pv_per_block;
+    const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
+    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    for (int pv = pv_begin; pv < pv_end; pv++) {
+        const int p = pv / groups, g = pv - p * groups;
+        const int go = g / q.add_inner, gi = g - go * q.add_inner;
+        const int ch0 = go * q.or_ch_per_group;
+        const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
+        u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
+        const uint32_t* ap = q.act + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
+        const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
+                            (size_t)gi * chs * q.w_k;
+        const uint32_t* wp = q.wgt_rail + line * C;
+        const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
+        auto channels = [&](auto cu_tag) {
+            constexpr int N = decltype(cu_tag)::value;
+            uint32_t aw[N][WK][R];
+#pragma unroll
+            for (int cu = 0; cu < N; cu++)
+#pragma unroll
+                for (int u = 0; u < WK; u++)
+#pragma unroll
+                    for (int j = 0; j < R; j++)
+                        aw[cu][u][j] = *reinterpret_cast<const uint32_t*>(
+                            reinterpret_cast<const char*>(ap + (size_t)cu * or_stride + (size_t)u * tap_stride) + loff[j]);
+            uint32_t wv[N * WK][C], iv[N * WK][C / 2];
+#pragma unroll
+            for (int l = 0; l < N * WK; l++) {
+#pragma unroll
+                for (int c = 0; c < C; c++) wv[l][c] = wp[l * C + c];
+#pragma unroll
+                for (int c = 0; c < C / 2; c++) iv[l][c] = ip[l * (C / 2) + c];
+            }
+#pragma unroll
+            for (int cu = 0; cu < N; cu++)
+#pragma unroll
+                for (int u = 0; u < WK; u++)
+                    rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u][0], aw[cu][u][1]);
+            wp += N * WK * C;
+            ip += N * WK * (C / 2);
+            ap += (size_t)N * or_stride;
+        };
+        int ci = 0;
+        for (; ci + CU <= chs; ci += CU) channels(std::integral_constant<int, CU>());
+        if constexpr (CU > 1)
+            for (; ci < chs; ci++) channels(std::integral_constant<int, 1>());
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            sum[i] += __popc(p0[i]) - __popc(n0[i]);
+            sum[C + i] += __popc(p1[i]) - __popc(n1[i]);
+        }
+    }
+
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const int co = cot * C + c;
+        if (co >= q.c_out) break;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const long long item = n + (long long)r * q.row_groups;
+            if (item < q.n) atomicAdd(q.y + ((size_t)item * q.c_out + co) * out_plane + b, sum[2 * c + r]);
+        }
+    }
+}
+
 // Rail-packed weight lines from the two-rail lines [line][cot][2][16]: word = pos | neg (at most one
 // is non-zero), stored [cot][line][16]; per channel a 16-bit field with what the rail kernels move
 // into M0: bits 7:0 the register offset of the channel's accumulators, 2 c for the positive rail
@@ -902,7 +1006,8 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     }
     q.pv_per_block = (pv + splits - 1) / splits;
     splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
-    const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y;
+    // (item-innermost launches always go through the accumulating rail kernel)
+    const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y && !(ROWS_IN_N && g.rail);
     if (!plain && ROWS_IN_N) {
         // the item-innermost split kernel's lane offsets are 32-bit byte offsets inside one pack of all items
         if ((unsigned long long)g.act_plane * g.n * 4 >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
@@ -913,10 +1018,18 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
     }
     if (!plain) {
-        if constexpr (ROWS_IN_N)
-            hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>), dim3((unsigned)blocks, (unsigned)splits),
-                               dim3(64), 0, s, q);
-        else if (g.rail) {
+        if constexpr (ROWS_IN_N) {
+            if constexpr (R == 2 && WK > 0) {
+                if (g.rail)
+                    hipLaunchKernelGGL((k_conv_fwd_items_rail<WK, CU>), dim3((unsigned)blocks, (unsigned)splits),
+                                       dim3(64), 0, s, q);
+                else
+                    hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>),
+                                       dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s, q);
+            } else
+                hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>), dim3((unsigned)blocks, (unsigned)splits),
+                                   dim3(64), 0, s, q);
+        } else if (g.rail) {
             if constexpr (R == 2 && WK > 0)
                 hipLaunchKernelGGL((k_conv_fwd_split_rail<WK>), dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s,
                                    q);
