@@ -141,7 +141,7 @@ int forward_impl(const geo_sc_conv_desc* desc, const void* x, const float* w, in
     uint32_t* act = (uint32_t*)(ws + g.off_act);
     if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
     if ((rc = launch_weight_streams(g, w, wgt, tables, s)) != GEO_SC_OK) return rc;
-    if ((rc = launch_rail_pack(g, wgt, s)) != GEO_SC_OK) return rc;
+    if ((rc = launch_rail_pack(g, wgt, s, true)) != GEO_SC_OK) return rc;
     rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)x, act, tables, s)
             : launch_act_streams(g, (const float*)x, act, tables, s);
     if (rc != GEO_SC_OK) return rc;
@@ -245,7 +245,7 @@ int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t
     if (rc != GEO_SC_OK) return rc;
     rc = launch_weight_streams(g, w, streams, (const uint32_t*)tables, s);
     if (rc != GEO_SC_OK) return rc;
-    return launch_rail_pack(g, streams, s);
+    return launch_rail_pack(g, streams, s, true);
 }
 
 int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams, geo_sc_stream_t stream)
@@ -254,7 +254,7 @@ int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams
     const int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
     if (!streams) return GEO_SC_ERR_INVALID_ARGUMENT;
-    return launch_rail_pack(g, streams, (hipStream_t)stream);
+    return launch_rail_pack(g, streams, (hipStream_t)stream, false);
 }
 
 int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,

@@ -79,8 +79,14 @@ int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* stre
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
-// fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.rail)
-int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s);
+// fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.rail;
+// with from_generator also where launch_weight_streams has written that part itself)
+int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator);
+// kernels long in dim 3 take the row-chunked LFSR weight generator, which also writes the rail-packed copy
+inline bool weight_rows_generator(const Geometry& g)
+{
+    return g.generator == GEO_SC_GEN_LFSR && (g.mode == GEO_SC_ACC_Y || g.mode == GEO_SC_ACC_FULL) && g.h_k >= 16;
+}
 size_t backward_workspace_bytes(const Geometry& g);
 int launch_conv_backward(const Geometry& g, const float* x, const float* w, const float* gy, float* gx, float* gw,
                          void* workspace, hipStream_t s);

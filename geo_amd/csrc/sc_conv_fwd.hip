@@ -1050,9 +1050,9 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
 
 }  // namespace
 
-int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s)
+int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator)
 {
-    if (!g.rail) return GEO_SC_OK;
+    if (!g.rail || (from_generator && weight_rows_generator(g))) return GEO_SC_OK;
     const size_t lines = g.wgt_rail_lines;
     size_t blocks = (lines * g.n_cotile + 255) / 256;
     hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,

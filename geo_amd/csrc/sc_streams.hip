@@ -210,7 +210,9 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float
                                                                     uint32_t* __restrict__ streams,
                                                                     const uint32_t* __restrict__ tables, GenParams gp,
                                                                     int c_out, int c_in, int w_k, int h_k, int n_cotile,
-                                                                    int v_chunks)
+                                                                    int v_chunks, uint32_t* __restrict__ rail_words,
+                                                                    uint16_t* __restrict__ rail_fields,
+                                                                    size_t rail_lines)
 {
     extern __shared__ uint32_t lds[];
     load_tables_to_lds(lds, tables, gp.L, gp.wpc);
@@ -239,8 +241,18 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float
         const int on = (int)posp1[(37 + k) % (gp.L - 1)];
         const size_t base = (((size_t)v * k_or + k) * n_cotile + cot) * (2 * kCoTile) + co_l;
         for (int pk = 0; pk < gp.packs; pk++) {
-            streams[pk * pack_stride + base] = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
-            streams[pk * pack_stride + base + kCoTile] = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+            const uint32_t wp = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
+            const uint32_t wn = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+            streams[pk * pack_stride + base] = wp;
+            streams[pk * pack_stride + base + kCoTile] = wn;
+            if (rail_words) {
+                // the rail-packed copy in the same pass (these tensors are large: a separate pass
+                // would read all lines back): [c_out tile][line][channel], the non-zero rail's word
+                // and the 16-bit M0 field of the channel's rail
+                const size_t dst = ((size_t)cot * rail_lines + ((size_t)pk * h_k + v) * k_or + k) * kCoTile + co_l;
+                rail_words[dst] = wp | wn;
+                rail_fields[dst] = (uint16_t)(0xC000u | ((cn ? 2u * kCoTile : 0u) + 2u * co_l));
+            }
         }
     }
 }
@@ -538,12 +550,14 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
                            g.mode == GEO_SC_ACC_Z ? 1 : 0, g.add_outer, g.add_inner, g.or_ch_total, g.or_ch_per_group);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
-    if (g.h_k >= 16) {
+    if (weight_rows_generator(g)) {
         const int v_chunks = (g.h_k + 15) / 16;
         const size_t n_blocks = (size_t)v_chunks * g.k_or * g.n_cotile;
         hipLaunchKernelGGL(k_weight_streams_rows, dim3((unsigned)(n_blocks > 256 * 8 ? 256 * 8 : n_blocks)),
                            dim3(kGenThreads), table_bytes(g.L), s, w, streams, tables, gp, g.c_out, g.c_in, g.w_k,
-                           g.h_k, g.n_cotile, v_chunks);
+                           g.h_k, g.n_cotile, v_chunks, g.rail ? streams + g.wgt_rail_off : nullptr,
+                           g.rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
+                           g.wgt_rail_lines);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
