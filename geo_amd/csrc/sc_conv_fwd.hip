@@ -350,212 +350,6 @@ __global__ __launch_bounds__(64) void k_conv_fwd_split(FwdParams q)
     }
 }
 
-// OR-accumulate CU channels for the item-innermost split kernel: activation words are addressed as a
-// wave-uniform pointer plus a 32-bit lane offset in bytes (scalar address arithmetic, one VGPR
-// per offset).  With ROWS_IN_N the lane offsets select the R batch items and the kernel taps advance
-// the uniform pointer by tap_stride; otherwise the lane offsets select the R+WK-1 rows.  FIRST:
-// the very first line of an OR group assigns instead of OR-ing, so accumulators need no zeroing.
-template <int R, int WK, int CU, int NL, bool ROWS_IN_N, bool FIRST>
-__device__ __forceinline__ void or_channels_u(uint32_t (&orp)[R][kCoTile], uint32_t (&orn)[R][kCoTile],
-                                              const uint32_t*& ap_u, const uint32_t*& wp, const unsigned (&loff)[NL],
-                                              unsigned ch_stride, unsigned tap_stride, unsigned k_stride)
-{
-    constexpr int C = kCoTile;
-    constexpr int NW = ROWS_IN_N ? R * WK : R + WK - 1;
-    uint32_t aw[CU][NW];
-#pragma unroll
-    for (int cu = 0; cu < CU; cu++)
-#pragma unroll
-        for (int j = 0; j < NW; j++) {
-            // uniform pointer + zero-extended 32-bit byte offset: the SGPR-base form of global_load
-            const char* base = reinterpret_cast<const char*>(ap_u + (size_t)cu * ch_stride +
-                                                             (ROWS_IN_N ? (size_t)(j % WK) * tap_stride : 0));
-            aw[cu][j] = *reinterpret_cast<const uint32_t*>(base + loff[ROWS_IN_N ? j / WK : j]);
-        }
-#pragma unroll
-    for (int cu = 0; cu < CU; cu++)
-#pragma unroll
-        for (int u = 0; u < WK; u++) {
-            uint32_t wv[2 * C];
-#pragma unroll
-            for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                const uint32_t a = aw[cu][ROWS_IN_N ? r * WK + u : r + u];
-#pragma unroll
-                for (int c = 0; c < C; c++) {
-                    if (FIRST && cu == 0 && u == 0) {
-                        orp[r][c] = a & wv[c];
-                        orn[r][c] = a & wv[C + c];
-                    } else {
-                        and_or(orp[r][c], a, wv[c]);
-                        and_or(orn[r][c], a, wv[C + c]);
-                    }
-                }
-            }
-            wp += k_stride;
-        }
-    ap_u += (size_t)CU * ch_stride;
-}
-
-// The split kernel for item-innermost activation streams (outputs with a single row: the SC-linear
-// mapping).  Its OR groups are short (16 members for a 4096-wide linear layer as 16 x 1 x 256), so
-// per-group overhead counts: the first weight line assigns the accumulators instead of OR-ing into
-// zeroed ones, and activation addresses are a wave-uniform base plus one 32-bit byte offset per
-// lane (4096 x 4096 linear at batch 1024: 6.3 -> 5.65 ms).  For position-major streams this
-// form is 5-6 % slower than k_conv_fwd_split, which therefore keeps them.
-// Each workgroup sums a contiguous range of (pack, add group) pairs and adds its partial result to y
-// with integer atomics (y is zeroed first).  Used for small layers that would otherwise leave most of the
-// GPU idle, and for the accumulation modes other than "OR over (c_in, w_k), add over h_k":
-// the add groups are (outer, inner) pairs, an outer group owning a range of OR channels
-//   Y : outer 1,              inner kernel rows,     OR channels = input channels
-//   YZ: outer channel groups, inner kernel rows,     OR channels = the group's input channels
-//   Z : outer 1,              inner input channels,  OR channels = kernel rows
-//   FULL: one group per pack; the OR runs over the input channels of or_rows = h_k kernel rows
-// (sc_cuda_kernel.cu:176-349, :1351-1366), expressed through the two activation strides in
-// FwdParams; the weight lines arrive in exactly the order the loop consumes them.
-// Template parameters as for k_conv_fwd.
-template <int R, int WK, int CU, bool ROWS_IN_N>
-__global__ __launch_bounds__(64) void k_conv_fwd_split_items(FwdParams q)
-{
-    constexpr int C = kCoTile;
-    static_assert(WK > 0 || (R == 1 && !ROWS_IN_N), "run-time kernel extent handles one row per lane");
-    const int cot = blockIdx.x % q.n_cotile;
-    const long long slot_first = (long long)(blockIdx.x / q.n_cotile) * 64;  // always a live slot
-    const long long slot0 = slot_first + threadIdx.x;
-    const bool live = slot0 < q.slots;
-    const long long slot = live ? slot0 : slot_first;
-    // lane slot -> (first item n, first output row a0, output column b).  With ROWS_IN_N the
-    // R rows of a lane are items n and n + row_groups, consecutive lanes are consecutive
-    // items, and the activation streams are stored item-innermost.
-    const int b = ROWS_IN_N ? (int)(slot / q.row_groups) : (int)(slot % q.ho);
-    const long long t = slot / q.ho;
-    const int a0 = ROWS_IN_N ? 0 : (int)(t % q.row_groups) * R;
-    const long long n = ROWS_IN_N ? slot % q.row_groups : t / q.row_groups;
-    const size_t item_stride = (size_t)q.packs * q.act_plane;
-    // first item of the tile: the uniform part of the activation address (lanes add the rest)
-    const long long n_first = ROWS_IN_N ? 0 : (slot_first / q.ho) / q.row_groups;
-
-    constexpr int NL = WK == 0 ? 1 : (ROWS_IN_N ? R : R + WK - 1);
-    // lane offsets (bytes).  Rows / items past the end (partial last group) are clamped to valid
-    // ones: they only feed outputs that are never stored.
-    unsigned loff[NL];
-    if constexpr (WK > 0) {
-#pragma unroll
-        for (int j = 0; j < NL; j++) {
-            if (ROWS_IN_N) {
-                loff[j] = 4u * ((unsigned)b * q.n + (unsigned)n +
-                                (n + (long long)j * q.row_groups < q.n ? (unsigned)j * q.row_groups : 0u));
-            } else {
-                const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
-                loff[j] = 4u * ((unsigned)((n - n_first) * item_stride) + (unsigned)row * q.hi + (unsigned)b);
-            }
-        }
-    } else {
-        loff[0] = 4u * ((unsigned)((n - n_first) * item_stride) + (unsigned)b);
-    }
-    // strides (words) of one pack, one kernel tap along dim 2 (item-innermost layout), one channel
-    const size_t pack_stride = ROWS_IN_N ? (size_t)q.act_plane * q.n : (size_t)q.act_plane;
-    const unsigned tap_stride = (unsigned)q.hi * q.n;
-    const unsigned add_stride = ROWS_IN_N ? (unsigned)q.n : q.add_stride;
-    const unsigned or_stride = ROWS_IN_N ? (unsigned)q.wi * q.hi * q.n : q.or_stride;
-    const uint32_t* act_u = q.act + (size_t)n_first * item_stride;
-    const unsigned k_stride = (unsigned)q.n_cotile * 2 * C;
-
-    int sum[R][C];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int c = 0; c < C; c++) sum[r][c] = 0;
-
-    // (pack, add group) pairs are independent partial sums: blockIdx.y takes a contiguous
-    // range of them when the launch is split to fill the GPU
-    const int groups = q.add_outer * q.add_inner;
-    const int pv_begin = blockIdx.y * q.pv_per_block;
-    const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
-    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
-    for (int pv = pv_begin; pv < pv_end; pv++) {
-        const int p = pv / groups, g = pv - p * groups;
-        const int go = g / q.add_inner, gi = g - go * q.add_inner;
-        const int ch0 = go * q.or_ch_per_group;
-        const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
-        uint32_t orp[R][C], orn[R][C];
-
-        const uint32_t* ap0 = act_u + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
-        const size_t line = p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k + (size_t)gi * chs * q.w_k;
-        const uint32_t* wp = q.wgt + (line * q.n_cotile + cot) * (2 * C);
-
-        if constexpr (WK > 0) {
-            for (int row = 0; row < q.or_rows; row++) {
-                const uint32_t* ap = ap0 + row;  // next kernel row: one word further (never with ROWS_IN_N)
-                int ci;
-                if (row == 0) {
-                    // the first line of the group assigns the accumulators
-                    if (CU > 1 && chs < CU) {
-                        or_channels_u<R, WK, 1, NL, ROWS_IN_N, true>(orp, orn, ap, wp, loff, or_stride, tap_stride, k_stride);
-                        ci = 1;
-                    } else {
-                        or_channels_u<R, WK, CU, NL, ROWS_IN_N, true>(orp, orn, ap, wp, loff, or_stride, tap_stride, k_stride);
-                        ci = CU;
-                    }
-                } else {
-                    ci = 0;
-                }
-                for (; ci + CU <= chs; ci += CU)
-                    or_channels_u<R, WK, CU, NL, ROWS_IN_N, false>(orp, orn, ap, wp, loff, or_stride, tap_stride, k_stride);
-                if constexpr (CU > 1)
-                    for (; ci < chs; ci++)
-                        or_channels_u<R, WK, 1, NL, ROWS_IN_N, false>(orp, orn, ap, wp, loff, or_stride, tap_stride, k_stride);
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < C; c++) orp[0][c] = orn[0][c] = 0u;
-            for (int row = 0; row < q.or_rows; row++) {
-                const uint32_t* ap = ap0 + row;
-                for (int ci = 0; ci < chs; ci++) {
-                    for (int u = 0; u < q.w_k; u++) {
-                        uint32_t wv[2 * C];
-#pragma unroll
-                        for (int c = 0; c < 2 * C; c++) wv[c] = wp[c];
-                        int arow = a0 + u;
-                        arow = arow < q.wi ? arow : q.wi - 1;
-                        const uint32_t aw = *reinterpret_cast<const uint32_t*>(
-                            reinterpret_cast<const char*>(ap + (size_t)arow * q.hi) + loff[0]);
-#pragma unroll
-                        for (int c = 0; c < C; c++) {
-                            and_or(orp[0][c], aw, wv[c]);
-                            and_or(orn[0][c], aw, wv[C + c]);
-                        }
-                        wp += k_stride;
-                    }
-                    ap += or_stride;
-                }
-            }
-        }
-        // binary add across add groups and packs: v_bcnt_u32_b32 folds the add
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int c = 0; c < C; c++) sum[r][c] += __popc(orp[r][c]) - __popc(orn[r][c]);
-    }
-
-    if (!live) return;
-    const size_t out_plane = (size_t)q.wo * q.ho;
-#pragma unroll
-    for (int c = 0; c < C; c++) {
-        const int co = cot * C + c;
-        if (co >= q.c_out) break;
-        int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const bool row_ok = ROWS_IN_N ? n + (long long)r * q.row_groups < q.n : a0 + r < q.wo;
-            int32_t* dst = yo + (ROWS_IN_N ? (size_t)r * q.row_groups * q.c_out * out_plane : (size_t)r * q.ho);
-            if (!row_ok) continue;
-            atomicAdd(dst, sum[r][c]);  // integer adds: order does not matter
-        }
-    }
-}
-
 // Layers with few output positions and large OR groups (classifier layers: 64 x 4 x 4 -> 10 at
 // batch 256 has 2560 outputs of 1024 products each): one wave per (output position, c_out tile,
 // pack, add group); the lanes run over the members of the OR group, each with its own weight
@@ -1007,44 +801,33 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     q.pv_per_block = (pv + splits - 1) / splits;
     splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
     // (item-innermost launches always go through the accumulating rail kernel)
-    const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y && !(ROWS_IN_N && g.rail);
-    if (!plain && ROWS_IN_N) {
-        // the item-innermost split kernel's lane offsets are 32-bit byte offsets inside one pack of all items
+    const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y && !ROWS_IN_N;
+    if (ROWS_IN_N) {
+        // its lane offsets are 32-bit byte offsets inside one pack of all items
         if ((unsigned long long)g.act_plane * g.n * 4 >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
+        if (!g.rail) return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail with act_item_inner
     }
     if (!plain) {
         const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
         size_t zb = (n_out + 255) / 256;
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
     }
-    if (!plain) {
-        if constexpr (ROWS_IN_N) {
-            if constexpr (R == 2 && WK > 0) {
-                if (g.rail)
-                    hipLaunchKernelGGL((k_conv_fwd_items_rail<WK, CU>), dim3((unsigned)blocks, (unsigned)splits),
-                                       dim3(64), 0, s, q);
-                else
-                    hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>),
-                                       dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s, q);
-            } else
-                hipLaunchKernelGGL((k_conv_fwd_split_items<R, WK, CU, true>), dim3((unsigned)blocks, (unsigned)splits),
-                                   dim3(64), 0, s, q);
-        } else if (g.rail) {
-            if constexpr (R == 2 && WK > 0)
-                hipLaunchKernelGGL((k_conv_fwd_split_rail<WK>), dim3((unsigned)blocks, (unsigned)splits), dim3(64), 0, s,
-                                   q);
-            else
-                return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail for these launches only
-        } else
-            hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, false>), dim3((unsigned)blocks, (unsigned)splits), dim3(64),
-                               0, s, q);
+    const dim3 grid((unsigned)blocks, (unsigned)(plain ? 1 : splits));
+    if constexpr (ROWS_IN_N) {
+        static_assert(R == 2 && WK > 0, "item-innermost launches take two items per lane");
+        hipLaunchKernelGGL((k_conv_fwd_items_rail<WK, CU>), grid, dim3(64), 0, s, q);
     } else if (g.rail) {
-        if constexpr (R == 2 && !ROWS_IN_N && WK > 0)
-            hipLaunchKernelGGL((k_conv_fwd_rail<WK>), dim3((unsigned)blocks), dim3(64), 0, s, q);
-        else
-            return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail for these launches only
-    } else
-        hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, ROWS_IN_N>), dim3((unsigned)blocks), dim3(64), 0, s, q);
+        if constexpr (R == 2 && WK > 0) {
+            if (plain)
+                hipLaunchKernelGGL((k_conv_fwd_rail<WK>), grid, dim3(64), 0, s, q);
+            else
+                hipLaunchKernelGGL((k_conv_fwd_split_rail<WK>), grid, dim3(64), 0, s, q);
+        } else
+            return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail for two-row launches only
+    } else if (plain)
+        hipLaunchKernelGGL((k_conv_fwd<R, WK, CU, false>), grid, dim3(64), 0, s, q);
+    else
+        hipLaunchKernelGGL((k_conv_fwd_split<R, WK, CU, false>), grid, dim3(64), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
