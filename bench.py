@@ -414,6 +414,9 @@ def main():
             # Instructions the kernel really issues.  A weight has at most one non-zero rail; the
             # rail-skipping kernel processes only that one, i.e. half of the algorithmic (two-rail)
             # count, which is how "achieved" can pass the peak.
+            "note": ("frac counts the algorithmic two-rail work (2*B/32 and-or word-ops) against the nominal VALU "
+                     "peak; the rail-skipping kernel issues one and-or per (activation word, weight) instead of "
+                     "two, so frac can pass 1: executed_* is what the hardware actually does") if rail else None,
             "executed_word_ops": executed_ops,
             "executed_rate": executed_ops / (k_avg * 1e-3) / 1e12,
             "executed_frac": executed_ops / (k_avg * 1e-3) / PEAK_VALU_WORD_OPS,
