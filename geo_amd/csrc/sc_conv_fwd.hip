@@ -478,7 +478,9 @@ static_assert(kCoTile == 16, "rail_line is written for tiles of 16 output channe
 
 // Two output rows per lane (R = 2), position-major activation streams, kernel extent WK in dim 2.
 // Same lane -> position mapping, grid and result as k_conv_fwd<2, WK, 1, false>.
-template <int WK>
+// CU: input channels per loop trip (their loads are issued together: 2 for 1-wide kernels, so that a
+// trip holds 64 vector instructions behind one wait instead of 32).
+template <int WK, int CU>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_rail(FwdParams q)
 {
     constexpr int C = kCoTile, R = 2, NW = R + WK - 1;
@@ -516,24 +518,34 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
             const size_t line0 = (size_t)cot * q.rail_lines + (size_t)(p * q.h_k + v) * k_or;
             const uint32_t* wp = q.wgt_rail + line0 * C;
             const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
-            for (int ci = 0; ci < q.c_in; ci++) {
-                uint32_t aw[NW];
+            auto channels = [&](auto cu_tag) {
+                constexpr int N = decltype(cu_tag)::value;
+                uint32_t aw[N][NW];
 #pragma unroll
-                for (int j = 0; j < NW; j++) aw[j] = ap[off[j]];
-                uint32_t wv[WK][C], iv[WK][C / 2];
+                for (int cu = 0; cu < N; cu++)
 #pragma unroll
-                for (int u = 0; u < WK; u++) {
+                    for (int j = 0; j < NW; j++) aw[cu][j] = ap[cu * ch_stride + off[j]];
+                uint32_t wv[N * WK][C], iv[N * WK][C / 2];
 #pragma unroll
-                    for (int c = 0; c < C; c++) wv[u][c] = wp[u * C + c];
+                for (int l = 0; l < N * WK; l++) {
 #pragma unroll
-                    for (int c = 0; c < C / 2; c++) iv[u][c] = ip[u * (C / 2) + c];
+                    for (int c = 0; c < C; c++) wv[l][c] = wp[l * C + c];
+#pragma unroll
+                    for (int c = 0; c < C / 2; c++) iv[l][c] = ip[l * (C / 2) + c];
                 }
 #pragma unroll
-                for (int u = 0; u < WK; u++) rail_line(p0, p1, n0, n1, wv[u], iv[u], aw[u], aw[u + 1]);
-                wp += WK * C;
-                ip += WK * (C / 2);
-                ap += ch_stride;
-            }
+                for (int cu = 0; cu < N; cu++)
+#pragma unroll
+                    for (int u = 0; u < WK; u++)
+                        rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u], aw[cu][u + 1]);
+                wp += N * WK * C;
+                ip += N * WK * (C / 2);
+                ap += N * ch_stride;
+            };
+            int ci = 0;
+            for (; ci + CU <= q.c_in; ci += CU) channels(std::integral_constant<int, CU>());
+            if constexpr (CU > 1)
+                for (; ci < q.c_in; ci++) channels(std::integral_constant<int, 1>());
             // binary add across kernel rows and packs: v_bcnt_u32_b32 folds the add
 #pragma unroll
             for (int i = 0; i < C; i++) {
@@ -559,7 +571,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 // The rail-skipping form of k_conv_fwd_split<2, WK, 1, false>: launches split over blockIdx.y and
 // the accumulation modes other than y, position-major activation streams, two output rows per lane.
 // Partial sums are added to the zeroed y with integer atomics.
-template <int WK>
+template <int WK, int CU>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_split_rail(FwdParams q)
 {
     constexpr int C = kCoTile, R = 2, NW = R + WK - 1;
@@ -601,24 +613,34 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
         for (int row = 0; row < q.or_rows; row++) {
             const uint32_t* ap = ap0 + row;  // next kernel row: one word further
-            for (int ci = 0; ci < chs; ci++) {
-                uint32_t aw[NW];
+            auto channels = [&](auto cu_tag) {
+                constexpr int N = decltype(cu_tag)::value;
+                uint32_t aw[N][NW];
 #pragma unroll
-                for (int j = 0; j < NW; j++) aw[j] = ap[off[j]];
-                uint32_t wv[WK][C], iv[WK][C / 2];
+                for (int cu = 0; cu < N; cu++)
 #pragma unroll
-                for (int u = 0; u < WK; u++) {
+                    for (int j = 0; j < NW; j++) aw[cu][j] = ap[cu * q.or_stride + off[j]];
+                uint32_t wv[N * WK][C], iv[N * WK][C / 2];
 #pragma unroll
-                    for (int c = 0; c < C; c++) wv[u][c] = wp[u * C + c];
+                for (int l = 0; l < N * WK; l++) {
 #pragma unroll
-                    for (int c = 0; c < C / 2; c++) iv[u][c] = ip[u * (C / 2) + c];
+                    for (int c = 0; c < C; c++) wv[l][c] = wp[l * C + c];
+#pragma unroll
+                    for (int c = 0; c < C / 2; c++) iv[l][c] = ip[l * (C / 2) + c];
                 }
 #pragma unroll
-                for (int u = 0; u < WK; u++) rail_line(p0, p1, n0, n1, wv[u], iv[u], aw[u], aw[u + 1]);
-                wp += WK * C;
-                ip += WK * (C / 2);
-                ap += q.or_stride;
-            }
+                for (int cu = 0; cu < N; cu++)
+#pragma unroll
+                    for (int u = 0; u < WK; u++)
+                        rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u], aw[cu][u + 1]);
+                wp += N * WK * C;
+                ip += N * WK * (C / 2);
+                ap += N * q.or_stride;
+            };
+            int ci = 0;
+            for (; ci + CU <= chs; ci += CU) channels(std::integral_constant<int, CU>());
+            if constexpr (CU > 1)
+                for (; ci < chs; ci++) channels(std::integral_constant<int, 1>());
         }
 #pragma unroll
         for (int i = 0; i < C; i++) {
@@ -818,10 +840,13 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         hipLaunchKernelGGL((k_conv_fwd_items_rail<WK, CU>), grid, dim3(64), 0, s, q);
     } else if (g.rail) {
         if constexpr (R == 2 && WK > 0) {
+            // two channels per trip for 1-wide kernels: with three, the six address pairs push the 32
+            // sums out of the 128 registers
+            constexpr int CR = WK == 1 ? 2 : 1;
             if (plain)
-                hipLaunchKernelGGL((k_conv_fwd_rail<WK>), grid, dim3(64), 0, s, q);
+                hipLaunchKernelGGL((k_conv_fwd_rail<WK, CR>), grid, dim3(64), 0, s, q);
             else
-                hipLaunchKernelGGL((k_conv_fwd_split_rail<WK>), grid, dim3(64), 0, s, q);
+                hipLaunchKernelGGL((k_conv_fwd_split_rail<WK, CR>), grid, dim3(64), 0, s, q);
         } else
             return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail for two-row launches only
     } else if (plain)
