@@ -100,14 +100,16 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     }
     g->act_item_inner = !g->thin && g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
                         (unsigned long long)g->act_words < 0xffffffffull;
-    // two output rows (or, item-innermost, two batch items) per lane and a compile-time kernel extent
-    // in dim 2: the launches launch_conv_forward gives to the rail-skipping kernels
-    g->rail = !g->thin && (wo >= 2 || g->act_item_inner) && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5);
+    // Weight stream buffers of 1-, 3- and 5-wide kernels carry the rail-packed copy, whatever the
+    // batch and input size (a buffer serves every geometry of the same weights); the launches with two
+    // output rows (or, item-innermost, two batch items) per lane read it: the rail-skipping kernels.
+    g->wgt_rail = d->w_k == 1 || d->w_k == 3 || d->w_k == 5;
+    g->rail = g->wgt_rail && !g->thin && (wo >= 2 || g->act_item_inner);
     const size_t lines = (size_t)g->packs * d->h_k * g->k_or;
     g->wgt_words = lines * g->n_cotile * 2 * kCoTile;
     g->wgt_rail_off = g->wgt_rail_idx_off = 0;
     g->wgt_rail_lines = lines;
-    if (g->rail) {
+    if (g->wgt_rail) {
         g->wgt_rail_off = (g->wgt_words + 63) & ~(size_t)63;
         g->wgt_rail_idx_off = g->wgt_rail_off + lines * g->n_cotile * kCoTile;
         g->wgt_words = g->wgt_rail_idx_off + lines * g->n_cotile * (kCoTile / 2);

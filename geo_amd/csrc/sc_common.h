@@ -52,8 +52,9 @@ struct Geometry {
     size_t wgt_words, wgt_rail_off, wgt_rail_idx_off, wgt_rail_lines;
     // Position-major launches with two output rows per lane run the rail-skipping kernels: per weight
     // at most one rail's stream is non-zero (codes of clamp(w, 0, .) and -clamp(w, ., 0)), and only
-    // that rail is processed.
-    bool rail;
+    // that rail is processed.  wgt_rail: the weight stream buffer carries the rail-packed copy (a
+    // property of the weights' shape alone); rail: this geometry's launch reads it.
+    bool wgt_rail, rail;
     // workspace carve-up (byte offsets, 256-aligned)
     size_t off_tables, off_wgt, off_act, ws_bytes;
 };
@@ -79,7 +80,7 @@ int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* stre
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
-// fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.rail;
+// fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.wgt_rail;
 // with from_generator also where launch_weight_streams has written that part itself)
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator);
 // kernels long in dim 3 take the row-chunked LFSR weight generator, which also writes the rail-packed copy

@@ -860,7 +860,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
 
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator)
 {
-    if (!g.rail || (from_generator && weight_rows_generator(g))) return GEO_SC_OK;
+    if (!g.wgt_rail || (from_generator && weight_rows_generator(g))) return GEO_SC_OK;
     const size_t lines = g.wgt_rail_lines;
     size_t blocks = (lines * g.n_cotile + 255) / 256;
     hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,
@@ -873,8 +873,8 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     FwdParams q;
     q.act = act;
     q.wgt = wgt;
-    q.wgt_rail = g.rail ? wgt + g.wgt_rail_off : nullptr;
-    q.wgt_rail_idx = g.rail ? wgt + g.wgt_rail_idx_off : nullptr;
+    q.wgt_rail = g.wgt_rail ? wgt + g.wgt_rail_off : nullptr;
+    q.wgt_rail_idx = g.wgt_rail ? wgt + g.wgt_rail_idx_off : nullptr;
     q.rail_lines = g.wgt_rail_lines;
     q.y = y;
     q.c_in = g.c_in;

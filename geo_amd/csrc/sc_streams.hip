@@ -555,8 +555,8 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
         const size_t n_blocks = (size_t)v_chunks * g.k_or * g.n_cotile;
         hipLaunchKernelGGL(k_weight_streams_rows, dim3((unsigned)(n_blocks > 256 * 8 ? 256 * 8 : n_blocks)),
                            dim3(kGenThreads), table_bytes(g.L), s, w, streams, tables, gp, g.c_out, g.c_in, g.w_k,
-                           g.h_k, g.n_cotile, v_chunks, g.rail ? streams + g.wgt_rail_off : nullptr,
-                           g.rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
+                           g.h_k, g.n_cotile, v_chunks, g.wgt_rail ? streams + g.wgt_rail_off : nullptr,
+                           g.wgt_rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
                            g.wgt_rail_lines);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }

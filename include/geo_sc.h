@@ -158,7 +158,7 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, c
  * order the lines by (pack, add group, OR member): Z [P][c_in][h_k*w_k] with member
  * h_index*w_k + w_index; YZ [P][channel group][h_k][channels of the group * w_k].
  * A weight has at most one non-zero rail (its codes are those of clamp(w, 0, .) and
- * -clamp(w, ., 0), sc.cpp:301-304).  For large y-mode layers the buffer continues behind these
+ * -clamp(w, ., 0), sc.cpp:301-304).  For 1-, 3- and 5-wide kernels the buffer continues behind these
  * lines with a second, rail-packed copy that the convolution kernel reads there (per line 16
  * words pos | neg, then per line 8 words holding 16 bits per channel: which rail);
  * geo_sc_weight_stream_words is the size of the whole buffer, geo_sc_weight_streams fills all of it.
