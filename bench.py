@@ -431,7 +431,10 @@ def main():
         "backward_flops": {"algorithmic": 12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H,
                            "achieved_tflops": (12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H
                                                / (bwd_avg * 1e-3) / 1e12) if bwd_avg else None,
-                           "peak_tflops_fp32_mfma": 157.3},
+                           "peak_tflops_fp32_mfma": 157.3,
+                           "note": "fp32 in and out; aligned operands form each fp32 product from six bf16 MFMA "
+                                   "products of a three-way split (fp32 accumulation, error as an fp32 GEMM), so "
+                                   "the fp32 MFMA peak is a yardstick, not a bound"},
     }
     if not args.no_cpu_baseline and not variant:  # the compiled reference has the y / LFSR op only
         kind, cores, sec, note = cpu_baseline(x, w, L, pad)

@@ -29,6 +29,8 @@
 // Members of a ragged last channel block that do not exist carry zero weights.
 #include "sc_common.h"
 
+#include <type_traits>
+
 namespace geo_sc {
 
 namespace {
@@ -53,7 +55,7 @@ struct GemmParams {
     float* __restrict__ c;
     int I, J, K;              // C[I][J] = sum_k A(k,i) * B(k,j)
     long long lda, ldb, ldc;  // leading dimensions (elements)
-    // blockIdx.z = batch * splits + split.  A batch member is one kernel row: its operands
+    // z = batch * splits + split.  A batch member is one kernel row: its operands
     // and result start batch_stride elements further; a split takes k_per_split of K and
     // writes its own partial result c_split_stride further.
     int splits;
@@ -66,32 +68,65 @@ struct GemmParams {
     // tile extent per workgroup in i and j: kTile, or kTile / 2 in at most one of them (set by
     // launch_gemm): the four waves then line up along the other dimension
     int tile_i, tile_j;
+    // Workgroup numbering (set by launch_gemm).  The grid is one-dimensional and the hardware deals
+    // consecutive workgroup ids to the 8 XCDs in turn, each with an L2 of its own.  Workgroups that read
+    // the same operand tiles form a cluster of `cluster` members (the tiles along the short dimension of
+    // the result, or all tiles of one split of a small result); cluster q runs on XCD q % 8 with its members
+    // next to each other, so a tile comes from memory once instead of once per member.
+    int ni, nj, nz;  // tiles in i and j, batch * splits
+    int cluster;     // members per cluster
+    int cluster_of;  // 0: members = j tiles of one i tile, 1: i tiles of one j tile, 2: all tiles of one z
 };
 
-// Staging of one kChunk x kTile operand tile, split in two so that the global loads of chunk
-// c+1 are in flight while the MFMAs of chunk c run: fetch() reads 8 elements per thread into
-// registers, commit() writes them to LDS as s[k][i].
+// The tile (it, jt, z) of workgroup w under the numbering above.
+__device__ __forceinline__ void gemm_tile_of(const GemmParams& q, int w, int& it, int& jt, int& z)
+{
+    const int c = q.cluster;
+    const int n_clusters = q.cluster_of == 2 ? q.nz : q.cluster_of == 0 ? q.nz * q.ni : q.nz * q.nj;
+    const int whole = (n_clusters / 8) * 8 * c;  // workgroups of the clusters that fill all 8 XCDs evenly
+    int cl, member;
+    if (w < whole) {
+        const int xcd = w & 7, r = w >> 3;
+        member = r % c;
+        cl = (r / c) * 8 + xcd;
+    } else {
+        const int r = w - whole;
+        member = r % c;
+        cl = (n_clusters / 8) * 8 + r / c;
+    }
+    if (q.cluster_of == 2) {
+        z = cl;
+        it = member % q.ni;
+        jt = member / q.ni;
+    } else if (q.cluster_of == 0) {
+        z = cl / q.ni;
+        it = cl - z * q.ni;
+        jt = member;
+    } else {
+        z = cl / q.nj;
+        jt = cl - z * q.nj;
+        it = member;
+    }
+}
+
+// Staging of one kChunk x kTile operand tile for the fp32 kernel, split in two so that the global
+// loads of chunk c+1 are in flight while the MFMAs of chunk c run: fetch() reads 8 elements per
+// thread into registers, commit() writes them to LDS as s[k][i].
 //   K-major operand: element (k, i) at p[k*ld + i]
 //   I-major operand: element (k, i) at p[i*ld + k]
-// VEC: the operand's leading dimension and extent along its contiguous axis are multiples of
-// 4 floats, so chunks move as two float4 per thread (K-major: always, with whole rows of a
-// partial last chunk dropped; I-major: full chunks only); otherwise guarded scalar loads (out-of-range lanes read a valid dummy address and
-// are zeroed by a select, no divergent branches).
-template <bool KMAJOR, bool VEC>
+// Guarded scalar loads for operands of any alignment and extent (lanes outside the operand read a valid
+// dummy address and are zeroed by a select, no divergent branches); aligned operands take k_gemm_split.
+template <bool KMAJOR>
 struct Stager {
     const float* p;      // this thread's first element of the current chunk
     const float* dummy;  // any valid address of the operand
     long long ld;
     int kk0, ii;         // first k (inside the chunk) and first i (inside the tile) of this thread
     bool i_ok;
-    // which elements of the last fetch lie inside the operand: per float4 after a vector fetch
-    // (vec_), else bit c of ok for element c
-    bool vec_, ok0_, ok1_;
-    unsigned ok;
+    unsigned ok;         // bit c: element c of the last fetch lies inside the operand
 
-    // element c (0..7) of this thread sits at (k, i) = (kk0 + kdelta(c), ii + idelta(c))
-    static __device__ __forceinline__ int kdelta(int c) { return KMAJOR ? (VEC ? (c >> 2) * 8 : c * 2) : c; }
-    static __device__ __forceinline__ int idelta(int c) { return KMAJOR && VEC ? (c & 3) : 0; }
+    // element c (0..7) of this thread sits at (k, i) = (kk0 + kdelta(c), ii)
+    static __device__ __forceinline__ int kdelta(int c) { return KMAJOR ? c * 2 : c; }
 
     __device__ __forceinline__ void init(const float* base, long long ld_, int i0, int k_begin, int I)
     {
@@ -99,13 +134,8 @@ struct Stager {
         ld = ld_;
         dummy = base;
         if (KMAJOR) {
-            if (VEC) {
-                kk0 = t >> 5;  // rows kk0 and kk0 + 8, four consecutive i
-                ii = (t & 31) * 4;
-            } else {
-                kk0 = t >> 7;  // rows kk0, kk0 + 2, ..., kk0 + 14, one i
-                ii = t & 127;
-            }
+            kk0 = t >> 7;  // rows kk0, kk0 + 2, ..., kk0 + 14, one i
+            ii = t & 127;
             p = base + (long long)(k_begin + kk0) * ld + i0 + ii;
         } else {
             ii = t >> 1;
@@ -119,47 +149,20 @@ struct Stager {
     // waits for the loads before those MFMAs.
     __device__ __forceinline__ void fetch(float (&r)[8], int k_left)
     {
-        if (VEC && (KMAJOR || k_left >= kChunk)) {
-            // K-major: the float4 runs along i, so a partial last chunk only drops whole rows
-            const bool ok0 = i_ok && (!KMAJOR || kk0 < k_left);
-            const bool ok1 = i_ok && (!KMAJOR || kk0 + 8 < k_left);
-            const float* q0 = ok0 ? p : dummy;
-            const float* q1 = ok1 ? p + (KMAJOR ? 8 * ld : 4) : dummy;
-            const float4 v0 = *(const float4*)q0, v1 = *(const float4*)q1;
-            r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
-            r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
-            ok0_ = ok0;
-            ok1_ = ok1;
-            vec_ = true;
-        } else {
-            ok = 0;
-            vec_ = false;
+        ok = 0;
 #pragma unroll
-            for (int c = 0; c < 8; c++) {
-                const bool okc = i_ok && kk0 + kdelta(c) < k_left;
-                const float* qq = okc ? p + (KMAJOR ? (long long)kdelta(c) * ld + idelta(c) : (long long)c) : dummy;
-                r[c] = *qq;
-                ok |= okc ? 1u << c : 0u;
-            }
+        for (int c = 0; c < 8; c++) {
+            const bool okc = i_ok && kk0 + kdelta(c) < k_left;
+            const float* qq = okc ? p + (KMAJOR ? (long long)kdelta(c) * ld : (long long)c) : dummy;
+            r[c] = *qq;
+            ok |= okc ? 1u << c : 0u;
         }
         p += KMAJOR ? (long long)kChunk * ld : (long long)kChunk;
     }
     __device__ __forceinline__ void commit(float (*s)[kLd], float (&r)[8]) const
     {
-        if (VEC && vec_) {
 #pragma unroll
-            for (int c = 0; c < 8; c++) r[c] = (c < 4 ? ok0_ : ok1_) ? r[c] : 0.0f;
-        } else {
-#pragma unroll
-            for (int c = 0; c < 8; c++) r[c] = (ok >> c & 1u) ? r[c] : 0.0f;
-        }
-        if (KMAJOR && VEC) {
-            *(float4*)&s[kk0][ii] = make_float4(r[0], r[1], r[2], r[3]);
-            *(float4*)&s[kk0 + 8][ii] = make_float4(r[4], r[5], r[6], r[7]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < 8; c++) s[kk0 + kdelta(c)][ii] = r[c];
-        }
+        for (int c = 0; c < 8; c++) s[kk0 + kdelta(c)][ii] = (ok >> c & 1u) ? r[c] : 0.0f;
     }
 };
 
@@ -170,7 +173,7 @@ struct Stager {
 // Conditions on single blocks inside one loop make the compiler copy all accumulators between
 // register classes on every trip.
 // v_mfma_f32_32x32x2_f32: lane l feeds A[i = l%32][k = l/32] and B[k = l/32][j = l%32].
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC, int NX, int NY>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int NX, int NY>
 __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChunk][kLd], float (*bs)[kChunk][kLd], int i0,
                                           int j0, int batch, int split, int k_begin, int k_end, int wi, int wj, int l32,
                                           int lk)
@@ -183,8 +186,8 @@ __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChun
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
 
-    Stager<A_KMAJOR, VEC> sa;
-    Stager<B_KMAJOR, VEC> sb;
+    Stager<A_KMAJOR> sa;
+    Stager<B_KMAJOR> sb;
     sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i));
     sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j));
     float ra[8], rb[8];
@@ -246,14 +249,16 @@ __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChun
         }
 }
 
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VEC>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
 // four waves per SIMD (at most 128 registers: four workgroups per CU)
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_gemm_f32(GemmParams q)
 {
     __shared__ __attribute__((aligned(16))) float as[2][kChunk][kLd];
     __shared__ __attribute__((aligned(16))) float bs[2][kChunk][kLd];
-    const int i0 = blockIdx.x * q.tile_i, j0 = blockIdx.y * q.tile_j;
-    const int batch = blockIdx.z / q.splits, split = blockIdx.z - batch * q.splits;
+    int it, jt, z;
+    gemm_tile_of(q, blockIdx.x, it, jt, z);
+    const int i0 = it * q.tile_i, j0 = jt * q.tile_j;
+    const int batch = z / q.splits, split = z - batch * q.splits;
     const int k_begin = split * q.k_per_split;
     const int k_end = min(q.K, k_begin + q.k_per_split);
     // the wave index through readfirstlane: the compiler then knows that everything derived from it
@@ -270,8 +275,327 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const bool y0 = j0 + wj < q.J, y1 = !narrow_i && j0 + wj + 32 < q.J;
     const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
 #define GEO_SC_GEMM_WAVE(NX, NY)                                                                                        \
-    gemm_wave<A_KMAJOR, B_KMAJOR, EPI, VEC, NX, NY>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk)
+    gemm_wave<A_KMAJOR, B_KMAJOR, EPI, NX, NY>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk)
     // every variant runs the same staging and the same number of barriers
+    switch (blocks_xy) {
+    case 3: GEO_SC_GEMM_WAVE(2, 2); break;
+    case 2: GEO_SC_GEMM_WAVE(2, 1); break;
+    case 1: GEO_SC_GEMM_WAVE(1, 2); break;
+    case 0: GEO_SC_GEMM_WAVE(1, 1); break;
+    default: GEO_SC_GEMM_WAVE(0, 0); break;
+    }
+#undef GEO_SC_GEMM_WAVE
+}
+
+// ---- the same GEMM on the bf16 matrix cores, fp32 results ----
+// Every fp32 operand element is split into three bf16 terms (x = hi + mid + lo to 2^-27 |x|: each
+// term is the round-to-nearest bf16 of what the previous ones leave) and a product is formed from
+// the six term products of relative size >= 2^-18 (hi hi, hi mid, mid hi, mid mid, hi lo, lo hi),
+// each exact in fp32 and accumulated in fp32 by v_mfma_f32_32x32x16_bf16; the dropped ones
+// (mid lo, lo mid, lo lo) are below 2^-26 of the product, less than the rounding of an fp32
+// multiply.  Six bf16 MFMAs of 16 k take 6 x 8 passes where eight fp32 MFMAs of 2 k take
+// 8 x 16.  The split happens once per element, when a staged chunk is written to LDS.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+constexpr int kLdx = 132;  // LDS stride between the two k halves of a chunk, in 16-byte slots
+
+// bf16(a) in the low half, bf16(b) in the high half (v_cvt_pk_bf16_f32, round to nearest even)
+__device__ __forceinline__ unsigned pack_bf16(float a, float b)
+{
+    const floatx2 v = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+}
+
+__device__ __forceinline__ void split3(float a, float b, unsigned& hi, unsigned& mid, unsigned& lo)
+{
+    hi = pack_bf16(a, b);
+    const float ra = a - __uint_as_float(hi << 16), rb = b - __uint_as_float(hi & 0xffff0000u);
+    mid = pack_bf16(ra, rb);
+    lo = pack_bf16(ra - __uint_as_float(mid << 16), rb - __uint_as_float(mid & 0xffff0000u));
+}
+
+// Staging for the split kernel: a thread owns eight consecutive k (one half of the chunk) of one i,
+// which is what one lane feeds to the MFMA, and commit() writes them as s[term][k half][i], 16 bytes
+// (four words of two bf16) per term.
+//   K-major operand (element (k, i) at p[k*ld + i]): eight dword loads from a wave-uniform row pointer
+//     each, lanes along i; the k half is the wave's (uniform)
+//   I-major operand (element (k, i) at p[i*ld + k]): two float4 along k
+// Rows i outside the operand are clamped to its last row: what they produce is never stored.  Only a
+// partial last chunk is zeroed beyond its k range.
+template <bool KMAJOR>
+struct SplitStager {
+    const float* p;   // K-major: row k_begin + 8 * half of the operand (uniform); I-major: this thread's first element
+    long long ld;
+    int off;          // K-major: this thread's i (clamped)
+    int half, ii;
+
+    __device__ __forceinline__ void init(const float* base, long long ld_, int i0, int k_begin, int I, int wave)
+    {
+        const int t = threadIdx.x;
+        ld = ld_;
+        if (KMAJOR) {
+            half = wave >> 1;
+            ii = t & 127;
+            off = min(i0 + ii, I - 1);
+            p = base + (long long)(k_begin + 8 * half) * ld;
+        } else {
+            ii = t >> 1;
+            half = t & 1;
+            p = base + (long long)min(i0 + ii, I - 1) * ld + k_begin + 8 * half;
+        }
+    }
+    // a whole chunk, no branches
+    __device__ __forceinline__ void fetch_whole(float (&r)[8])
+    {
+        if (KMAJOR) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = (p + (long long)c * ld)[off];
+            p += (long long)kChunk * ld;
+        } else {
+            const float4 v0 = *(const float4*)p, v1 = *(const float4*)(p + 4);
+            r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+            r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+            p += kChunk;
+        }
+    }
+    // k_left: what is left of the k range from this chunk's start (a partial last chunk has < kChunk)
+    __device__ __forceinline__ void fetch(float (&r)[8], int k_left)
+    {
+        const bool tail = k_left < kChunk;
+        if (KMAJOR) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                // rows past the end of a partial chunk read the chunk's first row instead
+                const long long row = (tail && 8 * half + c >= k_left) ? -8 * half : c;
+                r[c] = (p + row * ld)[off];
+            }
+            p += (long long)kChunk * ld;
+        } else {
+            if (!tail) {
+                const float4 v0 = *(const float4*)p, v1 = *(const float4*)(p + 4);
+                r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+                r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; c++) r[c] = p[8 * half + c < k_left ? c : -8 * half];
+            }
+            p += kChunk;
+        }
+    }
+    __device__ __forceinline__ void commit(uint4 (*s)[2][kLdx], float (&r)[8], int k_left) const
+    {
+        if (k_left < kChunk) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = 8 * half + c < k_left ? r[c] : 0.0f;
+        }
+        commit_whole(s, r);
+    }
+    __device__ __forceinline__ void commit_whole(uint4 (*s)[2][kLdx], const float (&r)[8]) const
+    {
+        unsigned hi[4], mid[4], lo[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) split3(r[2 * c], r[2 * c + 1], hi[c], mid[c], lo[c]);
+        s[0][half][ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        s[1][half][ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        s[2][half][ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    }
+};
+
+// v_mfma_f32_32x32x16_bf16: lane l feeds A[i = l%32][k = 8 (l/32) .. + 7] and B[those k][j = l%32]:
+// the 16 bytes at s[term][l/32][i]; results as in the fp32 instruction.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int NX, int NY>
+__device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)[3][2][kLdx], uint4 (*bs)[3][2][kLdx],
+                                                int i0, int j0, int batch, int split, int k_begin, int k_end, int wi,
+                                                int wj, int l32, int lk, int wave)
+{
+    floatx16 acc[NX ? NX : 1][NY ? NY : 1];
+#pragma unroll
+    for (int x = 0; x < NX; x++)
+#pragma unroll
+        for (int y = 0; y < NY; y++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
+
+    SplitStager<A_KMAJOR> sa;
+    SplitStager<B_KMAJOR> sb;
+    sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
+    sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
+    // Two chunks ahead: while chunk c is multiplied out of LDS, chunk c + 1 sits in one register set
+    // (its loads issued a whole trip ago) and the loads of chunk c + 2 go out into the other.
+    float ra[2][8], rb[2][8];
+    const int k_len = k_end - k_begin;
+    const int n_chunks = k_len > 0 ? (k_len + kChunk - 1) / kChunk : 0;
+    if (n_chunks > 0) {
+        sa.fetch(ra[0], k_len);
+        sb.fetch(rb[0], k_len);
+    }
+    if (n_chunks > 1) {
+        sa.fetch(ra[1], k_len - kChunk);
+        sb.fetch(rb[1], k_len - kChunk);
+    }
+    if (n_chunks > 0) {
+        sa.commit(as[0], ra[0], k_len);
+        sb.commit(bs[0], rb[0], k_len);
+    }
+    __syncthreads();
+    auto multiply = [&](int buf) {
+        bf16x8 a[NX ? NX : 1][3], b[NY ? NY : 1][3];
+#pragma unroll
+        for (int t = 0; t < 3; t++) {
+#pragma unroll
+            for (int x = 0; x < NX; x++) a[x][t] = __builtin_bit_cast(bf16x8, as[buf][t][lk][wi + 32 * x + l32]);
+#pragma unroll
+            for (int y = 0; y < NY; y++) b[y][t] = __builtin_bit_cast(bf16x8, bs[buf][t][lk][wj + 32 * y + l32]);
+        }
+        // smallest terms first; 0 = hi, 1 = mid, 2 = lo
+        constexpr int ta[6] = {2, 0, 1, 1, 0, 0}, tb[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+        for (int t = 0; t < 6; t++)
+#pragma unroll
+            for (int x = 0; x < NX; x++)
+#pragma unroll
+                for (int y = 0; y < NY; y++)
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x][ta[t]], b[y][tb[t]], acc[x][y], 0, 0, 0);
+    };
+    int c = 0;
+    // Whole chunks, no branches in the trip.  The split of chunk c + 1 (vector ALU, 24 steps: three per
+    // pair of elements) is written between the MFMAs of chunk c, one step per MFMA with four blocks, and
+    // scheduling barriers keep that order, so that it issues while the matrix pipe is busy.
+    const int n_whole = k_len > 0 ? k_len / kChunk : 0;
+    constexpr int kMfmas = NX * NY > 0 ? 6 * NX * NY : 1;  // per trip
+    constexpr int kStepsPerMfma = (24 + kMfmas - 1) / kMfmas;
+    auto multiply_and_split = [&](auto set) {
+        constexpr int S = decltype(set)::value;
+        sa.fetch_whole(ra[S]);
+        sb.fetch_whole(rb[S]);
+        bf16x8 a[NX ? NX : 1][3], b[NY ? NY : 1][3];
+#pragma unroll
+        for (int t = 0; t < 3; t++) {
+#pragma unroll
+            for (int x = 0; x < NX; x++) a[x][t] = __builtin_bit_cast(bf16x8, as[S][t][lk][wi + 32 * x + l32]);
+#pragma unroll
+            for (int y = 0; y < NY; y++) b[y][t] = __builtin_bit_cast(bf16x8, bs[S][t][lk][wj + 32 * y + l32]);
+        }
+        constexpr int ta[6] = {2, 0, 1, 1, 0, 0}, tb[6] = {0, 2, 1, 0, 1, 0};
+        // pairs 0..3: this thread's elements of A, 4..7: of B
+        unsigned hi[8], mid[8], lo[8];
+        float r0[8], r1[8];
+        auto step = [&](int n) {
+            const int pr = n / 3, st = n % 3;
+            const float* src = pr < 4 ? ra[S ^ 1] : rb[S ^ 1];
+            const int e = 2 * (pr & 3);
+            if (st == 0) {
+                hi[pr] = pack_bf16(src[e], src[e + 1]);
+                r0[pr] = src[e] - __uint_as_float(hi[pr] << 16);
+                r1[pr] = src[e + 1] - __uint_as_float(hi[pr] & 0xffff0000u);
+            } else if (st == 1) {
+                mid[pr] = pack_bf16(r0[pr], r1[pr]);
+                r0[pr] -= __uint_as_float(mid[pr] << 16);
+                r1[pr] -= __uint_as_float(mid[pr] & 0xffff0000u);
+            } else {
+                lo[pr] = pack_bf16(r0[pr], r1[pr]);
+            }
+        };
+#pragma unroll
+        for (int m = 0; m < kMfmas; m++) {
+            constexpr int kBlocks = NX * NY > 0 ? NX * NY : 1, kNy = NY > 0 ? NY : 1;
+            const int t = m / kBlocks, x = (m % kBlocks) / kNy, y = m % kNy;
+            acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x][ta[t]], b[y][tb[t]], acc[x][y], 0, 0, 0);
+#pragma unroll
+            for (int n = m * kStepsPerMfma; n < (m + 1) * kStepsPerMfma && n < 24; n++) step(n);
+        }
+        as[S ^ 1][0][sa.half][sa.ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        as[S ^ 1][1][sa.half][sa.ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        as[S ^ 1][2][sa.half][sa.ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        bs[S ^ 1][0][sb.half][sb.ii] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        bs[S ^ 1][1][sb.half][sb.ii] = make_uint4(mid[4], mid[5], mid[6], mid[7]);
+        bs[S ^ 1][2][sb.half][sb.ii] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        // order asked of the scheduler: LDS reads, then one MFMA and a share of the vector ALU work in turn
+        __builtin_amdgcn_sched_group_barrier(0x100, 3 * (NX + NY), 0);
+#pragma unroll
+        for (int m = 0; m < kMfmas; m++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, (88 + kMfmas - 1) / kMfmas, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x200, 6, 0);
+        __syncthreads();
+    };
+    if (NX * NY > 0) {
+        for (; c + 3 < n_whole; c += 2) {
+            multiply_and_split(std::integral_constant<int, 0>());
+            multiply_and_split(std::integral_constant<int, 1>());
+        }
+    }
+    for (; c + 1 < n_chunks; c += 2) {
+        // chunk c from LDS buffer 0; register set 1 holds chunk c + 1
+        if (c + 2 < n_chunks) {
+            sa.fetch(ra[0], k_len - (c + 2) * kChunk);
+            sb.fetch(rb[0], k_len - (c + 2) * kChunk);
+        }
+        multiply(0);
+        sa.commit(as[1], ra[1], k_len - (c + 1) * kChunk);
+        sb.commit(bs[1], rb[1], k_len - (c + 1) * kChunk);
+        __syncthreads();
+        // chunk c + 1 from LDS buffer 1; register set 0 holds chunk c + 2
+        if (c + 3 < n_chunks) {
+            sa.fetch(ra[1], k_len - (c + 3) * kChunk);
+            sb.fetch(rb[1], k_len - (c + 3) * kChunk);
+        }
+        multiply(1);
+        if (c + 2 < n_chunks) {
+            sa.commit(as[0], ra[0], k_len - (c + 2) * kChunk);
+            sb.commit(bs[0], rb[0], k_len - (c + 2) * kChunk);
+        }
+        __syncthreads();
+    }
+    if (c < n_chunks) multiply(0);  // an odd last chunk, already in buffer 0
+
+    float* out = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
+#pragma unroll
+    for (int x = 0; x < NX; x++)
+#pragma unroll
+        for (int y = 0; y < NY; y++) {
+            const int j = j0 + wj + y * 32 + l32;
+            if (j >= q.J) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = i0 + wi + x * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
+                if (i >= q.I) continue;
+                float v = acc[x][y][r];
+                if (EPI == EPI_EXP_TIMES_G) {
+                    const int co = j >= q.c_out ? j - q.c_out : j;
+                    v = q.g[(long long)i * q.c_out + co] * exp_neg(v);
+                }
+                out[(long long)i * q.ldc + j] = v;
+            }
+        }
+}
+
+// Operands with 16-byte aligned rows and chunks (launch_gemm checks).
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+// three waves per SIMD (at most 168 registers; three workgroups' LDS fit a CU)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void k_gemm_split(GemmParams q)
+{
+    __shared__ uint4 as[2][3][2][kLdx];
+    __shared__ uint4 bs[2][3][2][kLdx];
+    int it, jt, z;
+    gemm_tile_of(q, blockIdx.x, it, jt, z);
+    const int i0 = it * q.tile_i, j0 = jt * q.tile_j;
+    const int batch = z / q.splits, split = z - batch * q.splits;
+    const int k_begin = split * q.k_per_split;
+    const int k_end = min(q.K, k_begin + q.k_per_split);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const bool narrow_j = q.tile_j < kTile, narrow_i = q.tile_i < kTile;
+    const int wi = narrow_j ? wave * 32 : narrow_i ? 0 : (wave >> 1) * 64;
+    const int wj = narrow_j ? 0 : narrow_i ? wave * 32 : (wave & 1) * 64;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const bool x0 = i0 + wi < q.I, x1 = !narrow_j && i0 + wi + 32 < q.I;
+    const bool y0 = j0 + wj < q.J, y1 = !narrow_i && j0 + wj + 32 < q.J;
+    const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
+#define GEO_SC_GEMM_WAVE(NX, NY)                                                                                        \
+    gemm_wave_split<A_KMAJOR, B_KMAJOR, EPI, NX, NY>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk, wave)
     switch (blocks_xy) {
     case 3: GEO_SC_GEMM_WAVE(2, 2); break;
     case 2: GEO_SC_GEMM_WAVE(2, 1); break;
@@ -894,16 +1218,33 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
     auto half_tiles = [](int n) { return n <= 3 * kTile / 2 && (n - 1) % kTile < kTile / 2; };
     q.tile_j = half_tiles(q.J) ? kTile / 2 : kTile;
     q.tile_i = q.tile_j == kTile && half_tiles(q.I) ? kTile / 2 : kTile;
-    dim3 grid((q.I + q.tile_i - 1) / q.tile_i, (q.J + q.tile_j - 1) / q.tile_j, q.splits * batch);
-    // float4 staging needs every row start and every chunk start on a 16-byte boundary
-    const bool a_vec = q.lda % 4 == 0 && ((uintptr_t)q.a & 15) == 0 && q.a_batch_stride % 4 == 0 && (AK ? q.I % 4 == 0 : true);
-    const bool b_vec = q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0 && (BK ? q.J % 4 == 0 : true);
-    // an operand stored I-major moves float4 along k: its chunks must start on multiples of 4
-    const bool k_vec = (AK && BK) || q.k_per_split % 4 == 0;
-    if (a_vec && b_vec && k_vec)
-        hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
+    q.ni = (q.I + q.tile_i - 1) / q.tile_i;
+    q.nj = (q.J + q.tile_j - 1) / q.tile_j;
+    q.nz = q.splits * batch;
+    if ((long long)q.ni * q.nj <= 16) {
+        q.cluster_of = 2;
+        q.cluster = q.ni * q.nj;
+    } else if (q.nj <= q.ni) {
+        q.cluster_of = 0;
+        q.cluster = q.nj;
+    } else {
+        q.cluster_of = 1;
+        q.cluster = q.ni;
+    }
+    const long long n_groups = (long long)q.ni * q.nj * q.nz;
+    if (n_groups > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)n_groups);
+    // The split kernel reads a K-major operand with dword loads and an I-major one with float4 along k:
+    // every row start and every chunk start of the latter must lie on a 16-byte boundary.
+    auto rows_aligned = [&](const float* base, long long ld, long long batch_stride) {
+        return ld % 4 == 0 && ((uintptr_t)base & 15) == 0 && batch_stride % 4 == 0 && q.k_per_split % 4 == 0;
+    };
+    const bool a_vec = AK || rows_aligned(q.a, q.lda, q.a_batch_stride);
+    const bool b_vec = BK || rows_aligned(q.b, q.ldb, q.b_batch_stride);
+    if (a_vec && b_vec)
+        hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI>), grid, dim3(256), 0, s, q);
     else
-        hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI, false>), grid, dim3(256), 0, s, q);
+        hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI>), grid, dim3(256), 0, s, q);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

@@ -59,6 +59,35 @@ def test_backward_matches_float64_oracle(capi, shape_x, shape_w, pad, mode, scal
     assert torch.equal(gx2, gx) and rel_err(gw2, gw) <= 1e-6 and rel_err(gw2, rw) <= RTOL
 
 
+GEMM_CASES = [
+    # OR groups of more than 32 members take the three-GEMM path (K = c_in * w_k members per kernel row)
+    ((3, 12, 5, 3), (5, 12, 3, 1), (1, 0), 3.0),      # K = 36; 45 positions and 10 rails: unaligned operands (fp32 kernel)
+    ((4, 20, 6, 6), (6, 20, 2, 3), (0, 1), 2.0),      # K = 40: two whole chunks and a partial one
+    ((2, 16, 9, 8), (8, 16, 5, 2), (2, 0), 2.0),      # K = 80: five whole chunks
+    ((2, 64, 17, 16), (70, 64, 2, 1), (0, 0), 6.0),   # K = 128, four position tiles, 140 rails: a ragged second column tile
+    ((4, 24, 10, 10), (20, 24, 2, 2), (0, 0), 3.0),   # K = 48, 40 rails: 64-wide column tiles
+    ((4, 11, 20, 20), (16, 11, 3, 3), (1, 1), 2.0),   # K = 33: 1600 positions split over workgroups, a 1-member tail chunk
+    ((1, 40, 4, 6), (3, 40, 1, 3), (0, 1), 2.0),      # K = 40 with 24 positions and 6 rails: one partly filled tile, unaligned rails
+]
+
+
+@pytest.mark.parametrize("shape_x,shape_w,pad,scale", GEMM_CASES)
+def test_backward_through_the_gemm_kernels(capi, shape_x, shape_w, pad, scale):
+    """Chunk counts, partial chunks, edge tiles and operand alignments of the GEMM kernels (bf16 three-way
+    split products for aligned operands, fp32 MFMAs otherwise) against the float64 oracle."""
+    from oracle import surrogate
+    x, w = wl.make_inputs(shape_x, shape_w, "kaiming", seed=shape_x[1])
+    w = (w * scale).contiguous()
+    w.view(-1)[::5] = 0.0
+    d = capi.make_desc(x.shape, w.shape, 128, pad)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(2))
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad)
+    torch.cuda.synchronize()
+    rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad)
+    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
+    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+
+
 def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
     """128->128 3x3 at 16x16, batch 256: against torch's own fp32 autograd over the surrogate
     (the float64 oracle on the CPU would take minutes), plus linearity in grad_y."""
