@@ -166,6 +166,45 @@ struct Stager {
     }
 };
 
+// Epilogue of one wave: accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of a
+// 32 x 32 block; (iw, jw) is the wave's corner in the result.  No branches around the loads of the
+// upstream gradient: they go out 16 at a time from clamped addresses, then the exponentials, then
+// stores under the range conditions (a load inside a per-element branch is waited for element by
+// element: 64 memory latencies in a row).
+template <int EPI, int NX, int NY>
+__device__ __forceinline__ void store_tile(const GemmParams& q, const floatx16 (&acc)[NX ? NX : 1][NY ? NY : 1],
+                                           float* __restrict__ out, int iw, int jw, int l32, int lk)
+{
+#pragma unroll
+    for (int x = 0; x < NX; x++)
+#pragma unroll
+        for (int y = 0; y < NY; y++) {
+            const int j = jw + y * 32 + l32;
+            const bool j_ok = j < q.J;
+            const int ib = iw + x * 32 + 4 * lk;
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 16; r++) v[r] = acc[x][y][r];
+            if (EPI == EPI_EXP_TIMES_G) {
+                const int jc = j_ok ? j : q.J - 1;
+                const int co = jc >= q.c_out ? jc - q.c_out : jc;
+                float gv[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int i = min(ib + 8 * (r >> 2) + (r & 3), q.I - 1);
+                    gv[r] = q.g[(long long)i * q.c_out + co];
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) v[r] = gv[r] * exp_neg(v[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = ib + 8 * (r >> 2) + (r & 3);
+                if (j_ok && i < q.I) out[(long long)i * q.ldc + j] = v[r];
+            }
+        }
+}
+
 // The K loop and the epilogue of one wave that owns the first NX x NY of its 2 x 2 blocks of
 // 32 x 32 (edge tiles and narrow operands leave blocks without results; NX = 0: none, the wave only
 // stages).  A function of its own per (NX, NY), entered through a wave-uniform switch: the
@@ -227,26 +266,7 @@ __device__ __forceinline__ void gemm_wave(const GemmParams& q, float (*as)[kChun
         buf ^= 1;
     }
 
-    // accumulator register r of lane l holds C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile
-    float* c = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
-#pragma unroll
-    for (int x = 0; x < NX; x++)
-#pragma unroll
-        for (int y = 0; y < NY; y++) {
-            const int j = j0 + wj + y * 32 + l32;
-            if (j >= q.J) continue;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int i = i0 + wi + x * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                if (i >= q.I) continue;
-                float v = acc[x][y][r];
-                if (EPI == EPI_EXP_TIMES_G) {
-                    const int co = j >= q.c_out ? j - q.c_out : j;
-                    v = q.g[(long long)i * q.c_out + co] * exp_neg(v);
-                }
-                c[(long long)i * q.ldc + j] = v;
-            }
-        }
+    store_tile<EPI, NX, NY>(q, acc, q.c + batch * q.c_batch_stride + split * q.c_split_stride, i0 + wi, j0 + wj, l32, lk);
 }
 
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
@@ -552,25 +572,7 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
     }
     if (c < n_chunks) multiply(0);  // an odd last chunk, already in buffer 0
 
-    float* out = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
-#pragma unroll
-    for (int x = 0; x < NX; x++)
-#pragma unroll
-        for (int y = 0; y < NY; y++) {
-            const int j = j0 + wj + y * 32 + l32;
-            if (j >= q.J) continue;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int i = i0 + wi + x * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                if (i >= q.I) continue;
-                float v = acc[x][y][r];
-                if (EPI == EPI_EXP_TIMES_G) {
-                    const int co = j >= q.c_out ? j - q.c_out : j;
-                    v = q.g[(long long)i * q.c_out + co] * exp_neg(v);
-                }
-                out[(long long)i * q.ldc + j] = v;
-            }
-        }
+    store_tile<EPI, NX, NY>(q, acc, q.c + batch * q.c_batch_stride + split * q.c_split_stride, i0 + wi, j0 + wj, l32, lk);
 }
 
 // Operands with 16-byte aligned rows and chunks (launch_gemm checks).
@@ -1241,10 +1243,14 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
     };
     const bool a_vec = AK || rows_aligned(q.a, q.lda, q.a_batch_stride);
     const bool b_vec = BK || rows_aligned(q.b, q.ldb, q.b_batch_stride);
-    if (a_vec && b_vec)
+    if constexpr (AK && BK) {
         hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI>), grid, dim3(256), 0, s, q);
-    else
-        hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI>), grid, dim3(256), 0, s, q);
+    } else {
+        if (a_vec && b_vec)
+            hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI>), grid, dim3(256), 0, s, q);
+        else
+            hipLaunchKernelGGL((k_gemm_f32<AK, BK, EPI>), grid, dim3(256), 0, s, q);
+    }
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
