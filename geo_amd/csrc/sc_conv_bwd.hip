@@ -746,15 +746,22 @@ __global__ __launch_bounds__(256) void k_im2col_rows(const float* __restrict__ x
     const int k1 = min(G.n_members, k0 + kIm2colMembers);
     float* colg = col + (size_t)blockIdx.z * g_stride;
     for (int m = blockIdx.x * 256 + threadIdx.x; m < m_total; m += gridDim.x * 256) {
-        const int r0 = arow[m], c0 = bcol[m];
-        const float* src = x + base[m];
+        const int r0 = arow[m], c0 = bcol[m], b0 = base[m];
+        // all loads first, from x[0] where the member lies in the padding (a load inside a branch is
+        // waited for before the next one is issued), then the stores
+        float vals[kIm2colMembers];
         Member e = member_of(G, g, k0);
-        for (int k = k0; k < k1; k++, next_member(G, e)) {
+#pragma unroll
+        for (int q = 0; q < kIm2colMembers; q++) {
             const int r = r0 + e.u, c = c0 + e.v;
-            float val = 0.0f;
-            if (e.ok && c >= 0 && c < h_in && r >= 0 && r < w_in) val = src[(e.ci * w_in + e.u) * h_in + e.v];
-            colg[(size_t)k * m_total + m] = val;
+            const bool ok = k0 + q < k1 && e.ok && c >= 0 && c < h_in && r >= 0 && r < w_in;
+            const float val = x[ok ? b0 + (e.ci * w_in + e.u) * h_in + e.v : 0];
+            vals[q] = ok ? val : 0.0f;
+            next_member(G, e);
         }
+#pragma unroll
+        for (int q = 0; q < kIm2colMembers; q++)
+            if (k0 + q < k1) colg[(size_t)(k0 + q) * m_total + m] = vals[q];
     }
 }
 
@@ -848,11 +855,20 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
                 // the group does not depend on u, and the member index advances by k_step per tap
                 int g, k;
                 group_of(G, ci, 0, v, g, k);
-                if (g < g0 || g >= g0 + ng || b < 0 || b >= ho) continue;
-                const float* sg = src + (size_t)(g - g0) * g_stride + (size_t)k * m_total + b;
-                for (int u = 0; u < G.w_k; u++) {
-                    const int a = p + pad_w - u;
-                    if (a >= 0 && a < wo) s += sg[(size_t)u * k_step * m_total + a * ho];
+                if (g < g0 || g >= g0 + ng) continue;  // uniform
+                const bool b_ok = b >= 0 && b < ho;
+                const float* sg = src + (size_t)(g - g0) * g_stride + (size_t)k * m_total + (b_ok ? b : 0);
+                // four taps at a time: loads from clamped addresses first, then the sum
+                for (int u0 = 0; u0 < G.w_k; u0 += 4) {
+                    float t[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int u = u0 + q, a = p + pad_w - u;
+                        const bool ok = b_ok && u < G.w_k && a >= 0 && a < wo;
+                        const float val = sg[ok ? (size_t)u * k_step * m_total + a * ho : 0];
+                        t[q] = ok ? val : 0.0f;
+                    }
+                    s += (t[0] + t[1]) + (t[2] + t[3]);
                 }
             }
             dst[e] = g0 == 0 ? s : dst[e] + s;
