@@ -568,6 +568,120 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
 }
 
+// k_conv_fwd_rail for 3-wide kernels with the activation words staged through LDS.  The waves of the
+// c_out tiles of one position tile read the same four activation words per lane and channel; here
+// NWV of them form a workgroup, every wave fetches 8 / NWV channels of a chunk of 8 and leaves them in
+// LDS as 16 bytes per lane, and all read them back with one ds_read_b128 per channel: an eighth (a
+// quarter) of the global loads per wave, and the wait in front of a channel's 96 vector instructions is
+// for LDS and the scalar cache instead of the vector memory path.  The chunks are double-buffered:
+// the loads of chunk t + 1 are issued before chunk t is computed and written to LDS after it, one
+// barrier per chunk.  Needs c_in % 8 == 0 and n_cotile % NWV == 0 (the launcher checks).
+constexpr int kStageChannels = 8;
+template <int NWV>
+__global__ __launch_bounds__(64 * NWV) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_rail_lds(FwdParams q)
+{
+    constexpr int C = kCoTile, R = 2, WK = 3, NW = R + WK - 1, CH = kStageChannels, CPW = CH / NWV;
+    static_assert(NW == 4 && CH % NWV == 0, "a lane's words of one channel are one uint4");
+    __shared__ uint4 stage[2][CH][64];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int cot_groups = q.n_cotile / NWV;
+    const int cot = (blockIdx.x % cot_groups) * NWV + wave;
+    const long long slot0 = (long long)(blockIdx.x / cot_groups) * 64 + lane;
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : 0;
+    const int b = (int)(slot % q.ho);
+    const long long t = slot / q.ho;
+    const int a0 = (int)(t % q.row_groups) * R;
+    const long long n = t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
+    unsigned off[NW];
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+        const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+        off[j] = (unsigned)row * q.hi;
+    }
+    const unsigned ch_stride = (unsigned)q.wi * q.hi;
+    const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
+    const int k_or = q.c_in * WK;
+    const int chunks_per_pass = q.c_in / CH;
+    const int passes = q.packs * q.h_k;
+    const int total = passes * chunks_per_pass;
+
+    int sum[2 * C];  // [2 c + r]
+#pragma unroll
+    for (int i = 0; i < 2 * C; i++) sum[i] = 0;
+
+    // this wave's channels of chunk (pass, cc): wave + NWV * i
+    uint4 fetched[CPW];
+    auto fetch = [&](int pass, int cc) {
+        const int p = pass / q.h_k, v = pass - p * q.h_k;
+        const uint32_t* ap = act_n + (size_t)p * q.act_plane + v + (size_t)(cc * CH + wave) * ch_stride;
+#pragma unroll
+        for (int i = 0; i < CPW; i++) {
+            const uint32_t* ac = ap + (size_t)(NWV * i) * ch_stride;
+            fetched[i] = make_uint4(ac[off[0]], ac[off[1]], ac[off[2]], ac[off[3]]);
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < CPW; i++) stage[buf][wave + NWV * i][lane] = fetched[i];
+    };
+
+    const size_t line0 = (size_t)cot * q.rail_lines;
+    const uint32_t* wp = q.wgt_rail + line0 * C;
+    const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
+    fetch(0, 0);
+    commit(0);
+    __syncthreads();
+    int tc = 0;
+    for (int pass = 0; pass < passes; pass++) {
+        u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
+        for (int cc = 0; cc < chunks_per_pass; cc++, tc++) {
+            const int buf = tc & 1;
+            // the chunk after this one may belong to the next pass
+            const bool last_of_pass = cc + 1 == chunks_per_pass;
+            const bool more = tc + 1 < total;
+            if (more) fetch(last_of_pass ? pass + 1 : pass, last_of_pass ? 0 : cc + 1);
+            for (int ch = 0; ch < CH; ch++) {
+                const uint4 aw = stage[buf][ch][lane];
+                uint32_t wv[WK][C], iv[WK][C / 2];
+#pragma unroll
+                for (int l = 0; l < WK; l++) {
+#pragma unroll
+                    for (int c = 0; c < C; c++) wv[l][c] = wp[l * C + c];
+#pragma unroll
+                    for (int c = 0; c < C / 2; c++) iv[l][c] = ip[l * (C / 2) + c];
+                }
+                rail_line(p0, p1, n0, n1, wv[0], iv[0], aw.x, aw.y);
+                rail_line(p0, p1, n0, n1, wv[1], iv[1], aw.y, aw.z);
+                rail_line(p0, p1, n0, n1, wv[2], iv[2], aw.z, aw.w);
+                wp += WK * C;
+                ip += WK * (C / 2);
+            }
+            if (more) commit(buf ^ 1);
+            __syncthreads();
+        }
+        // end of a (pack, kernel row) pass: binary add across kernel rows and packs
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            sum[i] += __popc(p0[i]) - __popc(n0[i]);
+            sum[C + i] += __popc(p1[i]) - __popc(n1[i]);
+        }
+    }
+
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const int co = cot * C + c;
+        if (co >= q.c_out) break;
+        int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[2 * c + r];
+    }
+}
+
 // The rail-skipping form of k_conv_fwd_split<2, WK, 1, false>: launches split over blockIdx.y and
 // the accumulation modes other than y, position-major activation streams, two output rows per lane.
 // Partial sums are added to the zeroed y with integer atomics.
@@ -843,7 +957,15 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
             // two channels per trip for 1-wide kernels: with three, the six address pairs push the 32
             // sums out of the 128 registers
             constexpr int CR = WK == 1 ? 2 : 1;
-            if (plain)
+            if (plain && WK == 3 && g.c_in % kStageChannels == 0 && g.n_cotile % 4 == 0) {
+                // c_out tiles of one position tile share their activation words through LDS
+                const int nwv = g.n_cotile % 8 == 0 ? 8 : 4;
+                const dim3 grid_lds((unsigned)(tiles * (g.n_cotile / nwv)));
+                if (nwv == 8)
+                    hipLaunchKernelGGL((k_conv_fwd_rail_lds<8>), grid_lds, dim3(512), 0, s, q);
+                else
+                    hipLaunchKernelGGL((k_conv_fwd_rail_lds<4>), grid_lds, dim3(256), 0, s, q);
+            } else if (plain)
                 hipLaunchKernelGGL((k_conv_fwd_rail<WK, CR>), grid, dim3(64), 0, s, q);
             else
                 hipLaunchKernelGGL((k_conv_fwd_split_rail<WK, CR>), grid, dim3(64), 0, s, q);
