@@ -400,7 +400,8 @@ def main():
                      "bwd_min": min(bwd_ms) if with_bwd else None},
         "roofline": {
             "bound": "valu",
-            "kernel": ("k_conv_fwd_rail (v_and_or_b32 on register-indexed accumulators: one rail per weight)"
+            "kernel": ("k_conv_fwd_rail / k_conv_fwd_rail_lds (v_and_or_b32 on register-indexed accumulators: one "
+                       "rail per weight; the _lds form shares activation words between c_out tiles through LDS)"
                        if rail else "k_conv_fwd (v_and_or_b32 / v_bcnt_u32_b32)"),
             "achieved": achieved / 1e12,
             "peak": PEAK_VALU_WORD_OPS / 1e12,
