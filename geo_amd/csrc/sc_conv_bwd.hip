@@ -1,4 +1,4 @@
-// Surrogate-gradient backward of the SC convolution (gfx950, fp32, MFMA).
+// Surrogate-gradient backward of the SC convolution (gfx950, fp32 results, MFMA).
 //
 // The reference trains through a floating-point surrogate of the SC layer
 // (utils_functional.py:611-634, :235-252): with wp = clamp(w,0,100), wn = -clamp(w,-100,0)
@@ -15,9 +15,11 @@
 //     Z  [m][j]  = sum_k col[m][k] * Wcat[k][j]        m=(n,a,b)  k=(ci,u)  j=(rail,co)
 //     Gw [k][j]  = sum_m col[m][k] * E[m][j]
 //     dcol[k][m] = sum_j Wd[j][k]  * E[m][j]           Wd = (wp ; -wn)
-// All three run on one MFMA kernel (v_mfma_f32_32x32x2_f32, fp32 in, fp32 accumulate) that
-// takes each operand either K-major or I-major; exp and the product with g are fused into
-// the first GEMM's epilogue; the second is split over m and reduced deterministically.
+// All three run on MFMA kernels (fp32 in, fp32 accumulate, fp32 out) that take each operand either
+// K-major or I-major: k_gemm_split forms every fp32 product from six bf16 MFMA products of a three-way
+// split of the operands (aligned operands), k_gemm_f32 uses v_mfma_f32_32x32x2_f32 (any alignment);
+// exp and the product with g are fused into the first GEMM's epilogue; the second is split over m
+// and reduced deterministically.
 //
 // The other accumulation modes have the same surrogate with other add groups
 // (utils_functional.py:254-299): one exponential per add group, whose argument sums the OR
