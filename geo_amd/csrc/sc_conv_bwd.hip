@@ -1319,9 +1319,11 @@ BwdLayout bwd_layout(const Geometry& g)
         if (want > 65535) want = 65535;
         b.fused_splits = (int)(want < 1 ? 1 : want);
     }
-    // split the m-reduction of the weight gradient so that the grid covers the GPU
+    // split the m-reduction of the weight gradient so that all groups' tiles together make about two
+    // rounds of workgroups (three per CU): more splits only add partial sums to write and reduce
     const long long tiles = (long long)((K + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
-    long long want = (1024 + tiles - 1) / tiles;
+    long long want = 1536 / (tiles * b.G.n_groups);
+    if (want < 1) want = 1;
     long long per = (b.m_total + want - 1) / want;
     per = (per + kChunk - 1) / kChunk * kChunk;
     if (per < 256) per = 256;
