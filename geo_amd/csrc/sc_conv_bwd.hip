@@ -852,7 +852,10 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
         for (int e = blockIdx.y * 256 + threadIdx.x; e < plane; e += gridDim.y * 256) {
             const int p = e / h_in, qq = e - p * h_in;
             float s = 0.0f;
-            for (int v = 0; v < G.h_k; v++) {
+            // kernel rows v whose output column b = qq + pad_h - v exists (a 1 x 256 kernel on a 256-wide
+            // input has one such row per element, not 256)
+            const int v_lo = max(0, qq + pad_h - (ho - 1)), v_hi = min(G.h_k - 1, qq + pad_h);
+            for (int v = v_lo; v <= v_hi; v++) {
                 const int b = qq + pad_h - v;
                 // the group does not depend on u, and the member index advances by k_step per tap
                 int g, k;
