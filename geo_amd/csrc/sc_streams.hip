@@ -313,8 +313,9 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams_grouped(
 // :524-545, :1319-1333, which draw from cuRAND per-thread states).  Here every element owns a
 // counter-based Philox4x32-10 sequence: counter (block, index_lo, index_hi, tag), key (seed, 0);
 // word j of the element is output j % 4 of block j / 4.  Results do not depend on the launch shape.
-//   GEO_SC_GEN_RAND: bit t = [code > field (t % cpw) of word t / cpw], n_bits-wide fields from the
-//                    least significant end, cpw = 32 / n_bits: independent Bernoulli(code / L) bits
+//   GEO_SC_GEN_RAND: bit t = [code > low n_bits bits of byte t % 4 of word t / 4], bytes from the
+//                    least significant end: independent Bernoulli(code / L) bits.  The four comparisons
+//                    of a word run as two subtractions on 16-bit lanes.
 //   GEO_SC_GEN_ACC : bit t = [r16 * left_total < left_ones * 65536] with the 16-bit halves of word
 //                    t / 2; left_ones -= bit, left_total -= 1: exactly `code` ones
 __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
@@ -322,8 +323,10 @@ __device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
 {
 #pragma unroll
     for (int r = 0; r < 10; r++) {
-        const uint32_t h0 = __umulhi(0xD2511F53u, c0), l0 = 0xD2511F53u * c0;
-        const uint32_t h1 = __umulhi(0xCD9E8D57u, c2), l1 = 0xCD9E8D57u * c2;
+        // one 32 x 32 -> 64 multiply per product (v_mad_u64_u32) instead of separate high and low halves
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t h0 = (uint32_t)(p0 >> 32), l0 = (uint32_t)p0;
+        const uint32_t h1 = (uint32_t)(p1 >> 32), l1 = (uint32_t)p1;
         const uint32_t n0 = h1 ^ c1 ^ k0, n2 = h0 ^ c3 ^ k1;
         c0 = n0;
         c1 = l1;
@@ -345,8 +348,7 @@ struct RandParams {
 };
 
 // The P stream words of one element, handed to put(pack, word).  Bits are produced in stream
-// order, one Philox block (four words) at a time: field f of word w of block blk is stream bit
-// (4*blk + w) * cpw + f.
+// order, one Philox block (four words) at a time.
 template <typename Put>
 __device__ __forceinline__ void random_stream(const RandParams& rp, int code, uint32_t tag, uint64_t index, Put put)
 {
@@ -354,32 +356,55 @@ __device__ __forceinline__ void random_stream(const RandParams& rp, int code, ui
         for (int p = 0; p < rp.packs; p++) put(p, 0u);
         return;
     }
-    const bool bernoulli = rp.generator == GEO_SC_GEN_RAND;
-    const int cpw = bernoulli ? 32 / rp.n_bits : 2;
-    const int shift = bernoulli ? rp.n_bits : 16;
-    const uint32_t mask = bernoulli ? (uint32_t)(rp.L - 1) : 0xffffu;
-    uint32_t left_ones = (uint32_t)code, left_total = (uint32_t)rp.L;
     uint32_t word = 0;
     int t = 0, in_word = 0, p = 0;
+    if (rp.generator == GEO_SC_GEN_RAND) {
+        // code > r on the bytes of a word, two per subtraction: with c = (code - 1) | 0x100 in both 16-bit
+        // lanes and r < 0x100, bit 8 of a lane of c - r is set exactly when code - 1 >= r, and no lane borrows
+        const uint32_t lane_mask = (uint32_t)(rp.L - 1) * 0x00010001u;
+        const uint32_t c = (((uint32_t)code - 1u) | 0x100u) * 0x00010001u;
+        for (uint32_t blk = 0; t < rp.L; blk++) {
+            uint32_t r[4];
+            philox4x32_10(blk, (uint32_t)index, (uint32_t)(index >> 32), tag, rp.seed, 0u, r);
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                if (t < rp.L) {
+                    const uint32_t even = ((c - (r[w] & lane_mask)) >> 8) & 0x00010001u;         // bytes 0 and 2
+                    const uint32_t odd = ((c - ((r[w] >> 8) & lane_mask)) >> 8) & 0x00010001u;   // bytes 1 and 3
+                    // stream order, earlier bits more significant: byte 0, 1, 2, 3
+                    const uint32_t nibble = ((even * 8u + odd * 4u) & 0xcu) | ((even >> 15) + (odd >> 16));
+                    word = word * 16u + nibble;
+                    t += 4;
+                    in_word += 4;
+                    if (in_word == rp.bit_unit) {
+                        put(p++, word);
+                        word = 0;
+                        in_word = 0;
+                    }
+                }
+            }
+        }
+        return;
+    }
+    uint32_t left_ones = (uint32_t)code, left_total = (uint32_t)rp.L;
     for (uint32_t blk = 0; t < rp.L; blk++) {
         uint32_t r[4];
         philox4x32_10(blk, (uint32_t)index, (uint32_t)(index >> 32), tag, rp.seed, 0u, r);
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            uint32_t rw = r[w];
-            for (int f = 0; f < cpw && t < rp.L; f++, t++) {
-                const uint32_t field = rw & mask;
-                rw >>= shift;
-                uint32_t bit;
-                if (bernoulli) {
-                    bit = (uint32_t)code > field;
-                } else {
-                    bit = field * left_total < left_ones * 65536u;
+            if (t < rp.L) {
+#pragma unroll
+                for (int f = 0; f < 2; f++) {
+                    const uint32_t field = f == 0 ? (r[w] & 0xffffu) : (r[w] >> 16);
+                    // both factors are below 2^24
+                    const uint32_t bit = __umul24(field, left_total) < (left_ones << 16);
                     left_ones -= bit;
                     left_total -= 1u;
+                    word = word * 2u + bit;
                 }
-                word = word * 2u + bit;
-                if (++in_word == rp.bit_unit) {
+                t += 2;
+                in_word += 2;
+                if (in_word == rp.bit_unit) {
                     put(p++, word);
                     word = 0;
                     in_word = 0;

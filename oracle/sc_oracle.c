@@ -439,8 +439,8 @@ void sco_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
 /* Random stream of one value: the P words of an L-bit stream, MSB-first like the LFSR streams.
  * The element's random words are Philox outputs with counter (block, index_lo, index_hi, tag)
  * and key (seed_lo, seed_hi); word j of the element is output j%4 of block j/4.
- *   generator 2 "rand": bit t = [code > r], r the (t % cpw)-th n_bits-wide field (from the least
- *     significant end) of word t / cpw, cpw = 32 / n_bits: independent Bernoulli(code / L) bits,
+ *   generator 2 "rand": bit t = [code > r], r = byte t % 4 (from the least significant end) of word
+ *     t / 4, reduced to its low n_bits bits: independent Bernoulli(code / L) bits,
  *     the distribution of code > curand() % L (sc_cuda_kernel.cu:459-462, :1329-1330).
  *   generator 1 "acc": bit t = [r16 * left_total < left_ones * 65536], r16 the (t % 2)-th 16-bit
  *     half of word t / 2, then left_ones -= bit, left_total -= 1: sampling without replacement,
@@ -456,8 +456,9 @@ void sco_random_stream_words(int code, int L, int generator, uint32_t tag, uint6
     uint32_t ctr[4] = {0, (uint32_t)index, (uint32_t)(index >> 32), tag};
     uint32_t r[4] = {0, 0, 0, 0};
     int have_block = -1;
-    int cpw = generator == 2 ? 32 / n_bits : 2;
+    int cpw = generator == 2 ? 4 : 2;
     int left_ones = code, left_total = L;
+    (void)n_bits;
     for (int p = 0; p < P; p++) {
         uint32_t word = 0;
         for (int b = 0; b < bit_unit; b++) {
@@ -471,7 +472,7 @@ void sco_random_stream_words(int code, int L, int generator, uint32_t tag, uint6
             uint32_t rw = r[j % 4];
             uint32_t bit;
             if (generator == 2) {
-                bit = (uint32_t)code > ((rw >> (f * n_bits)) & (uint32_t)(L - 1));
+                bit = (uint32_t)code > ((rw >> (8 * f)) & (uint32_t)(L - 1));
             } else {
                 uint32_t r16 = (rw >> (16 * f)) & 0xffffu;
                 bit = r16 * (uint32_t)left_total < (uint32_t)left_ones * 65536u;
