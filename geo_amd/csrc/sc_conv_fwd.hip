@@ -602,7 +602,6 @@ __global__ __launch_bounds__(64 * NWV) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
     const unsigned ch_stride = (unsigned)q.wi * q.hi;
     const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
-    const int k_or = q.c_in * WK;
     const int chunks_per_pass = q.c_in / CH;
     const int passes = q.packs * q.h_k;
     const int total = passes * chunks_per_pass;

@@ -397,7 +397,7 @@ __device__ __forceinline__ void random_stream(const RandParams& rp, int code, ui
                 for (int f = 0; f < 2; f++) {
                     const uint32_t field = f == 0 ? (r[w] & 0xffffu) : (r[w] >> 16);
                     // both factors are below 2^24
-                    const uint32_t bit = __umul24(field, left_total) < (left_ones << 16);
+                    const uint32_t bit = (uint32_t)__umul24(field, left_total) < (left_ones << 16);
                     left_ones -= bit;
                     left_total -= 1u;
                     word = word * 2u + bit;
