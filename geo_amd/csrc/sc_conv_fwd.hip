@@ -605,8 +605,11 @@ __global__ __launch_bounds__(64 * NWV * NPT) __attribute__((amdgpu_waves_per_eu(
     const unsigned ch_stride = (unsigned)q.wi * q.hi;
     const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
     const int chunks_per_pass = q.c_in / CH;
-    const int passes = q.packs * q.h_k;
-    const int total = passes * chunks_per_pass;
+    // this launch row's share of the (pack, kernel row) passes; with more than one row the partial sums
+    // are added to the zeroed y with integer atomics
+    const int pass_begin = blockIdx.y * q.pv_per_block;
+    const int passes = min(q.packs * q.h_k, pass_begin + q.pv_per_block);
+    const int total = (passes - pass_begin) * chunks_per_pass;
 
     int sum[2 * C];  // [2 c + r]
 #pragma unroll
@@ -628,14 +631,14 @@ __global__ __launch_bounds__(64 * NWV * NPT) __attribute__((amdgpu_waves_per_eu(
         for (int i = 0; i < CPW; i++) stage_all[buf][pt][wave + NWV * i][lane] = fetched[i];
     };
 
-    const size_t line0 = (size_t)cot * q.rail_lines;
+    const size_t line0 = (size_t)cot * q.rail_lines + (size_t)pass_begin * q.c_in * WK;
     const uint32_t* wp = q.wgt_rail + line0 * C;
     const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
-    fetch(0, 0);
+    fetch(pass_begin, 0);
     commit(0);
     __syncthreads();
     int tc = 0;
-    for (int pass = 0; pass < passes; pass++) {
+    for (int pass = pass_begin; pass < passes; pass++) {
         u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
         for (int cc = 0; cc < chunks_per_pass; cc++, tc++) {
             const int buf = tc & 1;
@@ -678,8 +681,13 @@ __global__ __launch_bounds__(64 * NWV * NPT) __attribute__((amdgpu_waves_per_eu(
         if (co >= q.c_out) break;
         int32_t* yo = q.y + ((size_t)n * q.c_out + co) * out_plane + (size_t)a0 * q.ho + b;
 #pragma unroll
-        for (int r = 0; r < R; r++)
-            if (a0 + r < q.wo) yo[(size_t)r * q.ho] = sum[2 * c + r];
+        for (int r = 0; r < R; r++) {
+            if (a0 + r >= q.wo) continue;
+            if (gridDim.y == 1)
+                yo[(size_t)r * q.ho] = sum[2 * c + r];
+            else
+                atomicAdd(yo + (size_t)r * q.ho, sum[2 * c + r]);  // integer adds: order does not matter
+        }
     }
 }
 
@@ -931,9 +939,23 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     // atomics.  Measured on MI355X: 4096x4096 linear at batch 1024 7.05 -> 6.24 ms.
     const int pv = g.packs * g.add_outer * g.add_inner;
     int splits = 1;
+    // the LDS-staged kernel: y mode, 3-wide kernels, whole chunks of 8 channels, 4 or 8 c_out tiles
+    const bool lds = R == 2 && WK == 3 && !ROWS_IN_N && g.rail && g.mode == GEO_SC_ACC_Y &&
+                     g.c_in % kStageChannels == 0 && g.n_cotile % 4 == 0;
     if (waves < 4096) {
         splits = (int)((12288 + waves - 1) / waves);
         if (splits > pv) splits = pv;
+    } else if (lds) {
+        // Equal waves run in rounds of 4096 (four per SIMD): 3.06 rounds take the time of 4.  Splitting the
+        // passes 2-, 3- or 4-fold makes the rounds shorter and the last one fuller (C5: 12544 waves, 0.77 ->
+        // 0.94 of the rounded-up time); taken when it gains more than the atomics cost.
+        auto fill = [&](int sp) { const double r = (double)waves * sp / 4096.0; return r / (double)(long long)(r + 0.999999); };
+        double best = fill(1) * 1.08;
+        for (int sp = 2; sp <= 4; sp++)
+            if (pv % sp == 0 && fill(sp) > best) {
+                best = fill(sp);
+                splits = sp;
+            }
     }
     q.pv_per_block = (pv + splits - 1) / splits;
     splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
@@ -958,7 +980,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
             // two channels per trip for 1-wide kernels: with three, the six address pairs push the 32
             // sums out of the 128 registers
             constexpr int CR = WK == 1 ? 2 : 1;
-            if (plain && WK == 3 && g.c_in % kStageChannels == 0 && g.n_cotile % 4 == 0) {
+            if (lds && (plain || waves >= 4096)) {
                 // c_out tiles of one position tile share their activation words through LDS
                 const int nwv = g.n_cotile % 8 == 0 ? 8 : 4;
                 // With eight tiles, two position tiles share a workgroup (16 waves, the whole CU in step): their
@@ -966,7 +988,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
                 // (C3 1.38 -> 1.31 ms; with four tiles the common barrier costs more than that saves).
                 const int npt = nwv == 8 ? 2 : 1;
                 const long long tile_sets = (tiles + npt - 1) / npt;
-                const dim3 grid_lds((unsigned)(tile_sets * (g.n_cotile / nwv)));
+                const dim3 grid_lds((unsigned)(tile_sets * (g.n_cotile / nwv)), (unsigned)splits);
                 if (nwv == 8)
                     hipLaunchKernelGGL((k_conv_fwd_rail_lds<8, 2>), grid_lds, dim3(1024), 0, s, q);
                 else
