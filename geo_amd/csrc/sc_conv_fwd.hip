@@ -945,7 +945,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     if (waves < 4096) {
         splits = (int)((12288 + waves - 1) / waves);
         if (splits > pv) splits = pv;
-    } else if (lds) {
+    } else if (g.rail && !ROWS_IN_N) {
         // Equal waves run in rounds of 4096 (four per SIMD): 3.06 rounds take the time of 4.  Splitting the
         // passes 2-, 3- or 4-fold makes the rounds shorter and the last one fuller (C5: 12544 waves, 0.77 ->
         // 0.94 of the rounded-up time); taken when it gains more than the atomics cost.
