@@ -982,15 +982,17 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
             constexpr int CR = WK == 1 ? 2 : 1;
             if (lds && (plain || waves >= 4096)) {
                 // c_out tiles of one position tile share their activation words through LDS
-                const int nwv = g.n_cotile % 8 == 0 ? 8 : 4;
-                // With eight tiles, two position tiles share a workgroup (16 waves, the whole CU in step): their
-                // waves read the same weight lines at the same time, which the scalar cache then serves once
-                // (C3 1.38 -> 1.31 ms; with four tiles the common barrier costs more than that saves).
-                const int npt = nwv == 8 ? 2 : 1;
+                // Four c_out tiles per workgroup.  With eight tiles or more, four position tiles share the
+                // workgroup and its barrier (16 waves, the whole CU in step): the four waves of a c_out tile
+                // read the same weight lines at the same time, which the scalar cache then serves once
+                // (C3 1.38 -> 1.29 ms; 8 c_out tiles x 2 position tiles 1.31, 2 x 8 1.33).  With four tiles
+                // in all the common barrier costs more than that saves (C5).
+                const int nwv = 4;
+                const int npt = g.n_cotile % 8 == 0 ? 4 : 1;
                 const long long tile_sets = (tiles + npt - 1) / npt;
                 const dim3 grid_lds((unsigned)(tile_sets * (g.n_cotile / nwv)), (unsigned)splits);
-                if (nwv == 8)
-                    hipLaunchKernelGGL((k_conv_fwd_rail_lds<8, 2>), grid_lds, dim3(1024), 0, s, q);
+                if (npt == 4)
+                    hipLaunchKernelGGL((k_conv_fwd_rail_lds<4, 4>), grid_lds, dim3(1024), 0, s, q);
                 else
                     hipLaunchKernelGGL((k_conv_fwd_rail_lds<4, 1>), grid_lds, dim3(256), 0, s, q);
             } else if (plain)
