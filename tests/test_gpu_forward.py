@@ -316,8 +316,8 @@ def test_long_kernels_use_the_row_chunked_weight_generator(capi, so, sx, sw, pad
     ((128, 4, 32, 32), (65, 4, 3, 2), (1, 0), 8, (7, 8, 1, 1), "lfsr"),     # L = 8, even kernel extent in dim 3
     ((128, 3, 32, 32), (50, 3, 3, 3), (1, 1), 64, (7, 8, 1, 1), "acc"),     # random generators: same kernel
     # 3-wide kernels with c_in % 8 == 0 and 4 or 8 c_out tiles: activation words staged through LDS
-    ((128, 8, 33, 32), (50, 8, 3, 3), (1, 1), 32, (7, 8, 1, 1), "lfsr"),    # four waves per workgroup, odd row count, partial tile
-    ((73, 16, 30, 31), (113, 16, 3, 3), (1, 1), 64, (7, 2, 2, 2), "lfsr"),  # eight tiles, two packs, odd number of position tiles, the last one ragged
+    ((128, 8, 33, 32), (50, 8, 3, 3), (1, 1), 32, (7, 8, 1, 1), "lfsr"),    # four c_out tiles (one position tile per workgroup), odd row count, partial c_out tile
+    ((73, 16, 30, 31), (113, 16, 3, 3), (1, 1), 64, (7, 2, 2, 2), "lfsr"),  # eight c_out tiles, two packs, 531 position tiles (not a multiple of the four per workgroup), the last one ragged
     ((128, 8, 32, 32), (128, 8, 3, 2), (1, 0), 128, (7, 8, 1, 1), "lfsr"),  # two kernel rows, four packs
     ((144, 24, 32, 32), (64, 24, 3, 1), (0, 0), 16, (7, 8, 1, 1), "acc"),   # three chunks of channels per pass
 ])
