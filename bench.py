@@ -2,7 +2,7 @@
 """Benchmark of the SC convolution hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--length 128]
-                    [--no-cpu-baseline]
+                    [--no-cpu-baseline] [--no-configs]
 
 One step = one pass of the hot path over one batch of synthetic input that is already
 resident in HBM: float->code conversion, LFSR stream generation for weights and
@@ -14,7 +14,9 @@ duration (the backward does no bit-MACs, so the forward-only rate is reported ne
 The default workload is the configuration the headline metric is quoted on: SC conv2d
 128->128 3x3 at 16x16, batch 256, pad 1, stream length 128, activations U[0,1), weights
 U[-1,1) (with these distributions every OR rail saturates, so this input is for timing
-only; the kernels have no data-dependent early exit).
+only; the kernels have no data-dependent early exit).  After the headline the default run also times
+the other benchmark configurations (C3 at stream lengths 32 and 256, C5, C4, the C2 training step) and
+reports them under the key ``configs``.
 """
 from __future__ import annotations
 
@@ -47,6 +49,8 @@ def parse():
     ap.add_argument("--generator", default="lfsr", choices=["lfsr", "acc", "rand"])
     ap.add_argument("--pass", dest="passes", default="fwdbwd", choices=["fwd", "fwdbwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the other benchmark configurations that the default run times after the headline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="also launch one plain device copy of this many MiB (reads MIB, writes MIB): the known-size "
                          "kernel that hardware traffic counters are scaled by")
@@ -67,15 +71,16 @@ def time_events(fn, steps, warmup, torch):
     return [a.elapsed_time(b) for a, b in evs]
 
 
-def measured_traffic(workload, L):
-    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 counters
-    (profiles/traffic.json); None for a workload that has not been profiled."""
+def profiled_traffic(workload, L):
+    """(HBM bytes per launch, kernel name) of the dominant kernel from the rocprofv3 counter runs
+    summarised in profiles/traffic.json; (None, None) for a workload that has not been profiled.
+    Not measured in this run: hardware counters need the profiler around the process."""
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
             t = json.load(f).get(f"{workload}_L{L}")
     except OSError:
-        return None
-    return None if t is None else t["fetch_bytes"] + t["write_bytes"]
+        return None, None
+    return (None, None) if t is None else (t["fetch_bytes"] + t["write_bytes"], t["kernel"])
 
 
 def cpu_baseline(x, w, L, pad):
@@ -126,7 +131,7 @@ C2_LAYERS = [  # (name, x shape, w shape, pad) of CONV_tiny_add_partial at batch
 ]
 
 
-def bench_network_step(args, torch):
+def network_step_result(args, torch):
     """4-layer SC CNN training step (network.py:126-190 topology, utils_own.py:81-114 step):
     batch 256 synthetic 3x32x32 images U[0,1), 10 uniform random classes, stream length 64,
     LFSR generators, progressive loading load_unit=2 / load_wait=2 (the training script's
@@ -185,16 +190,17 @@ def bench_network_step(args, torch):
         k = time_events(lambda: capi.conv2d_add_partial_from_streams(act, wgt, d, out=out), args.steps, 2, torch)
         B = wl.bit_macs(sx, sw, pad, L)
         B_total += B
-        word_ops_total += 2 * B / 32
+        ops = min_word_ops(sx, sw, pad, L)
+        word_ops_total += ops
         k_total += sum(k) / len(k)
         layers[name] = {"fwd_ms": sum(f) / len(f), "bwd_ms": sum(b) / len(b), "conv_kernel_ms": sum(k) / len(k),
-                        "bit_macs": B, "valu_frac": (2 * B / 32) / (sum(k) / len(k) * 1e-3) / PEAK_VALU_WORD_OPS}
+                        "bit_macs": B, "valu_frac": ops / (sum(k) / len(k) * 1e-3) / PEAK_VALU_WORD_OPS}
     achieved = word_ops_total / (k_total * 1e-3)
     result = {
         "metric": f"SC bit-MACs/sec over one training step of the 4-layer SC CNN at stream len {L}",
         "value": B_total / (ms_per_step * 1e-3), "unit": "bit-MAC/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "u32 bit-packed streams, int32 accumulate; fp32 backward",
+        "vs_baseline": None, "dtype": DTYPE_FWD_BWD,
         "data": "synthetic (torch.manual_seed(0); images U[0,1), uniform random labels)",
         "config": {"workload": "C2: 4-layer SC CNN (3->32 k5 @32, 32->32 k5 @16, 32->64 k5 @8, 64->10 k4 @4), batch "
                                f"256, stream length {L}, load_unit 2 / load_wait 2, fwd+bwd+Adam step, fused "
@@ -202,11 +208,11 @@ def bench_network_step(args, torch):
                    "pass": "train step", "bit_macs_per_step": B_total},
         "module_chain_ms_per_step": ms_module_chain,
         "layers": layers,
-        "roofline": {"bound": "valu", "kernel": "k_conv_fwd, the four layers' launches together",
+        "roofline": {"bound": "valu", "kernel": "the four layers' convolution launches together",
                      "achieved": achieved / 1e12, "peak": PEAK_VALU_WORD_OPS / 1e12, "unit": "T word-op/s",
                      "frac": achieved / PEAK_VALU_WORD_OPS, "kernel_ms_sum": k_total, "traffic": None},
     }
-    print(json.dumps(result))
+    return result
 
 
 def bench_network_inference(args, torch):
@@ -281,6 +287,118 @@ def bench_network_inference(args, torch):
     }))
 
 
+DTYPE_FWD = "u32 bit-packed streams, int32 popcount accumulate"
+DTYPE_FWD_BWD = (DTYPE_FWD + " (forward); fp32 gradients: each fp32 product from bf16 MFMA products of a three-way "
+                 "operand split, fp32 accumulate (backward)")
+
+
+def min_word_ops(x_shape, w_shape, pad, L):
+    """32-bit VALU lane operations no kernel for this problem can do without: one and-or per (activation
+    word, weight) - a weight has a single non-zero rail (sc.cpp:301-304), so B/32 of them, not the 2*B/32
+    of a kernel that processes both rails - plus one popcount-add per (output, rail, add group, pack)."""
+    N, Cin, Wx, Hx = x_shape
+    Cout, _, W, H = w_shape
+    Wo, Ho = Wx + 2 * pad - W + 1, Hx + 2 * pad - H + 1
+    B = N * Cout * Wo * Ho * Cin * W * H * L
+    return B / 32 + 2 * N * Cout * Wo * Ho * H * ((L + 31) // 32)
+
+
+def measure_layer(torch, workload, L, steps, warmup, with_bwd=True, accumulate="y", z_unit=32, generator="lfsr"):
+    """Times one single-layer workload: whole step (wall clock around synchronised loops), forward and
+    backward with events, the convolution kernel alone on pre-generated streams, stream generation."""
+    from geo_amd import capi
+    from geo_amd import workloads as wl
+
+    sx, sw, pad, _, vx, vw = wl.SHAPES[workload]
+    x, w = wl.make_inputs(sx, sw, "prescribed", 0, vx, vw)
+    xd, wd = x.cuda(), w.cuda()
+    desc = capi.make_desc(xd.shape, wd.shape, L, (pad, pad), accumulate=accumulate, z_unit=z_unit,
+                          generator=generator, seed=1)
+    ws = torch.empty(capi.workspace_size(desc), dtype=torch.uint8, device="cuda")
+    out = torch.empty(capi.output_shape(desc), dtype=torch.int32, device="cuda")
+    gy = torch.randn(out.shape, generator=torch.Generator().manual_seed(1)).cuda()
+    ws_b = torch.empty(capi.backward_workspace_size(desc), dtype=torch.uint8, device="cuda") if with_bwd else None
+
+    def fwd():
+        capi.conv2d_add_partial_forward(xd, wd, L, (pad, pad), out=out, workspace=ws, desc=desc)
+
+    def bwd():
+        capi.conv2d_add_partial_backward(xd, wd, gy, L, (pad, pad), workspace=ws_b, desc=desc)
+
+    def step():
+        fwd()
+        if with_bwd:
+            bwd()
+
+    # whole step: barrier-free on one GPU, synchronise both sides of the timed region
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    m = {"x": x, "w": w, "pad": pad, "desc": desc, "out_shape": tuple(out.shape)}
+    m["ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+    m["fwd_ms"] = time_events(fwd, steps, 2, torch)
+    m["bwd_ms"] = time_events(bwd, steps, 2, torch) if with_bwd else None
+    # dominant kernel alone (AND/OR/popcount on pre-generated streams), events on its stream
+    act = capi.act_streams(xd, desc)
+    wgt = capi.weight_streams(wd, desc)
+    m["kernel_ms"] = time_events(lambda: capi.conv2d_add_partial_from_streams(act, wgt, desc, out=out), steps,
+                                 warmup, torch)
+    m["gen_ms"] = time_events(lambda: (capi.act_streams(xd, desc), capi.weight_streams(wd, desc)), min(steps, 10),
+                              2, torch)
+    m["rail"] = capi.skips_zero_rail(desc)
+    m["B"] = wl.bit_macs(xd.shape, wd.shape, pad, L)
+    m["min_word_ops"] = min_word_ops(xd.shape, wd.shape, pad, L)
+    N, Cin, _, _ = xd.shape
+    Cout, _, W, H = wd.shape
+    m["bwd_flops"] = 12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H
+    m["alg_bytes"] = 4 * (xd.numel() + wd.numel() + out.numel())
+    m["stream_bytes"] = 4 * (act.numel() + wgt.numel())
+    m["out_bytes"] = 4 * out.numel()
+    return m
+
+
+def avg(v):
+    return sum(v) / len(v)
+
+
+def config_summary(m):
+    """The per-configuration entry of the ``configs`` key."""
+    k = avg(m["kernel_ms"])
+    e = {"ms_per_step": m["ms_per_step"], "fwd_ms": avg(m["fwd_ms"]),
+         "bwd_ms": avg(m["bwd_ms"]) if m["bwd_ms"] else None, "kernel_ms": k,
+         "bit_macs_per_s": m["B"] / (m["ms_per_step"] * 1e-3),
+         "fwd_bit_macs_per_s": m["B"] / (avg(m["fwd_ms"]) * 1e-3),
+         "executed_frac": m["min_word_ops"] / (k * 1e-3) / PEAK_VALU_WORD_OPS,
+         "bwd_tflops": m["bwd_flops"] / (avg(m["bwd_ms"]) * 1e-3) / 1e12 if m["bwd_ms"] else None}
+    return e
+
+
+def other_configs(args, torch):
+    """The benchmark configurations besides the headline, timed the same way with fewer steps."""
+    steps, warmup = min(args.steps, 10), min(args.warmup, 3)
+    out = {}
+    for name, workload, L in (("C3_L32", "C3", 32), ("C3_L256", "C3", 256), ("C5_L256", "C5", 256),
+                              ("C4_L128", "C4", 128)):
+        m = measure_layer(torch, workload, L, steps, warmup)
+        out[name] = config_summary(m)
+        del m
+        torch.cuda.empty_cache()
+    net_args = argparse.Namespace(**vars(args))
+    net_args.steps, net_args.warmup, net_args.length = steps, warmup, 64
+    r = network_step_result(net_args, torch)
+    out["C2_L64_train_step"] = {
+        "ms_per_step": r["ms_per_step"], "module_chain_ms_per_step": r["module_chain_ms_per_step"],
+        "bit_macs_per_s": r["value"], "kernel_ms": r["roofline"]["kernel_ms_sum"],
+        "executed_frac": r["roofline"]["frac"],
+        "fwd_ms": sum(l["fwd_ms"] for l in r["layers"].values()),
+        "bwd_ms": sum(l["bwd_ms"] for l in r["layers"].values()), "bwd_tflops": None}
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -297,35 +415,14 @@ def main():
         if args.passes == "fwd":
             bench_network_inference(args, torch)
         else:
-            bench_network_step(args, torch)
+            print(json.dumps(network_step_result(args, torch)))
         return
     from geo_amd import capi
     from geo_amd import workloads as wl
 
-    sx, sw, pad, L0, vx, vw = wl.SHAPES[args.workload]
-    L = args.length or L0
-    x, w = wl.make_inputs(sx, sw, "prescribed", 0, vx, vw)
-    xd, wd = x.cuda(), w.cuda()
-    desc = capi.make_desc(xd.shape, wd.shape, L, (pad, pad), accumulate=args.accumulate, z_unit=args.z_unit,
-                          generator=args.generator, seed=1)
+    L = args.length or wl.SHAPES[args.workload][3]
     variant = args.accumulate != "y" or args.generator != "lfsr"
-    ws = torch.empty(capi.workspace_size(desc), dtype=torch.uint8, device="cuda")
-    out = torch.empty(capi.output_shape(desc), dtype=torch.int32, device="cuda")
-
     with_bwd = args.passes == "fwdbwd"
-    gy = torch.randn(out.shape, generator=torch.Generator().manual_seed(1)).cuda()
-    ws_b = torch.empty(capi.backward_workspace_size(desc), dtype=torch.uint8, device="cuda") if with_bwd else None
-
-    def fwd():
-        capi.conv2d_add_partial_forward(xd, wd, L, (pad, pad), out=out, workspace=ws, desc=desc)
-
-    def bwd():
-        capi.conv2d_add_partial_backward(xd, wd, gy, L, (pad, pad), workspace=ws_b, desc=desc)
-
-    def step():
-        fwd()
-        if with_bwd:
-            bwd()
 
     if args.copy_calibration:
         src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device="cuda").fill_(1)
@@ -333,45 +430,21 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
 
-    # whole step: barrier-free on one GPU, synchronise both sides of the timed region
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-
-    B = wl.bit_macs(xd.shape, wd.shape, pad, L)
+    m = measure_layer(torch, args.workload, L, args.steps, args.warmup, with_bwd, args.accumulate, args.z_unit,
+                      args.generator)
+    x, w, pad = m["x"], m["w"], m["pad"]
+    B = m["B"]
+    ms_per_step = m["ms_per_step"]
     value = B / (ms_per_step * 1e-3)
-
-    fwd_ms = time_events(fwd, args.steps, 2, torch)
-    fwd_avg = sum(fwd_ms) / len(fwd_ms)
-    bwd_avg = None
-    if with_bwd:
-        bwd_ms = time_events(bwd, args.steps, 2, torch)
-        bwd_avg = sum(bwd_ms) / len(bwd_ms)
-
-    # dominant kernel alone (AND/OR/popcount on pre-generated streams), HIP events on its stream
-    act = capi.act_streams(xd, desc)
-    wgt = capi.weight_streams(wd, desc)
-    k_ms = time_events(lambda: capi.conv2d_add_partial_from_streams(act, wgt, desc, out=out), args.steps,
-                       args.warmup, torch)
-    k_avg = sum(k_ms) / len(k_ms)
-    word_ops = 2 * B / 32
-    rail = capi.skips_zero_rail(desc)
-    executed_ops = word_ops / 2 if rail else word_ops
-    achieved = word_ops / (k_avg * 1e-3)
+    fwd_ms, bwd_ms, k_ms = m["fwd_ms"], m["bwd_ms"], m["kernel_ms"]
+    fwd_avg, k_avg = avg(fwd_ms), avg(k_ms)
+    bwd_avg = avg(bwd_ms) if with_bwd else None
+    rail = m["rail"]
+    ops = m["min_word_ops"]
+    achieved = ops / (k_avg * 1e-3)
+    issued = (B / 32 if rail else 2 * B / 32)
     probe_rate = capi.probe_and_or_rate()
-    traffic = None if variant else measured_traffic(args.workload, L)
-    gen_ms = time_events(lambda: (capi.act_streams(xd, desc), capi.weight_streams(wd, desc)), min(args.steps, 10),
-                         2, torch)
-    N, Cin, Wx, Hx = xd.shape
-    Cout, _, W, H = wd.shape
-    alg_bytes = 4 * (xd.numel() + wd.numel() + out.numel())
-    stream_bytes = 4 * (act.numel() + wgt.numel())
+    traffic, traffic_kernel = (None, None) if variant else profiled_traffic(args.workload, L)
 
     result = {
         "metric": "SC bit-MACs/sec over one layer step ("
@@ -385,7 +458,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u32 bit-packed streams, int32 accumulate",
+        "dtype": DTYPE_FWD_BWD if with_bwd else DTYPE_FWD,
         "data": "synthetic (torch.manual_seed(0); activations U[0,1), weights U[-1,1))",
         "config": {"workload": f"{args.workload}: SC conv2d {tuple(x.shape)} * {tuple(w.shape)} pad {pad}, "
                                f"stream length {L}, " + {
@@ -400,50 +473,58 @@ def main():
                      "bwd_min": min(bwd_ms) if with_bwd else None},
         "roofline": {
             "bound": "valu",
-            "kernel": ("k_conv_fwd_rail / k_conv_fwd_rail_lds (v_and_or_b32 on register-indexed accumulators: one "
-                       "rail per weight; the _lds form shares activation words between c_out tiles through LDS)"
-                       if rail else "k_conv_fwd (v_and_or_b32 / v_bcnt_u32_b32)"),
+            "kernel": ("the rail-skipping convolution kernel (v_and_or_b32 on register-indexed accumulators: one "
+                       "and-or per activation word and weight; k_conv_fwd_rail_lds where activation words are "
+                       "shared through LDS)" if rail else "k_conv_fwd (v_and_or_b32 / v_bcnt_u32_b32, both rails)"),
+            # work no kernel can avoid (one and-or per activation word and weight, plus the popcount-adds) per
+            # second of the kernel's average launch duration, against lanes x clock
             "achieved": achieved / 1e12,
             "peak": PEAK_VALU_WORD_OPS / 1e12,
             "unit": "T word-op/s",
             "frac": achieved / PEAK_VALU_WORD_OPS,
-            "measured_issue_rate": probe_rate / 1e12,
-            "frac_of_measured_issue_rate": achieved / probe_rate,
+            "min_word_ops": ops,
             "kernel_ms_avg": k_avg,
             "kernel_ms_min": min(k_ms),
-            "algorithmic_word_ops": word_ops,
-            # Instructions the kernel really issues.  A weight has at most one non-zero rail; the
-            # rail-skipping kernel processes only that one, i.e. half of the algorithmic (two-rail)
-            # count, which is how "achieved" can pass the peak.
-            "note": ("frac counts the algorithmic two-rail work (2*B/32 and-or word-ops) against the nominal VALU "
-                     "peak; the rail-skipping kernel issues one and-or per (activation word, weight) instead of "
-                     "two, so frac can pass 1: executed_* is what the hardware actually does") if rail else None,
-            "executed_word_ops": executed_ops,
-            "executed_rate": executed_ops / (k_avg * 1e-3) / 1e12,
-            "executed_frac": executed_ops / (k_avg * 1e-3) / PEAK_VALU_WORD_OPS,
-            "executed_frac_of_measured_issue_rate": executed_ops / (k_avg * 1e-3) / probe_rate,
-            "hbm_algorithmic_bytes": alg_bytes,
-            "hbm_stream_bytes_read_by_kernel": stream_bytes,
+            "measured_issue_rate": probe_rate / 1e12,
+            "frac_of_measured_issue_rate": achieved / probe_rate,
+            # and-or instructions this kernel issues (lane operations): B/32 when it skips the zero rail, else 2B/32
+            "issued_and_or_word_ops": issued,
+            # the same time priced with the two-rail count 2*B/32 that a kernel processing both rails would
+            # execute (can pass the peak; not a roofline fraction)
+            "two_rail_word_ops": 2 * B / 32,
+            "two_rail_equivalent_rate": 2 * B / 32 / (k_avg * 1e-3) / 1e12,
+            "hbm_algorithmic_bytes": m["alg_bytes"],
+            "hbm_stream_bytes_read_by_kernel": m["stream_bytes"],
             "traffic": traffic,
-            "hbm_frac_of_peak": (traffic if traffic else stream_bytes + 4 * out.numel()) / (k_avg * 1e-3)
+            "traffic_source": (f"static: profiles/traffic.json, rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of "
+                               f"{traffic_kernel}, scaled by a device copy of known size; not measured in this run")
+                              if traffic else None,
+            "hbm_frac_of_peak": (traffic if traffic else m["stream_bytes"] + m["out_bytes"]) / (k_avg * 1e-3)
                                 / PEAK_HBM_BYTES,
         },
-        "stages_ms": {"stream_generation": sum(gen_ms) / len(gen_ms), "conv_kernel": k_avg, "backward": bwd_avg},
-        "backward_flops": {"algorithmic": 12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H,
-                           "achieved_tflops": (12 * N * Cout * out.shape[2] * out.shape[3] * Cin * W * H
-                                               / (bwd_avg * 1e-3) / 1e12) if bwd_avg else None,
+        "stages_ms": {"stream_generation": avg(m["gen_ms"]), "conv_kernel": k_avg, "backward": bwd_avg},
+        "backward_flops": {"algorithmic": m["bwd_flops"],
+                           "achieved_tflops": (m["bwd_flops"] / (bwd_avg * 1e-3) / 1e12) if bwd_avg else None,
                            "peak_tflops_fp32_mfma": 157.3,
+                           "frac_of_bf16_mfma_peak_as_executed": (6 * m["bwd_flops"] / (bwd_avg * 1e-3) / 2.5e15)
+                                                                 if bwd_avg else None,
                            "note": "fp32 in and out; aligned operands form each fp32 product from six bf16 MFMA "
                                    "products of a three-way split (fp32 accumulation, error as an fp32 GEMM), so "
-                                   "the fp32 MFMA peak is a yardstick, not a bound"},
+                                   "the fp32 MFMA peak is a yardstick, not a bound; the bf16 fraction counts the six "
+                                   "products against 2.5 PFLOP/s"},
     }
     if not args.no_cpu_baseline and not variant:  # the compiled reference has the y / LFSR op only
         kind, cores, sec, note = cpu_baseline(x, w, L, pad)
         result["cpu_baseline"] = {
             "value": B / sec, "unit": "bit-MAC/s", "cores": cores, "kind": kind,
-            "sample": f"same workload, full batch, median of up to 5 runs after 1 warm-up ({sec:.3f} s/run); {note}",
-            "gpu_over_cpu": value / (B / sec),
+            "sample": f"same workload, forward only (the reference has no native backward), full batch, median of "
+                      f"up to 5 runs after 1 warm-up ({sec:.3f} s/run); {note}",
+            "gpu_forward_over_cpu_forward": (B / (fwd_avg * 1e-3)) / (B / sec),
         }
+    if not args.no_configs and not variant and args.workload == "C3" and L == 128 and with_bwd:
+        del m
+        torch.cuda.empty_cache()
+        result["configs"] = other_configs(args, torch)
     print(json.dumps(result))
 
 

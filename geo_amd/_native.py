@@ -40,7 +40,6 @@ C_API = {
     "geo_sc_weight_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
     "geo_sc_act_streams_q7": (ctypes.c_int, [_D, _P, _P, _P, _P]),
     "geo_sc_act_stream_words": (ctypes.c_int, [_D, _SZ]),
-    "geo_sc_probe_and_or_rate": (ctypes.c_int, [ctypes.c_int, _P, ctypes.c_size_t, ctypes.POINTER(ctypes.c_double), _P]),
     "geo_sc_conv2d_add_partial_backward_workspace_size": (ctypes.c_int, [_D, _SZ]),
     "geo_sc_conv2d_add_partial_backward": (ctypes.c_int, [_D, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_weight_stream_words": (ctypes.c_int, [_D, _SZ]),
@@ -53,9 +52,11 @@ C_API = {
     "geo_sc_conv2d_add_partial_forward_q7": (ctypes.c_int, [_D, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_quantize": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, _P]),
     "geo_sc_weight_streams_finish": (ctypes.c_int, [_D, _P, _P]),
+    "geo_sc_weight_streams_check": (ctypes.c_int, [_D, _P, _P]),
 }
 
 _lib = None
+_probe = None
 _modules = {}
 
 
@@ -77,6 +78,20 @@ def lib() -> ctypes.CDLL:
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+def probe_lib() -> ctypes.CDLL:
+    """libgeo_sc_probe.so: the benchmark's issue-rate probe (csrc/sc_probe.hip), not part of the C ABI."""
+    global _probe
+    if _probe is None:
+        path = os.path.join(LIBDIR, "libgeo_sc_probe.so")
+        if not os.path.isfile(path):
+            raise ImportError(f"{path} not found; {_BUILD_HINT}")
+        L = ctypes.CDLL(path)
+        L.geo_sc_probe_and_or_rate.restype = ctypes.c_int
+        L.geo_sc_probe_and_or_rate.argtypes = [ctypes.c_int, _P, ctypes.c_size_t, ctypes.POINTER(ctypes.c_double), _P]
+        _probe = L
+    return _probe
 
 
 def module(name: str):

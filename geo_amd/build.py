@@ -1,6 +1,7 @@
 """In-tree build of the native code: ``python -m geo_amd.build``.
 
 * ``geo_amd/lib/libgeo_sc.so``            - HIP kernels + C ABI (hipcc, gfx950 only)
+* ``geo_amd/lib/libgeo_sc_probe.so``      - the benchmark's instruction issue-rate probe
 * ``geo_amd/lib/sc_extension_cuda*.so``   - PyTorch module with the reference's GPU op names
 * ``geo_amd/lib/sc_extension*.so``        - PyTorch module with the reference's CPU op name
                                            (runs the same GPU kernels)
@@ -20,7 +21,8 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 INCLUDE = os.path.join(ROOT, "include")
 
-HIP_SOURCES = ["sc_streams.hip", "sc_conv_fwd.hip", "sc_conv_bwd.hip", "sc_probe.hip", "sc_epilogue.hip", "sc_api.hip"]
+HIP_SOURCES = ["sc_streams.hip", "sc_conv_fwd.hip", "sc_conv_bwd.hip", "sc_epilogue.hip", "sc_api.hip"]
+PROBE_SOURCE = "sc_probe.hip"   # the benchmark's issue-rate probe: a library of its own, outside the C ABI
 TORCH_MODULES = {"sc_extension_cuda": "sc_extension_cuda.cpp", "sc_extension": "sc_extension.cpp"}
 
 # gfx950 only; packed-FP32 instruction selection is switched off for every device pass
@@ -55,6 +57,8 @@ def build_hip_library() -> str:
         list(ex.map(lambda so: _run(["hipcc", *HIPCC_FLAGS, "-c", os.path.join(CSRC, so[0]), "-o", so[1]]),
                     zip(sources, objs)))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", lib_path()])
+    _run(["hipcc", *HIPCC_FLAGS, "-shared", os.path.join(CSRC, PROBE_SOURCE), "-o",
+          os.path.join(LIBDIR, "libgeo_sc_probe.so")])
     return lib_path()
 
 

@@ -266,6 +266,17 @@ def weight_streams_from_lines(lines, desc: ConvDesc, stream=None):
     return out
 
 
+def weight_streams_ok(wgt, desc: ConvDesc, stream=None) -> bool:
+    """geo_sc_weight_streams_check on a buffer view as weight_streams() / weight_streams_from_lines()
+    return it: False when a caller-written line has two non-zero rails for one channel.  Waits for the
+    stream."""
+    rc = _native.lib().geo_sc_weight_streams_check(ctypes.byref(desc), _ptr(wgt), _stream_ptr(stream))
+    if rc == 1:   # GEO_SC_ERR_INVALID_ARGUMENT: the flagged buffer (the descriptor was valid when the buffer was made)
+        return False
+    _check(rc, "geo_sc_weight_streams_check")
+    return True
+
+
 def skips_zero_rail(desc: ConvDesc) -> bool:
     """True when the forward of this geometry runs the kernel that processes only the non-zero rail
     of every weight (its weight stream buffer then carries the rail-packed copy)."""
@@ -326,7 +337,7 @@ def probe_and_or_rate(iters=20000, stream=None):
     ops = ctypes.c_double(0)
 
     def launch(n):
-        _check(_native.lib().geo_sc_probe_and_or_rate(n, _ptr(scratch), scratch.numel(), ctypes.byref(ops),
+        _check(_native.probe_lib().geo_sc_probe_and_or_rate(n, _ptr(scratch), scratch.numel(), ctypes.byref(ops),
                                                       _stream_ptr(stream)), "geo_sc_probe_and_or_rate")
     launch(200)
     torch.cuda.synchronize()

@@ -107,12 +107,13 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     g->rail = g->wgt_rail && !g->thin && (wo >= 2 || g->act_item_inner);
     const size_t lines = (size_t)g->packs * d->h_k * g->k_or;
     g->wgt_words = lines * g->n_cotile * 2 * kCoTile;
-    g->wgt_rail_off = g->wgt_rail_idx_off = 0;
+    g->wgt_rail_off = g->wgt_rail_idx_off = g->wgt_flag_off = 0;
     g->wgt_rail_lines = lines;
     if (g->wgt_rail) {
         g->wgt_rail_off = (g->wgt_words + 63) & ~(size_t)63;
         g->wgt_rail_idx_off = g->wgt_rail_off + lines * g->n_cotile * kCoTile;
-        g->wgt_words = g->wgt_rail_idx_off + lines * g->n_cotile * (kCoTile / 2);
+        g->wgt_flag_off = g->wgt_rail_idx_off + lines * g->n_cotile * (kCoTile / 2);
+        g->wgt_words = g->wgt_flag_off + 64;
     }
     g->off_tables = 0;
     g->off_wgt = align256(table_bytes(g->L));
@@ -257,6 +258,21 @@ int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams
     if (rc != GEO_SC_OK) return rc;
     if (!streams) return GEO_SC_ERR_INVALID_ARGUMENT;
     return launch_rail_pack(g, streams, (hipStream_t)stream, false);
+}
+
+int geo_sc_weight_streams_check(const geo_sc_conv_desc* desc, const uint32_t* streams, geo_sc_stream_t stream)
+{
+    Geometry g;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!streams) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (!g.wgt_rail) return GEO_SC_OK;  // no rail-packed copy: the two-rail kernels take any lines
+    uint32_t flag = 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (hipMemcpyAsync(&flag, streams + g.wgt_flag_off, sizeof(flag), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess)
+        return GEO_SC_ERR_LAUNCH;
+    return flag ? GEO_SC_ERR_INVALID_ARGUMENT : GEO_SC_OK;
 }
 
 int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const uint32_t* act_streams,

@@ -49,7 +49,10 @@ struct Geometry {
     // at wgt_rail_off kCoTile words per line (the non-zero rail's word), at wgt_rail_idx_off
     // kCoTile / 2 words per line (16 bits per channel: which rail), both ordered [n_cotile][line]
     // with wgt_rail_lines lines per tile.
-    size_t wgt_words, wgt_rail_off, wgt_rail_idx_off, wgt_rail_lines;
+    // Behind the rail-packed copy: wgt_flag_off, one word that the packing kernel sets when a caller's
+    // line carries two non-zero rails for one channel (which the rail-packed form cannot hold), then
+    // padding to 64 words.
+    size_t wgt_words, wgt_rail_off, wgt_rail_idx_off, wgt_rail_lines, wgt_flag_off;
     // Position-major launches with two output rows per lane run the rail-skipping kernels: per weight
     // at most one rail's stream is non-zero (codes of clamp(w, 0, .) and -clamp(w, ., 0)), and only
     // that rail is processed.  wgt_rail: the weight stream buffer carries the rail-packed copy (a

@@ -892,11 +892,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 // into M0: bits 7:0 the register offset of the channel's accumulators, 2 c for the positive rail
 // (and for zero weights), 32 + 2 c for the negative one, bits 15:12 the SRC2 and DST enables of
 // the VGPR index mode; stored [cot][line][8].  One thread per (line, tile).
+// `both` (one word, cleared by the launcher) is set when a channel of a line has two non-zero rails.
 __global__ __launch_bounds__(256) void k_rail_pack(const uint32_t* __restrict__ lines2, uint32_t* __restrict__ words,
-                                                   uint32_t* __restrict__ idx, size_t n_lines, int n_cotile)
+                                                   uint32_t* __restrict__ idx, size_t n_lines, int n_cotile,
+                                                   uint32_t* __restrict__ both)
 {
     constexpr int C = kCoTile;
     const size_t total = n_lines * n_cotile;
+    bool two_rails = false;
     for (size_t l = (size_t)blockIdx.x * 256 + threadIdx.x; l < total; l += (size_t)gridDim.x * 256) {
         const size_t cot = l % n_cotile, line = l / n_cotile;
         const size_t dst = cot * n_lines + line;
@@ -907,6 +910,7 @@ __global__ __launch_bounds__(256) void k_rail_pack(const uint32_t* __restrict__ 
 #pragma unroll
         for (int c = 0; c < C; c++) {
             const uint32_t wp = src[c], wn = src[C + c];
+            two_rails |= wp != 0u && wn != 0u;
             words[dst * C + c] = wp | wn;
             const uint32_t field = 0xC000u | ((wn != 0u ? 2u * C : 0u) + 2u * c);
             packed[c >> 1] |= field << (16 * (c & 1));
@@ -914,6 +918,7 @@ __global__ __launch_bounds__(256) void k_rail_pack(const uint32_t* __restrict__ 
 #pragma unroll
         for (int c2 = 0; c2 < C / 2; c2++) idx[dst * (C / 2) + c2] = packed[c2];
     }
+    if (two_rails) atomicOr(both, 1u);
 }
 
 __global__ __launch_bounds__(256) void k_zero_i32(int32_t* __restrict__ p, size_t n)
@@ -1012,11 +1017,13 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
 
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator)
 {
-    if (!g.wgt_rail || (from_generator && weight_rows_generator(g))) return GEO_SC_OK;
+    if (!g.wgt_rail) return GEO_SC_OK;
+    hipLaunchKernelGGL(k_zero_i32, dim3(1), dim3(256), 0, s, reinterpret_cast<int32_t*>(wgt + g.wgt_flag_off), (size_t)64);
+    if (from_generator && weight_rows_generator(g)) return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     const size_t lines = g.wgt_rail_lines;
     size_t blocks = (lines * g.n_cotile + 255) / 256;
     hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,
-                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines, g.n_cotile);
+                       wgt + g.wgt_rail_off, wgt + g.wgt_rail_idx_off, lines, g.n_cotile, wgt + g.wgt_flag_off);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

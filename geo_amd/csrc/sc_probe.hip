@@ -2,7 +2,12 @@
 // operand, 64 independent accumulators, four waves per SIMD) in a loop with no memory
 // traffic.  Timing it gives the rate the hardware sustains for that instruction, which is
 // what the convolution kernel's achieved rate should be read against besides the nominal
-// lanes x clock figure.
+// lanes x clock figure.  Built into a library of its own (libgeo_sc_probe.so) for the benchmark;
+// not part of the C ABI of libgeo_sc.so.
+//
+// geo_sc_probe_and_or_rate enqueues `iters` x 64 v_and_or_b32 per wave on 4 waves per SIMD of 256 CUs
+// and reports in *word_ops how many 32-bit lane operations that is; the caller times it.  scratch: at
+// least 128 + 4096*64*4 bytes of device memory (its first 128 bytes are read as operands).
 #include "sc_common.h"
 
 namespace geo_sc {
@@ -34,7 +39,7 @@ __global__ __launch_bounds__(64) void k_probe_and_or(const uint32_t* __restrict_
 
 }  // namespace geo_sc
 
-extern "C" int geo_sc_probe_and_or_rate(int iters, void* scratch, size_t scratch_bytes, double* word_ops,
+extern "C" GEO_SC_API int geo_sc_probe_and_or_rate(int iters, void* scratch, size_t scratch_bytes, double* word_ops,
                                         geo_sc_stream_t stream)
 {
     const int waves = 256 * 4 * 4;  // 256 CUs x 4 SIMDs x 4 waves

@@ -154,9 +154,9 @@ def main(argv=None):
         if va[1] > best:
             best = va[1]
             torch.save(net.state_dict(), save_file)
-            print(f"\\n Epoch: {epoch + 1}\\tTraining Prec {tr[1]:.3f} \\tBinary Prec {va[1]:.3f}")
+            print(f"\n Epoch: {epoch + 1}\tTraining Prec {tr[1]:.3f} \tBinary Prec {va[1]:.3f}")
         scheduler.step(va[0])
-    print("\\nTraining finished!")
+    print("\nTraining finished!")
     return dict(history=history, save_file=save_file)
 
 

@@ -258,15 +258,10 @@ def make_param_copies(model):
     return [p.detach().clone().float().requires_grad_(True) for p in model.parameters()]
 
 
-def train_step(model, inputs, target, criterion, optimizer, param_copy):
-    """One step of the reference's loop (utils_own.py:79-114): scaled loss, backward, restore
-    full-precision weights, hand gradients to the master copies, un-scale, optimiser step,
-    copy back, refresh ``weight_org`` clamped to [-1, 0.999].  Returns the unscaled loss."""
-    output = model(inputs)
-    loss = criterion(output, target) * SCALE_FACTOR
-    for p in model.parameters():
-        p.grad = None
-    loss.backward()
+def apply_update(model, optimizer, param_copy):
+    """The part of the reference's step that follows ``loss.backward()`` (utils_own.py:98-114): restore
+    the full-precision weights, hand the gradients to the master copies and un-scale them, optimiser
+    step on the copies, copy back, refresh ``weight_org`` clamped to [-1, 0.999]."""
     for m in model.modules():
         if hasattr(m, "weight_org"):
             m.weight.data.copy_(m.weight_org)
@@ -286,4 +281,15 @@ def train_step(model, inputs, target, criterion, optimizer, param_copy):
         if hasattr(m, "weight_org"):
             m.weight_org.copy_(m.weight.data.clamp(-1, 0.999))
     optimizer.zero_grad()
+
+
+def train_step(model, inputs, target, criterion, optimizer, param_copy):
+    """One step of the reference's loop (utils_own.py:79-114): scaled loss, backward, then
+    ``apply_update``.  Returns the unscaled loss."""
+    output = model(inputs)
+    loss = criterion(output, target) * SCALE_FACTOR
+    for p in model.parameters():
+        p.grad = None
+    loss.backward()
+    apply_update(model, optimizer, param_copy)
     return loss.detach() / SCALE_FACTOR

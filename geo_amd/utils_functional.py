@@ -14,7 +14,6 @@ reference overwrites its value with the SC result anyway (utils_functional.py:63
 from __future__ import annotations
 
 import torch
-import torch.nn.functional as F
 
 from . import capi
 
@@ -40,53 +39,6 @@ def quantize_shift(tensor, scale=None, scale_only=False):
         scale = 2 ** torch.ceil(torch.log2(torch.mean(tensor) * 3))
     q = ((tensor / scale) * 128).round().clamp(-127, 127) / 128
     return q * scale, scale
-
-
-def conv2d_or_bin_1d(activation, w_pos, w_neg, padding, stride):
-    """The surrogate itself, in plain torch (utils_functional.py:235-252): one W x 1
-    convolution per kernel row and rail, 1 - exp(-z), summed over rows.  Kept as the
-    executable definition of what the HIP backward differentiates; the layer does not
-    call it."""
-    i_y = activation.size(3)
-    f_y = w_pos.size(3)
-    pos, neg = [], []
-    for j in range(f_y):
-        a_sec = activation[..., j:i_y - f_y + j + 1]
-        pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[..., j:j + 1], stride=stride)))
-        neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[..., j:j + 1], stride=stride)))
-    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
-
-
-def conv2d_or_approx(activation, weight, padding, stride):
-    """Surrogate of full OR accumulation (utils_functional.py:189-210, its default branch)."""
-    return 1 - torch.exp(-F.conv2d(activation, weight, padding=padding, stride=stride))
-
-
-def conv2d_or_bin_z(activation, w_pos, w_neg, padding, stride):
-    """Surrogate of z-dimension accumulation (utils_functional.py:254-270): one single-channel
-    convolution per input channel and rail, 1 - exp(-z), summed over channels."""
-    pos, neg = [], []
-    for c in range(activation.size(1)):
-        a_sec = activation[:, c:c + 1]
-        pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[:, c:c + 1], stride=stride)))
-        neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[:, c:c + 1], stride=stride)))
-    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
-
-
-def conv2d_or_bin_yz(activation, w_pos, w_neg, padding, stride, z_unit):
-    """Surrogate of yz accumulation (utils_functional.py:272-299): one W x 1 convolution per
-    block of ``z_unit`` input channels, kernel row and rail, 1 - exp(-z), summed."""
-    c_in = activation.size(1)
-    i_y = activation.size(3)
-    f_y = w_pos.size(3)
-    pos, neg = [], []
-    for c in range(0, c_in, z_unit):
-        c_end = min(c + z_unit, c_in)
-        for j in range(f_y):
-            a_sec = activation[:, c:c_end, :, j:i_y - f_y + j + 1]
-            pos.append(1 - torch.exp(-F.conv2d(a_sec, w_pos[:, c:c_end, :, j:j + 1], stride=stride)))
-            neg.append(1 - torch.exp(-F.conv2d(a_sec, w_neg[:, c:c_end, :, j:j + 1], stride=stride)))
-    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
 
 
 class _SCConv2dAddPartial(torch.autograd.Function):
@@ -207,24 +159,3 @@ def sc_counts(activation, weight, bit_length, padding, forward="1d_bin", load_un
     if activation.dtype == torch.uint8:
         return capi.conv2d_add_partial_forward_q7(activation.contiguous(), w, int(bit_length), pad, **kw)
     return capi.conv2d_add_partial_forward(activation.detach().float().contiguous(), w, int(bit_length), pad, **kw)
-
-
-def smoke_layer_step():
-    """One SC layer forward + backward on cuda:0 against the torch surrogate (used by the
-    smoke check)."""
-    from . import workloads as wl
-
-    x, w = wl.make_inputs((2, 4, 8, 8), (6, 4, 3, 3), "q7", seed=3)
-    x = x.cuda().requires_grad_(True)
-    w = (w * 4).cuda().requires_grad_(True)
-    y = conv2d_generic(x, w, (1, 1), (1, 1), bit_length=64, forward="1d_bin", generator="lfsr")
-    g = torch.linspace(-1, 1, y.numel(), device="cuda").reshape(y.shape)
-    y.backward(g)
-    xr = x.detach().double().requires_grad_(True)
-    wr = w.detach().double().requires_grad_(True)
-    xp = F.pad(xr, (1, 1, 1, 1))
-    p, n = conv2d_or_bin_1d(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)), (0, 0), (1, 1))
-    (p - n).backward(g.double())
-    for got, ref in ((x.grad, xr.grad), (w.grad, wr.grad)):
-        err = (got.double() - ref).abs().max().item()
-        assert err <= 1e-5 * ref.abs().max().item(), err

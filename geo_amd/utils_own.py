@@ -9,7 +9,7 @@ import time
 import torch
 import torch.nn as nn
 
-# loss scale (utils_own.py:14)
+# loss scale (utils_own.py:14); the step itself reads network.SCALE_FACTOR
 scale_factor = 128.0
 
 
@@ -38,73 +38,73 @@ def accuracy(output, target, topk=(1,)):
     return [correct[:k].reshape(-1).float().sum(0).mul_(100.0 / batch) for k in topk]
 
 
-def set_grad(params, params_with_grad):
-    """Hand the model's gradients to the master copies (utils_own.py:19-24)."""
-    for param, src in zip(params, params_with_grad):
-        if param.grad is None:
-            param.grad = torch.zeros_like(param.data)
-        if src.grad is not None:
-            param.grad.data.copy_(src.grad.data)
+class _Progress:
+    """Meters of one pass and the two line formats the loops print."""
+
+    def __init__(self):
+        self.loss, self.top1, self.top5, self.seconds = AverageMeter(), AverageMeter(), AverageMeter(), AverageMeter()
+        self._tick = time.time()
+
+    def record(self, loss, output, target, samples):
+        p1, p5 = accuracy(output, target, topk=(1, 5))
+        self.loss.update(float(loss), samples)
+        self.top1.update(p1.item(), samples)
+        self.top5.update(p5.item(), samples)
+        now = time.time()
+        self.seconds.update(now - self._tick)
+        self._tick = now
+
+    def batch_line(self, epoch, done, total):
+        cells = [f"Epoch: [{epoch}][{done}/{total}]",
+                 f"Time {self.seconds.val:.3f} ({self.seconds.avg:.6f})",
+                 f"Loss {self.loss.val:.4f} ({self.loss.avg:.4f})",
+                 f"Acc@1 {self.top1.val:.3f} ({self.top1.avg:.3f})",
+                 f"Acc@5 {self.top5.val:.3f} ({self.top5.avg:.3f})"]
+        return "\t".join(cells)
+
+    def epoch_line(self, epoch):
+        cells = [f"Epoch: [{epoch}]", f"Loss {self.loss.val:.4f} ({self.loss.avg:.4f})",
+                 f"Prec@1 {self.top1.val:.3f} ({self.top1.avg:.3f})", f"Prec@5 {self.top5.val:.3f} ({self.top5.avg:.3f})"]
+        return "\t".join(cells)
 
 
 def forward(data_loader, model, criterion, epoch=0, training=True, optimizer=None, verbal=False, iteration=None,
             param_copy=None, modules=None, use_target=False, monitor=False):
-    """One pass over ``data_loader`` (utils_own.py:31-140).  Training: loss * 128, backward,
-    restore the full-precision weights, gradients to the master copies and / 128, optimiser step,
-    copy back, ``weight_org = weight.clamp(-1, 0.999)``; the step is taken once at least 128
-    samples have been accumulated.  Returns (average scaled loss, prec@1, prec@5)."""
-    losses, top1, top5, batch_time = AverageMeter(), AverageMeter(), AverageMeter(), AverageMeter()
-    end = time.time()
-    acc = 0
-    if modules is None:
-        modules = model
-    ref = model.module.fc1.weight if isinstance(model, nn.DataParallel) else model.fc1.weight
-    for i, (inputs, target) in enumerate(data_loader):
-        if iteration is not None and i >= iteration:
+    """One pass over ``data_loader`` with the reference's call (utils_own.py:31-140).  Training runs
+    the step of ``network.apply_update`` (loss * 128, master copies, ``weight_org`` refresh) once at
+    least 128 samples have been seen since the last update, on the gradients of the batch that
+    completed them, as the reference does.  Returns (average scaled loss, prec@1, prec@5)."""
+    from . import network
+
+    net = model if modules is None else modules
+    anchor = (model.module if isinstance(model, nn.DataParallel) else model).fc1.weight
+    progress = _Progress()
+    since_update = 0
+    for done, (inputs, target) in enumerate(data_loader, start=1):
+        if iteration is not None and done > iteration:
             break
-        target = target.to(ref.device, non_blocking=True)
-        input_var = inputs.to(dtype=ref.dtype).to(ref.device, non_blocking=True)
-        output = model(input_var, target) if use_target else model(input_var)
-        loss = criterion(output, target) * scale_factor
-        prec1, prec5 = accuracy(output.data, target, topk=(1, 5))
-        losses.update(loss.item(), inputs.size(0))
-        top1.update(prec1.item(), inputs.size(0))
-        top5.update(prec5.item(), inputs.size(0))
-        acc += inputs.size(0)
+        target = target.to(anchor.device, non_blocking=True)
+        batch = inputs.to(anchor.device, anchor.dtype, non_blocking=True)
+        output = model(batch, target) if use_target else model(batch)
+        loss = criterion(output, target) * network.SCALE_FACTOR
         if training:
-            for param in modules.parameters():
-                param.grad = None
+            for p in net.parameters():
+                p.grad = None
             loss.backward()
-            if acc >= 128:
-                for p in modules.modules():
-                    if hasattr(p, "weight_org"):
-                        p.weight.data.copy_(p.weight_org)
-                set_grad(param_copy, list(modules.parameters()))
-                if scale_factor != 1:
-                    for param in param_copy:
-                        param.grad.data = param.grad.data / scale_factor
-                optimizer.step()
-                for dst, src in zip(modules.parameters(), param_copy):
-                    dst.data.copy_(src.data)
-                for p in modules.modules():
-                    if hasattr(p, "weight_org"):
-                        p.weight_org.copy_(p.weight.data.clamp(-1, 0.999))
-                optimizer.zero_grad()
-                acc = 0
-        batch_time.update(time.time() - end)
-        end = time.time()
+            since_update += inputs.size(0)
+            if since_update >= 128:
+                network.apply_update(net, optimizer, param_copy)
+                since_update = 0
+        progress.record(loss.item(), output.detach(), target, inputs.size(0))
         if monitor:
-            print(f"Epoch: [{epoch}][{i + 1}/{len(data_loader)}]\\tTime {batch_time.val:.3f} ({batch_time.avg:.6f})\\t"
-                  f"Loss {losses.val:.4f} ({losses.avg:.4f})\\tAcc@1 {top1.val:.3f} ({top1.avg:.3f})\\t"
-                  f"Acc@5 {top5.val:.3f} ({top5.avg:.3f})")
+            print(progress.batch_line(epoch, done, len(data_loader)))
     if training:
-        for p in model.modules():
-            if isinstance(p, (nn.Linear, nn.Conv2d)):
-                p.weight.data.clamp_(-1, 0.999)
+        for layer in model.modules():
+            if isinstance(layer, (nn.Linear, nn.Conv2d)):
+                layer.weight.data.clamp_(-1, 0.999)
     elif verbal:
-        print(f"Epoch: [{epoch}]\\tLoss {losses.val:.4f} ({losses.avg:.4f})\\tPrec@1 {top1.val:.3f} ({top1.avg:.3f})\\t"
-              f"Prec@5 {top5.val:.3f} ({top5.avg:.3f})")
-    return losses.avg, top1.avg, top5.avg
+        print(progress.epoch_line(epoch))
+    return progress.loss.avg, progress.top1.avg, progress.top5.avg
 
 
 def train(data_loader, model, criterion, epoch, optimizer, param_copy, iteration=None, modules=None, target=False,

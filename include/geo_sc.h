@@ -183,9 +183,16 @@ GEO_SC_API int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* de
  * For callers that write the two-rail weight lines themselves (layout above) into a buffer of
  * geo_sc_weight_stream_words words: fills the rest of the buffer (the rail-packed copy) from those
  * lines.  geo_sc_weight_streams does this itself.  Every (line, channel) must have at most one
- * non-zero rail, as streams of the reference's codes have.
+ * non-zero rail, as streams of the reference's codes have (sc.cpp:301-304); the rail-packed form
+ * cannot hold two.  A line that breaks the rule is recorded in the buffer (its last 64 words are a
+ * flag area) and reported by geo_sc_weight_streams_check, which waits for `stream` and returns
+ * GEO_SC_ERR_INVALID_ARGUMENT for such a buffer, GEO_SC_OK otherwise (also for buffers filled by
+ * geo_sc_weight_streams and for kernel widths that carry no rail-packed copy).  Counts computed from
+ * a buffer that fails the check are undefined.
  */
 GEO_SC_API int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams, geo_sc_stream_t stream);
+GEO_SC_API int geo_sc_weight_streams_check(const geo_sc_conv_desc* desc, const uint32_t* streams,
+                                           geo_sc_stream_t stream);
 /* Word counts of the two stream buffers above. */
 GEO_SC_API int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
 GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);
@@ -291,16 +298,6 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc
  * geo_sc_conv2d_add_partial_from_streams, then geo_sc_layer_epilogue per layer. */
 GEO_SC_API int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, uint32_t* streams,
                                      void* tables, geo_sc_stream_t stream);
-
-/*
- * Measurement aid, no counterpart in the reference: enqueues a loop of `iters` x 64
- * v_and_or_b32 instructions per wave (SGPR weight operand, no memory traffic) on 4 waves per
- * SIMD of 256 CUs and reports in *word_ops how many 32-bit lane operations that is; the
- * caller times it.  scratch: at least 128 + 4096*64*4 bytes of device memory (its first 128
- * bytes are read as operands, any content).
- */
-GEO_SC_API int geo_sc_probe_and_or_rate(int iters, void* scratch, size_t scratch_bytes, double* word_ops,
-                                        geo_sc_stream_t stream);
 
 #ifdef __cplusplus
 }

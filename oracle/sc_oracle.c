@@ -11,7 +11,7 @@
  *
  * Pinning status of each function (what, other than this file, fixes it):
  *   sco_lfsr_step        pinned  - known first states, period 2^n-1, all
- *                                  states visited (tests/test_oracle_lfsr.py)
+ *                                  states visited (tests/test_oracle.py)
  *   sco_codes_*          pinned  - closed form, exact in fp32; end-to-end
  *                                  golden outputs of the compiled reference
  *   sco_weight_streams   pinned  - popcount invariant + end-to-end goldens
@@ -19,11 +19,18 @@
  *   sco_conv_scalar/fast pinned  - SHA-256 of compiled sc.cpp outputs, the
  *                                  committed fixtures, an independent per-bit
  *                                  numpy formulation, oracle/_ref when built
- *   progressive loading (load_width < total_width+1)
- *                        PARITY PINNED BY SPEC TEXT ONLY: no CPU code in the
- *                        reference executes it; checked for neutrality at
- *                        load_width >= total_width+1 and for the width
- *                        sequence 1,3,3,5,5,7,7.. of (7,2,2).
+ *   sco_loaded_code (progressive loading, load_width < total_width+1)
+ *                        pinned  - no CPU code in the reference executes it, so
+ *                                  it is fixed by known answers worked out by
+ *                                  hand, cycle by cycle, from the CUDA source
+ *                                  text (tests/loading_vectors.py: 18 streams
+ *                                  over three (width, unit, wait) settings,
+ *                                  windows at cycles 1-8, 37-42, 77-82); the
+ *                                  mistakes "first cycle counted as 0",
+ *                                  "rounded-up division by the wait" and "no
+ *                                  growth before the first wait has passed" each
+ *                                  fail them; plus neutrality at
+ *                                  load_width >= total_width+1
  *   sco_conv2d_modes, mode yz
  *                        pinned  - equals the sum over channel blocks of the
  *                                  pinned y-mode path on the blocks, for every

@@ -40,6 +40,18 @@ def _groups(act, w_pos, w_neg, mode, z_unit):
             yield act[..., j:i_y - f_y + j + 1].clone(), w_pos[..., j:j + 1].clone(), w_neg[..., j:j + 1].clone()
 
 
+def surrogate_rails(act, w_pos, w_neg, mode="y", z_unit=1):
+    """(positive rail, negative rail) of the surrogate on an already padded activation, as torch
+    tensors that carry the autograd graph: per add group one convolution per rail, 1 - exp(-z),
+    stacked and summed (conv2d_or_bin_1d utils_functional.py:235-252, conv2d_or_bin_z :254-270,
+    conv2d_or_bin_yz :272-299, conv2d_or_approx :189-210 for mode "full").  Any dtype / device."""
+    pos, neg = [], []
+    for a_sec, wp_sec, wn_sec in _groups(act, w_pos, w_neg, mode, z_unit):
+        pos.append(1 - torch.exp(-F.conv2d(a_sec, wp_sec)))
+        neg.append(1 - torch.exp(-F.conv2d(a_sec, wn_sec)))
+    return torch.stack(pos, 0).sum(0), torch.stack(neg, 0).sum(0)
+
+
 def surrogate_autograd(x, w, grad_out, padding=(0, 0), sc_value=None, dtype=torch.float64, mode="y", z_unit=1):
     """(grad_x, grad_w, surrogate_value) as torch tensors of ``dtype``.
 
@@ -53,12 +65,7 @@ def surrogate_autograd(x, w, grad_out, padding=(0, 0), sc_value=None, dtype=torc
     act = F.pad(x, (padding[0], padding[0], padding[1], padding[1]))
     w_pos = w.clamp(0, 100)
     w_neg = -(w.clamp(-100, 0))
-    pos, neg = [], []
-    for a_sec, wp_sec, wn_sec in _groups(act, w_pos, w_neg, mode, z_unit):
-        pos.append(1 - torch.exp(-F.conv2d(a_sec, wp_sec)))
-        neg.append(1 - torch.exp(-F.conv2d(a_sec, wn_sec)))
-    pos_v = torch.stack(pos, 0).sum(0)
-    neg_v = torch.stack(neg, 0).sum(0)
+    pos_v, neg_v = surrogate_rails(act, w_pos, w_neg, mode, z_unit)
     value = (pos_v - neg_v).detach().clone()
     if sc_value is not None:
         pos_v.data = torch.as_tensor(sc_value).to(dtype)

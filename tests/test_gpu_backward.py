@@ -91,7 +91,7 @@ def test_backward_through_the_gemm_kernels(capi, shape_x, shape_w, pad, scale):
 def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
     """128->128 3x3 at 16x16, batch 256: against torch's own fp32 autograd over the surrogate
     (the float64 oracle on the CPU would take minutes), plus linearity in grad_y."""
-    from geo_amd import utils_functional as uf
+    from oracle import surrogate
     x, w, pad, _ = wl.named("C3", "q7")
     w = (w * 8).contiguous()
     xd, wd = x.cuda(), w.cuda()
@@ -100,7 +100,7 @@ def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
     xr = xd.clone().double().requires_grad_(True)
     wr = wd.clone().double().requires_grad_(True)
     xp = torch.nn.functional.pad(xr, (pad, pad, pad, pad))
-    p, n = uf.conv2d_or_bin_1d(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)), (0, 0), (1, 1))
+    p, n = surrogate.surrogate_rails(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)))
     (p - n).backward(g.double())
     assert rel_err(gx, xr.grad) <= RTOL, rel_err(gx, xr.grad)
     assert rel_err(gw, wr.grad) <= RTOL, rel_err(gw, wr.grad)

@@ -108,6 +108,26 @@ def test_conv_kernel_alone_on_oracle_streams(capi, so):
     assert np.array_equal(y.cpu().numpy(), exp)
 
 
+def test_caller_written_lines_with_two_rails_are_reported(capi):
+    """The rail-packed copy holds one rail per (line, channel); geo_sc_weight_streams_finish records a
+    line that has two and geo_sc_weight_streams_check reports it."""
+    d = capi.make_desc((2, 4, 6, 6), (20, 4, 3, 3), 64, (1, 1))
+    lines = torch.zeros((2, 3, 12, 2, 2, 16), dtype=torch.int32)
+    lines[1, 2, 7, 1, 0, 3] = 0x00f0
+    lines[0, 0, 0, 0, 1, 0] = 0x0001
+    good = capi.weight_streams_from_lines(lines.cuda(), d)
+    assert capi.weight_streams_ok(good, d)
+    lines[1, 2, 7, 1, 1, 3] = 0x0100            # same line and channel, other rail
+    bad = capi.weight_streams_from_lines(lines.cuda(), d)
+    assert not capi.weight_streams_ok(bad, d)
+    _, w = wl.make_inputs((2, 4, 6, 6), (20, 4, 3, 3), "prescribed", seed=5)
+    assert capi.weight_streams_ok(capi.weight_streams(w.cuda(), d), d)   # generated buffers always pass
+    # a kernel width without rail-packed copy has nothing to break
+    d7 = capi.make_desc((1, 2, 9, 9), (3, 2, 7, 7), 16, (3, 3))
+    _, w7 = wl.make_inputs((1, 2, 9, 9), (3, 2, 7, 7), "prescribed", seed=5)
+    assert capi.weight_streams_ok(capi.weight_streams(w7.cuda(), d7), d7)
+
+
 # ------------------------------------------------------------------ forward: fixtures
 def test_forward_matches_reference_fixtures(capi, fixtures_small):
     for name, d in fixtures_small.items():
@@ -152,6 +172,41 @@ def test_forward_progressive_loading_matches_oracle(capi, so, loading, L):
     assert np.array_equal(got, exp)
     neutral = gpu_forward(capi, x, w, L, (1, 1))
     assert not np.array_equal(got, neutral) or L == 16
+
+
+def _window(words_msb_first, first, count):
+    """bits first .. first+count-1 (cycle numbers from 1) of a 128-cycle stream given as 4 uint32 words"""
+    bits = [(int(words_msb_first[c // 32]) >> (31 - c % 32)) & 1 for c in range(128)]
+    return bits[first - 1:first - 1 + count]
+
+
+def test_progressive_loading_literal_known_answers(capi):
+    """The hand-derived bits of tests/loading_vectors.py (from sc_cuda_kernel.cu:155-160, :681-685) on
+    the GPU generators.  Activation element 0 has seed 1; the positive rail of input channel 60 and the
+    negative rail of input channel 90 of a 1x1 kernel have seed 1 as well ((67 + 60) % 127 + 1,
+    (37 + 90) % 127 + 1)."""
+    from tests import loading_vectors as lv
+
+    L = 128
+    for (tw, lw, wait), first, table in lv.VECTORS:
+        codes = sorted(table)
+        # activations: one item per code, a single element each
+        x = torch.tensor(codes, dtype=torch.float32).view(-1, 1, 1, 1) / L
+        d = capi.make_desc(x.shape, (1, 1, 1, 1), L, (0, 0), tw, lw, 1, wait)
+        got = u32(capi.act_streams(x.cuda(), d)).reshape(len(codes), 4)
+        for i, code in enumerate(codes):
+            assert _window(got[i], first, len(table[code])) == table[code], ("act", (tw, lw, wait), first, code)
+        # weights: output channel i carries code i on the positive rail of channel 60 and on the
+        # negative rail of channel 90
+        w = torch.zeros((len(codes), 91, 1, 1))
+        w[:, 60, 0, 0] = torch.tensor(codes, dtype=torch.float32) / L
+        w[:, 90, 0, 0] = -torch.tensor(codes, dtype=torch.float32) / L
+        d = capi.make_desc((1, 91, 1, 1), w.shape, L, (0, 0), tw, lw, wait, 1)
+        lines = u32(capi.weight_streams(w.cuda(), d)).reshape(4, 1, 91, 1, 2, 16)   # [P][H][K][cot][rail][16]
+        for i, code in enumerate(codes):
+            assert _window(lines[:, 0, 60, 0, 0, i], first, len(table[code])) == table[code], ("w+", first, code)
+            assert _window(lines[:, 0, 90, 0, 1, i], first, len(table[code])) == table[code], ("w-", first, code)
+            assert not lines[:, 0, 60, 0, 1, i].any() and not lines[:, 0, 90, 0, 0, i].any()
 
 
 # ------------------------------------------------------------------ forward: full sizes

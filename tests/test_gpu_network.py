@@ -61,6 +61,7 @@ def test_network_gradients_match_autograd_over_the_torch_surrogate():
     utils_functional.py:611-634)."""
     import torch.nn.functional as F
     from geo_amd import capi, utils_functional as uf
+    from oracle import surrogate
     x, t = _batch(64, seed=1)
     crit = torch.nn.CrossEntropyLoss()
 
@@ -79,7 +80,7 @@ def test_network_gradients_match_autograd_over_the_torch_surrogate():
                                                  tuple(padding), 7, kw["load_unit"], kw["load_wait_w"],
                                                  kw["load_wait_w"])
         act = F.pad(activation, (padding[0], padding[0], padding[1], padding[1]))
-        pos, neg = uf.conv2d_or_bin_1d(act, weight.clamp(0, 100), -(weight.clamp(-100, 0)), (0, 0), stride)
+        pos, neg = surrogate.surrogate_rails(act, weight.clamp(0, 100), -(weight.clamp(-100, 0)))
         pos.data = counts.float() / L
         neg.data = torch.zeros_like(neg)
         return pos - neg

@@ -120,6 +120,24 @@ def test_progressive_loading_widths_and_neutrality():
     assert _unpack(words, L)[0] == (1 if 0b1000000 > s1 else 0)
 
 
+def test_progressive_loading_literal_known_answers():
+    """Hand-derived bits (tests/loading_vectors.py, worked out from sc_cuda_kernel.cu:155-160 cycle by cycle)
+    applied to the oracle's generator: fixes that the first cycle has cur_bit == 1, that the division
+    by load_wait is an integer division, and that the register advances before the comparison."""
+    from tests import loading_vectors as lv
+
+    s, states = 1, {}
+    for cycle in range(1, 83):
+        s = so.lfsr_step(7, s)
+        states[cycle] = s
+    assert {c: states[c] for c in lv.STATES_FROM_SEED_1} == lv.STATES_FROM_SEED_1
+    for (tw, lw, wait), first, table in lv.VECTORS:
+        for code, bits in table.items():
+            words, _ = so.stream_of(code, 1, 128, tw, lw, wait)
+            got = _unpack(words, 128)[first - 1:first - 1 + len(bits)]
+            assert got == bits, ((tw, lw, wait), first, code)
+
+
 def _unpack(words, L):
     unit = min(L, 32)
     return [(int(words[p]) >> (unit - 1 - b)) & 1 for p in range(len(words)) for b in range(unit)]
