@@ -40,6 +40,7 @@ C_API = {
     "geo_sc_weight_streams": (ctypes.c_int, [_D, _P, _P, _P, _P]),
     "geo_sc_act_streams_q7": (ctypes.c_int, [_D, _P, _P, _P, _P]),
     "geo_sc_act_stream_words": (ctypes.c_int, [_D, _SZ]),
+    "geo_sc_act_stream_layout": (ctypes.c_int, [_D, ctypes.POINTER(ctypes.c_int)]),
     "geo_sc_conv2d_add_partial_backward_workspace_size": (ctypes.c_int, [_D, _SZ]),
     "geo_sc_conv2d_add_partial_backward": (ctypes.c_int, [_D, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_weight_stream_words": (ctypes.c_int, [_D, _SZ]),

@@ -210,8 +210,10 @@ def _tables(bit_length, device):
 
 
 def act_streams(x, desc: ConvDesc, stream=None):
-    """int32-typed tensor of stream words [N][P][Cin][Wi][Hi] (reinterpret as uint32).  ``x`` is
-    fp32, or uint8 holding the 7-bit integers round(x * 128)."""
+    """int32-typed tensor of stream words (reinterpret as uint32), shaped as the library stores them:
+    (N, P, Cin, Wi, Hi), or (P, Cin, Wi, Hi, N) for the geometries whose streams are batch-item-innermost
+    (geo_sc_act_stream_layout: single-row outputs of 1/3/5-wide kernels with N >= 2).  ``x`` is fp32, or
+    uint8 holding the 7-bit integers round(x * 128)."""
     q7 = x.dtype == torch.uint8
     if q7:
         if not (x.is_cuda and x.is_contiguous()):
@@ -222,7 +224,10 @@ def act_streams(x, desc: ConvDesc, stream=None):
     _check(_native.lib().geo_sc_act_stream_words(ctypes.byref(desc), ctypes.byref(n)), "act words")
     packs = (desc.bit_length + 31) // 32
     wi, hi = desc.w_in + 2 * desc.pad_w, desc.h_in + 2 * desc.pad_h
-    out = torch.empty((desc.n, packs, desc.c_in, wi, hi), dtype=torch.int32, device=x.device)
+    inner = ctypes.c_int(0)
+    _check(_native.lib().geo_sc_act_stream_layout(ctypes.byref(desc), ctypes.byref(inner)), "act layout")
+    shape = (packs, desc.c_in, wi, hi, desc.n) if inner.value else (desc.n, packs, desc.c_in, wi, hi)
+    out = torch.empty(shape, dtype=torch.int32, device=x.device)
     assert out.numel() == n.value
     tables = _tables(desc.bit_length, x.device)
     fn = _native.lib().geo_sc_act_streams_q7 if q7 else _native.lib().geo_sc_act_streams

@@ -200,6 +200,16 @@ int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words)
     return GEO_SC_OK;
 }
 
+int geo_sc_act_stream_layout(const geo_sc_conv_desc* desc, int* item_innermost)
+{
+    Geometry g;
+    if (!item_innermost) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    *item_innermost = g.act_item_inner ? 1 : 0;
+    return GEO_SC_OK;
+}
+
 int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words)
 {
     Geometry g;

@@ -193,8 +193,10 @@ GEO_SC_API int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* de
 GEO_SC_API int geo_sc_weight_streams_finish(const geo_sc_conv_desc* desc, uint32_t* streams, geo_sc_stream_t stream);
 GEO_SC_API int geo_sc_weight_streams_check(const geo_sc_conv_desc* desc, const uint32_t* streams,
                                            geo_sc_stream_t stream);
-/* Word counts of the two stream buffers above. */
+/* Word counts of the two stream buffers above; *item_innermost = 1 when the activation streams of `desc`
+ * are stored batch-item-innermost ([P][c_in][Wi][Hi][n]), 0 for [n][P][c_in][Wi][Hi]. */
 GEO_SC_API int geo_sc_act_stream_words(const geo_sc_conv_desc* desc, size_t* words);
+GEO_SC_API int geo_sc_act_stream_layout(const geo_sc_conv_desc* desc, int* item_innermost);
 GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* words);
 
 /*

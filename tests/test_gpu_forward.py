@@ -64,7 +64,8 @@ def test_activation_streams_item_innermost_layout(capi, so):
     L = 64
     x, _ = wl.make_inputs((5, 4, 3, 6), (2, 4, 3, 3), "prescribed", seed=77)
     d = capi.make_desc(x.shape, (2, 4, 3, 3), L, (0, 0))
-    got = u32(capi.act_streams(x.cuda(), d)).reshape(2, 4, 3, 6, 5)
+    got = u32(capi.act_streams(x.cuda(), d))
+    assert got.shape == (2, 4, 3, 6, 5)
     for n in range(5):
         assert np.array_equal(got[..., n], so.act_streams(x[n].numpy(), L))
 
@@ -193,7 +194,10 @@ def test_progressive_loading_literal_known_answers(capi):
         # activations: one item per code, a single element each
         x = torch.tensor(codes, dtype=torch.float32).view(-1, 1, 1, 1) / L
         d = capi.make_desc(x.shape, (1, 1, 1, 1), L, (0, 0), tw, lw, 1, wait)
-        got = u32(capi.act_streams(x.cuda(), d)).reshape(len(codes), 4)
+        # single-row output, several items: the words are stored batch-item-innermost, [P][1][1][1][N]
+        got = u32(capi.act_streams(x.cuda(), d))
+        assert got.shape == (4, 1, 1, 1, len(codes))
+        got = got.reshape(4, len(codes)).T
         for i, code in enumerate(codes):
             assert _window(got[i], first, len(table[code])) == table[code], ("act", (tw, lw, wait), first, code)
         # weights: output channel i carries code i on the positive rail of channel 60 and on the
