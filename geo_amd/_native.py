@@ -54,6 +54,7 @@ C_API = {
     "geo_sc_quantize": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, _P]),
     "geo_sc_weight_streams_finish": (ctypes.c_int, [_D, _P, _P]),
     "geo_sc_weight_streams_check": (ctypes.c_int, [_D, _P, _P]),
+    "geo_sc_conv2d_add_partial_forward_static": (ctypes.c_int, [_D, _P, _P, _P, _P]),
 }
 
 _lib = None

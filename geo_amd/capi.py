@@ -98,6 +98,23 @@ def conv2d_add_partial_forward(x, w, bit_length, padding=(0, 0), total_width=7, 
     return out
 
 
+STATIC_WORKSPACE_BYTES = 32 << 20   # GEO_SC_STATIC_WORKSPACE_BYTES of include/geo_sc.h
+
+
+def conv2d_add_partial_forward_static(x, w, out, desc: ConvDesc, stream=None):
+    """geo_sc_conv2d_add_partial_forward_static: the forward on the library's static device workspace;
+    allocates nothing (``out`` is the caller's int32 tensor of output_shape(desc))."""
+    _require_gpu_f32(x, "x")
+    _require_gpu_f32(w, "w")
+    if not (out.is_cuda and out.dtype == torch.int32 and out.is_contiguous()
+            and tuple(out.shape) == output_shape(desc)):
+        raise ValueError("out must be a contiguous int32 GPU tensor of the output's shape")
+    _check(_native.lib().geo_sc_conv2d_add_partial_forward_static(ctypes.byref(desc), _ptr(x), _ptr(w), _ptr(out),
+                                                                  _stream_ptr(stream)),
+           "geo_sc_conv2d_add_partial_forward_static")
+    return out
+
+
 def conv2d_add_partial_forward_q7(x_q7, w, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
                                   load_wait_a=1, out=None, workspace=None, stream=None, accumulate="y", z_unit=1):
     """The forward for activations given as uint8 integers k = round(x * 128), k <= 127

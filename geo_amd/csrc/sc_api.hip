@@ -1,6 +1,8 @@
 // C ABI of libgeo_sc.so: argument validation, workspace carve-up, kernel sequencing.
 #include "sc_common.h"
 
+#include <mutex>
+
 namespace geo_sc {
 
 namespace {
@@ -125,6 +127,30 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
 }  // namespace geo_sc
 
 using namespace geo_sc;
+
+// Workspace of geo_sc_conv2d_add_partial_forward_static.  In host code this name is only a handle
+// for hipGetSymbolAddress; kernels get the address that call returns.
+static __device__ __align__(256) unsigned char scratch[GEO_SC_STATIC_WORKSPACE_BYTES];
+
+namespace {
+// Device address of `scratch` on the current device (every GPU holds its own copy of the array at an
+// address of its own), looked up once per device; nullptr if the runtime refuses.
+void* static_workspace()
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* addr[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+        addr[dev] = p;
+    }
+    return addr[dev];
+}
+}  // namespace
 
 namespace {
 // x is fp32, or with Q7 the uint8 integers k of activations k / 128
@@ -299,6 +325,21 @@ int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float*
                                       void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
 {
     return forward_impl<false>(desc, x, w, y, workspace, workspace_bytes, stream);
+}
+
+int geo_sc_conv2d_add_partial_forward_static(const geo_sc_conv_desc* desc, const float* x, const float* w,
+                                             int32_t* y, geo_sc_stream_t stream)
+{
+    Geometry g;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (g.ws_bytes > GEO_SC_STATIC_WORKSPACE_BYTES) return GEO_SC_ERR_WORKSPACE;
+    void* ws = static_workspace();
+    if (!ws) return GEO_SC_ERR_LAUNCH;
+    // Every word the kernels read from the workspace is written by this call's own kernels first
+    // (tables, all weight lines including the channel padding, the flag area, every activation word),
+    // so nothing left by an earlier call needs clearing.
+    return forward_impl<false>(desc, x, w, y, ws, GEO_SC_STATIC_WORKSPACE_BYTES, stream);
 }
 
 int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, const float* w,

@@ -301,6 +301,20 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc
 GEO_SC_API int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, uint32_t* streams,
                                      void* tables, geo_sc_stream_t stream);
 
+/*
+ * geo_sc_conv2d_add_partial_forward for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and result, without the workspace: tables and both stream buffers live
+ * in a static device array of GEO_SC_STATIC_WORKSPACE_BYTES inside the library, which every GPU the
+ * library runs on holds until the process ends.  The call allocates and frees nothing and clears
+ * nothing with memset nodes.  A problem whose geo_sc_conv2d_add_partial_workspace_size exceeds the
+ * limit returns GEO_SC_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls that overlap
+ * on one GPU (different streams, different threads) race; calls on one stream do not.
+ */
+#define GEO_SC_STATIC_WORKSPACE_BYTES ((size_t)32 << 20)
+GEO_SC_API int geo_sc_conv2d_add_partial_forward_static(const geo_sc_conv_desc* desc, const float* x, const float* w,
+                                                        int32_t* y, geo_sc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
