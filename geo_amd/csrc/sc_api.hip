@@ -101,7 +101,7 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
         g->thin = pos_waves < 2048 && members >= 64;
     }
     g->act_item_inner = !g->thin && g->mode == GEO_SC_ACC_Y && g->generator == GEO_SC_GEN_LFSR && wo == 1 && d->n >= 2 && (d->w_k == 1 || d->w_k == 3 || d->w_k == 5) &&
-                        (unsigned long long)g->act_words < 0xffffffffull;
+                        (unsigned long long)g->act_words * 4 < 0xffffffffull;  // its kernel addresses the buffer with 32-bit byte offsets
     // Weight stream buffers of 1-, 3- and 5-wide kernels carry the rail-packed copy, whatever the
     // batch and input size (a buffer serves every geometry of the same weights); the launches with two
     // output rows (or, item-innermost, two batch items) per lane read it: the rail-skipping kernels.

@@ -38,6 +38,7 @@ struct FwdParams {
     int add_outer, add_inner, or_ch_total, or_ch_per_group;
     unsigned add_stride, or_stride;
     int or_rows;  // kernel rows OR-ed together before the popcount (1, or h_k for the full OR)
+    int keep_touches;  // always 0; k_conv_fwd_items_rail_wg: makes the values of its cache touches count as used
 };
 
 // acc |= a & w with w wave-uniform: a single v_and_or_b32 whose first source is the SGPR.
@@ -471,9 +472,50 @@ __device__ __forceinline__ void rail_line(u32x16& p0, u32x16& p1, u32x16& n0, u3
           [i3] "s"(ix[3]), [i4] "s"(ix[4]), [i5] "s"(ix[5]), [i6] "s"(ix[6]), [i7] "s"(ix[7]), [a0] "v"(a0), [a1] "v"(a1)
         : "m0", "scc");
 }
+// The first weight line of an OR group: assigns instead of accumulating, and clears the channel's other
+// rail (index ^ 32), so that the 64 accumulators need no zeroing pass.  v_and_b32 and v_mov_b32 are
+// two-operand instructions, which issue at twice the rate of v_and_or_b32: the line costs what an
+// accumulating line costs.
+#define GEO_SC_RAIL_FIRST(W, SET)                                                                                      \
+    SET "v_and_b32 v64, %[" W "], %[a0]\n"                                                                            \
+        "v_and_b32 v65, %[" W "], %[a1]\n"                                                                            \
+        "s_xor_b32 m0, m0, 32\n"                                                                                      \
+        "v_mov_b32 v64, 0\n"                                                                                          \
+        "v_mov_b32 v65, 0\n"
+__device__ __forceinline__ void rail_line_first(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1,
+                                                const uint32_t (&w)[kCoTile], const uint32_t (&ix)[kCoTile / 2],
+                                                uint32_t a0, uint32_t a1)
+{
+    asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n"
+        GEO_SC_RAIL_FIRST("w0", "") GEO_SC_RAIL_FIRST("w1", GEO_SC_RAIL_HI("i0"))
+        GEO_SC_RAIL_FIRST("w2", GEO_SC_RAIL_LO("i1")) GEO_SC_RAIL_FIRST("w3", GEO_SC_RAIL_HI("i1"))
+        GEO_SC_RAIL_FIRST("w4", GEO_SC_RAIL_LO("i2")) GEO_SC_RAIL_FIRST("w5", GEO_SC_RAIL_HI("i2"))
+        GEO_SC_RAIL_FIRST("w6", GEO_SC_RAIL_LO("i3")) GEO_SC_RAIL_FIRST("w7", GEO_SC_RAIL_HI("i3"))
+        GEO_SC_RAIL_FIRST("w8", GEO_SC_RAIL_LO("i4")) GEO_SC_RAIL_FIRST("w9", GEO_SC_RAIL_HI("i4"))
+        GEO_SC_RAIL_FIRST("w10", GEO_SC_RAIL_LO("i5")) GEO_SC_RAIL_FIRST("w11", GEO_SC_RAIL_HI("i5"))
+        GEO_SC_RAIL_FIRST("w12", GEO_SC_RAIL_LO("i6")) GEO_SC_RAIL_FIRST("w13", GEO_SC_RAIL_HI("i6"))
+        GEO_SC_RAIL_FIRST("w14", GEO_SC_RAIL_LO("i7")) GEO_SC_RAIL_FIRST("w15", GEO_SC_RAIL_HI("i7"))
+        "s_set_gpr_idx_off\n"
+        : "={v[64:79]}"(p0), "={v[80:95]}"(p1), "={v[96:111]}"(n0), "={v[112:127]}"(n1)
+        : [w0] "s"(w[0]), [w1] "s"(w[1]), [w2] "s"(w[2]), [w3] "s"(w[3]), [w4] "s"(w[4]), [w5] "s"(w[5]), [w6] "s"(w[6]),
+          [w7] "s"(w[7]), [w8] "s"(w[8]), [w9] "s"(w[9]), [w10] "s"(w[10]), [w11] "s"(w[11]), [w12] "s"(w[12]),
+          [w13] "s"(w[13]), [w14] "s"(w[14]), [w15] "s"(w[15]), [i0] "s"(ix[0]), [i1] "s"(ix[1]), [i2] "s"(ix[2]),
+          [i3] "s"(ix[3]), [i4] "s"(ix[4]), [i5] "s"(ix[5]), [i6] "s"(ix[6]), [i7] "s"(ix[7]), [a0] "v"(a0), [a1] "v"(a1)
+        : "m0", "scc");
+}
+#undef GEO_SC_RAIL_FIRST
 #undef GEO_SC_RAIL_PAIR
 #undef GEO_SC_RAIL_LO
 #undef GEO_SC_RAIL_HI
+
+// sum += popcount(pos) - popcount(neg) in three instructions (the compiler's form takes four)
+__device__ __forceinline__ void popc_diff(int& sum, uint32_t pos, uint32_t neg)
+{
+    uint32_t t;
+    asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(sum) : "v"(pos));
+    asm("v_bcnt_u32_b32 %0, %1, 0" : "=v"(t) : "v"(neg));
+    sum -= (int)t;
+}
 static_assert(kCoTile == 16, "rail_line is written for tiles of 16 output channels");
 
 // Two output rows per lane (R = 2), position-major activation streams, kernel extent WK in dim 2.
@@ -785,57 +827,82 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
 }
 
-// The rail-skipping kernel for item-innermost activation streams (outputs with a single row: the
-// SC-linear mapping).  A lane's two accumulator rows are the batch items n and n + row_groups;
-// consecutive lanes are consecutive items.  Activation addresses are a wave-uniform pointer plus one
-// 32-bit byte offset per lane and item; the kernel taps advance the uniform pointer.  Partial sums
-// over blockIdx.y's (pack, add group) range are added to the zeroed y with integer atomics.
-// CU: input channels per loop trip (their loads are issued together: 3 for 1-wide kernels, so that a
-// trip still holds 96 vector instructions behind one wait).
-template <int WK, int CU>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_items_rail(FwdParams q)
+// The rail-skipping kernel for item-innermost activation streams (y mode, outputs with a single row: the
+// SC-linear mapping, classifier layers) as a workgroup of S waves that share 128 items x 16 channels:
+// every wave sums a contiguous range of (pack, kernel row) groups, the partial sums meet in LDS
+// (ds_add_u32), and the workgroup stores the finished counts, channel fastest, so that the 16 channels of
+// an item leave as one 64-byte run when the output has a single position (y is then (N, Cout)).  No
+// zeroing pass over y, no global atomics.
+// Everything that moves between groups is scalar: the activation words are read with buffer loads
+// (resource over the whole stream buffer, per-lane byte offset of the lane's two items, the line's
+// offset as the scalar operand), the rail-packed weight lines of a c_out tile follow each other in the
+// order of the loop, so the two weight pointers only ever advance.
+// Weight lines are a stream without reuse inside a wave (the 4096 x 4096 layer: 403 MB for 256 c_out
+// tiles): every kTouchGroups groups the wave touches the lines of the groups after those with one vector
+// load per 128 bytes, so that the scalar loads that follow find them in L2.
+constexpr int kTouchGroups = 4;
+template <int WK, int CU, int S>
+__global__ __launch_bounds__(64 * S) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_items_rail_wg(FwdParams q)
 {
     constexpr int C = kCoTile, R = 2;
+    __shared__ int red[R * 64 * C];  // [r][lane][c]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int cot = blockIdx.x % q.n_cotile;
     const long long slot_first = (long long)(blockIdx.x / q.n_cotile) * 64;  // always a live slot
-    const long long slot0 = slot_first + threadIdx.x;
+    const long long slot0 = slot_first + lane;
     const bool live = slot0 < q.slots;
     const long long slot = live ? slot0 : slot_first;
     const int b = (int)(slot / q.row_groups);
     const long long n = slot % q.row_groups;
-    // lane offsets (bytes) of the two items; an item past the end is clamped to the first one: it
-    // only feeds an output that is never stored
+    // lane offsets (bytes) of the two items inside a line's words; an item past the end is clamped to
+    // the first one: it only feeds an output that is never stored
     unsigned loff[R];
 #pragma unroll
     for (int j = 0; j < R; j++)
         loff[j] = 4u * ((unsigned)b * q.n + (unsigned)n +
                         (n + (long long)j * q.row_groups < q.n ? (unsigned)j * q.row_groups : 0u));
-    const size_t pack_stride = (size_t)q.act_plane * q.n;
-    const unsigned tap_stride = (unsigned)q.hi * q.n;
-    const unsigned add_stride = (unsigned)q.n;
-    const unsigned or_stride = (unsigned)q.wi * q.hi * q.n;
+    // byte strides inside the stream buffer [P][c_in][wi][hi][n] (the launcher keeps it under 4 GB)
+    const unsigned pack_b = 4u * q.act_plane * (unsigned)q.n;
+    const unsigned tap_b = 4u * (unsigned)q.hi * q.n;
+    const unsigned row_b = 4u * (unsigned)q.n;
+    const unsigned ch_b = 4u * (unsigned)q.wi * q.hi * q.n;
+    const __amdgpu_buffer_rsrc_t act = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(q.act), 0,
+                                                                          (int)(pack_b * (unsigned)q.packs), 0x00020000);
 
     int sum[2 * C];  // [2 c + r]
 #pragma unroll
     for (int i = 0; i < 2 * C; i++) sum[i] = 0;
 
-    const int groups = q.add_outer * q.add_inner;
-    const int pv_begin = blockIdx.y * q.pv_per_block;
-    const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
-    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    const int k_or = q.c_in * WK;
+    const int pv_begin = wave * q.pv_per_block;
+    const int pv_end = min(q.packs * q.h_k, pv_begin + q.pv_per_block);
+    int v = pv_begin % q.h_k;
+    unsigned group_off = (unsigned)(pv_begin / q.h_k) * pack_b + (unsigned)v * row_b;
+    const size_t line0 = (size_t)cot * q.rail_lines + (size_t)pv_begin * k_or;
+    const uint32_t* wp = q.wgt_rail + line0 * C;
+    const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
+    // last words of this tile's rail-packed lines that a touch may read
+    const uint32_t* wp_last = q.wgt_rail + ((size_t)(cot + 1) * q.rail_lines) * C - 1;
+    const uint32_t* ip_last = q.wgt_rail_idx + ((size_t)(cot + 1) * q.rail_lines) * (C / 2) - 1;
+    uint32_t touched = 0, touch_acc = 0;
     for (int pv = pv_begin; pv < pv_end; pv++) {
-        const int p = pv / groups, g = pv - p * groups;
-        const int go = g / q.add_inner, gi = g - go * q.add_inner;
-        const int ch0 = go * q.or_ch_per_group;
-        const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
-        u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
-        const uint32_t* ap = q.act + (size_t)p * pack_stride + (size_t)gi * add_stride + (size_t)ch0 * or_stride;
-        const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
-                            (size_t)gi * chs * q.w_k;
-        const uint32_t* wp = q.wgt_rail + line * C;
-        const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
-        auto channels = [&](auto cu_tag) {
+        u32x16 p0, p1, n0, n1;  // written by the group's first line
+        bool first = true;
+        if (((pv - pv_begin) & (kTouchGroups - 1)) == 0) {
+            // the lines of groups pv + kTouchGroups .. pv + 2 kTouchGroups - 1: one lane per 128 bytes,
+            // first of the words, then of the fields
+            touch_acc ^= touched;  // the previous touch has long arrived: no wait in practice
+            const size_t ahead = (size_t)kTouchGroups * k_or;
+            const int w_lanes = kTouchGroups * k_or * C / 32;      // 128-byte pieces of the words
+            const uint32_t* tw = wp + ahead * C + lane * 32;
+            const uint32_t* ti = ip + ahead * (C / 2) + (lane - w_lanes) * 32;
+            const uint32_t* t = lane < w_lanes ? (tw < wp_last ? tw : wp_last) : (ti < ip_last ? ti : ip_last);
+            touched = *t;
+        }
+        unsigned ch_off = group_off;
+        auto channels_of = [&](auto cu_tag, auto first_tag) {
             constexpr int N = decltype(cu_tag)::value;
+            constexpr bool FIRST = decltype(first_tag)::value;
             uint32_t aw[N][WK][R];
 #pragma unroll
             for (int cu = 0; cu < N; cu++)
@@ -843,8 +910,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 for (int u = 0; u < WK; u++)
 #pragma unroll
                     for (int j = 0; j < R; j++)
-                        aw[cu][u][j] = *reinterpret_cast<const uint32_t*>(
-                            reinterpret_cast<const char*>(ap + (size_t)cu * or_stride + (size_t)u * tap_stride) + loff[j]);
+                        aw[cu][u][j] = __builtin_amdgcn_raw_buffer_load_b32(
+                            act, (int)loff[j], (int)(ch_off + (unsigned)cu * ch_b + (unsigned)u * tap_b), 0);
             uint32_t wv[N * WK][C], iv[N * WK][C / 2];
 #pragma unroll
             for (int l = 0; l < N * WK; l++) {
@@ -856,34 +923,240 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
             for (int cu = 0; cu < N; cu++)
 #pragma unroll
-                for (int u = 0; u < WK; u++)
-                    rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u][0], aw[cu][u][1]);
+                for (int u = 0; u < WK; u++) {
+                    if (FIRST && cu == 0 && u == 0)
+                        rail_line_first(p0, p1, n0, n1, wv[0], iv[0], aw[0][0][0], aw[0][0][1]);
+                    else
+                        rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u][0], aw[cu][u][1]);
+                }
             wp += N * WK * C;
             ip += N * WK * (C / 2);
-            ap += (size_t)N * or_stride;
+            ch_off += (unsigned)N * ch_b;
         };
-        int ci = 0;
-        for (; ci + CU <= chs; ci += CU) channels(std::integral_constant<int, CU>());
-        if constexpr (CU > 1)
-            for (; ci < chs; ci++) channels(std::integral_constant<int, 1>());
+        auto channels = [&](auto cu_tag) {
+            if (first)
+                channels_of(cu_tag, std::true_type());
+            else
+                channels_of(cu_tag, std::false_type());
+            first = false;
+        };
+        // trips of CU channels, the remainder in trips of two where that avoids a trip of one (16
+        // channels with CU = 3: 3 3 3 3 2 2)
+        int left = q.c_in;
+        if constexpr (CU > 2) {
+            while (left >= CU + 2 || left == CU) {
+                channels(std::integral_constant<int, CU>());
+                left -= CU;
+            }
+        }
+        if constexpr (CU > 1) {
+            for (; left >= 2; left -= 2) channels(std::integral_constant<int, 2>());
+        }
+        for (; left > 0; left--) channels(std::integral_constant<int, 1>());
 #pragma unroll
         for (int i = 0; i < C; i++) {
-            sum[i] += __popc(p0[i]) - __popc(n0[i]);
-            sum[C + i] += __popc(p1[i]) - __popc(n1[i]);
+            popc_diff(sum[i], p0[i], n0[i]);
+            popc_diff(sum[C + i], p1[i], n1[i]);
+        }
+        // next (pack, kernel row): one row further, or the first row of the next pack
+        group_off += row_b;
+        if (++v == q.h_k) {
+            v = 0;
+            group_off += pack_b - (unsigned)q.h_k * row_b;
         }
     }
+    // keeps the touches alive: the values read are never used (q.keep_touches is 0)
+    if (q.keep_touches && (touch_acc ^ touched) == 0x9e3779b9u) sum[0] += 1;
 
-    if (!live) return;
+    // partial sums of the S waves meet in LDS: wave 0 writes, the others add
+    if (wave == 0) {
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int r = 0; r < R; r++) red[(r * 64 + lane) * C + c] = sum[2 * c + r];
+    }
+    __syncthreads();
+    if (wave != 0 && pv_begin < pv_end) {
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int r = 0; r < R; r++) atomicAdd(&red[(r * 64 + lane) * C + c], sum[2 * c + r]);
+    }
+    __syncthreads();
     const size_t out_plane = (size_t)q.wo * q.ho;
-#pragma unroll
-    for (int c = 0; c < C; c++) {
+    for (int e = threadIdx.x; e < R * 64 * C; e += 64 * S) {
+        const int c = e % C, sl = (e / C) % 64, r = e / (C * 64);
+        const long long s_out = slot_first + sl;
         const int co = cot * C + c;
-        if (co >= q.c_out) break;
+        if (s_out >= q.slots || co >= q.c_out) continue;
+        const long long item = s_out % q.row_groups + (long long)r * q.row_groups;
+        if (item >= q.n) continue;
+        q.y[((size_t)item * q.c_out + co) * out_plane + (size_t)(s_out / q.row_groups)] = red[e];
+    }
+}
+
+// The item-innermost kernel for OR groups of LPG = 16 one-wide lines (the SC-linear mapping with groups of
+// 16 inputs), as one workgroup of 16 waves per (128 items, 8 c_out tiles): wave = (c_out tile, half of
+// the (pack, kernel row) groups).  The eight waves of a half read the same activation words; per group
+// every wave fetches two of the 16 lines (buffer loads, 4 dwords per lane) and leaves them in LDS, and
+// all read a line back with one ds_read_b64: an eighth of the vector loads, and what a wave waits for in
+// front of a line's 32 vector instructions is LDS and the scalar cache.  Groups are double-buffered
+// (the loads of group t + 1 are issued before group t is computed and written to LDS after it), one
+// barrier per group.  The two halves add their sums in LDS and the workgroup stores 128 items x 128
+// channels, 512-byte runs per item.  With 8 position tiles x 32 tile groups (4096 x 4096 at batch 1024)
+// that is 256 workgroups, one per CU, in a single round.
+// The 256 workgroups walk their weight streams in step (768 KB of lines per group and L2): a touch two
+// groups ahead is still in L2 when its lines are read (1 or 2 groups ahead 3.06 ms, 4: 3.19, 8: 4.43, none: 5.2).
+constexpr int kLinLines = 16, kLinTiles = 8, kLinHalves = 2, kLinTouchGroups = 2;
+__global__ __launch_bounds__(64 * kLinTiles * kLinHalves) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void k_conv_fwd_items_rail_lds(FwdParams q)
+{
+    constexpr int C = kCoTile, R = 2, LPG = kLinLines, NWV = kLinTiles, G = kLinHalves, LPW = LPG / NWV;
+    __shared__ uint2 stage[G][2][LPG][64];           // 32 KB
+    __shared__ int red[NWV][R * 64 * C];             // 64 KB
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int cw = wave_all % NWV, half = wave_all / NWV;
+    const int cot_groups = q.n_cotile / NWV;
+    const int cot = (blockIdx.x % cot_groups) * NWV + cw;
+    const long long slot_first = (long long)(blockIdx.x / cot_groups) * 64;  // always a live slot
+    const long long slot0 = slot_first + lane;
+    const long long slot = slot0 < q.slots ? slot0 : slot_first;
+    const int b = (int)(slot / q.row_groups);
+    const long long n = slot % q.row_groups;
+    unsigned loff[R];
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const long long item = n + (long long)r * q.row_groups;
-            if (item < q.n) atomicAdd(q.y + ((size_t)item * q.c_out + co) * out_plane + b, sum[2 * c + r]);
+    for (int j = 0; j < R; j++)
+        loff[j] = 4u * ((unsigned)b * q.n + (unsigned)n +
+                        (n + (long long)j * q.row_groups < q.n ? (unsigned)j * q.row_groups : 0u));
+    const unsigned pack_b = 4u * q.act_plane * (unsigned)q.n;
+    const unsigned row_b = 4u * (unsigned)q.n;
+    const unsigned ch_b = 4u * (unsigned)q.wi * q.hi * q.n;
+    const __amdgpu_buffer_rsrc_t act = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(q.act), 0,
+                                                                          (int)(pack_b * (unsigned)q.packs), 0x00020000);
+    int sum[2 * C];  // [2 c + r]
+#pragma unroll
+    for (int i = 0; i < 2 * C; i++) sum[i] = 0;
+
+    // this half's groups (the launcher makes the halves equal: every wave meets every barrier)
+    const int pv_begin = half * q.pv_per_block;
+    const int n_groups = q.pv_per_block;
+    int v = pv_begin % q.h_k;
+    unsigned group_off = (unsigned)(pv_begin / q.h_k) * pack_b + (unsigned)v * row_b;
+    const size_t line0 = (size_t)cot * q.rail_lines + (size_t)pv_begin * LPG;
+    const uint32_t* wp = q.wgt_rail + line0 * C;
+    const uint32_t* ip = q.wgt_rail_idx + line0 * (C / 2);
+    const uint32_t* wp_last = q.wgt_rail + ((size_t)(cot + 1) * q.rail_lines) * C - 1;
+    const uint32_t* ip_last = q.wgt_rail_idx + ((size_t)(cot + 1) * q.rail_lines) * (C / 2) - 1;
+    uint32_t touched = 0, touch_acc = 0;
+
+    // this wave's lines of a group: cw + NWV * i
+    uint2 fetched[LPW];
+    auto fetch = [&](unsigned goff) {
+#pragma unroll
+        for (int i = 0; i < LPW; i++) {
+            const unsigned so = goff + (unsigned)(cw + NWV * i) * ch_b;
+            fetched[i].x = __builtin_amdgcn_raw_buffer_load_b32(act, (int)loff[0], (int)so, 0);
+            fetched[i].y = __builtin_amdgcn_raw_buffer_load_b32(act, (int)loff[1], (int)so, 0);
         }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LPW; i++) stage[half][buf][cw + NWV * i][lane] = fetched[i];
+    };
+    auto next_group = [&]() {
+        group_off += row_b;
+        if (++v == q.h_k) {
+            v = 0;
+            group_off += pack_b - (unsigned)q.h_k * row_b;
+        }
+    };
+    fetch(group_off);
+    commit(0);
+    __syncthreads();
+    for (int t = 0; t < n_groups; t++) {
+        const int buf = t & 1;
+        const bool more = t + 1 < n_groups;
+        next_group();
+        if (more) fetch(group_off);
+        if ((t & (kLinTouchGroups - 1)) == 0) {
+            touch_acc ^= touched;
+            const size_t ahead = (size_t)kLinTouchGroups * LPG;
+            const int w_lanes = kLinTouchGroups * LPG * C / 32;
+            const uint32_t* tw = wp + ahead * C + lane * 32;
+            const uint32_t* ti = ip + ahead * (C / 2) + (lane - w_lanes) * 32;
+            const uint32_t* tp = lane < w_lanes ? (tw < wp_last ? tw : wp_last) : (ti < ip_last ? ti : ip_last);
+            touched = *tp;
+        }
+        u32x16 p0, p1, n0, n1;  // written by the group's first line
+        auto lines = [&](auto n_tag, auto first_tag, int l0) {
+            constexpr int N = decltype(n_tag)::value;
+            constexpr bool FIRST = decltype(first_tag)::value;
+            uint2 aw[N];
+#pragma unroll
+            for (int l = 0; l < N; l++) aw[l] = stage[half][buf][l0 + l][lane];
+            uint32_t wv[N][C], iv[N][C / 2];
+#pragma unroll
+            for (int l = 0; l < N; l++) {
+#pragma unroll
+                for (int c = 0; c < C; c++) wv[l][c] = wp[l * C + c];
+#pragma unroll
+                for (int c = 0; c < C / 2; c++) iv[l][c] = ip[l * (C / 2) + c];
+            }
+#pragma unroll
+            for (int l = 0; l < N; l++) {
+                if (FIRST && l == 0)
+                    rail_line_first(p0, p1, n0, n1, wv[0], iv[0], aw[0].x, aw[0].y);
+                else
+                    rail_line(p0, p1, n0, n1, wv[l], iv[l], aw[l].x, aw[l].y);
+            }
+            wp += N * C;
+            ip += N * (C / 2);
+        };
+        using T3 = std::integral_constant<int, 3>;
+        using T2 = std::integral_constant<int, 2>;
+        lines(T3(), std::true_type(), 0);
+        lines(T3(), std::false_type(), 3);
+        lines(T3(), std::false_type(), 6);
+        lines(T3(), std::false_type(), 9);
+        lines(T2(), std::false_type(), 12);
+        lines(T2(), std::false_type(), 14);
+        static_assert(LPG == 16, "the trips above cover 16 lines");
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            popc_diff(sum[i], p0[i], n0[i]);
+            popc_diff(sum[C + i], p1[i], n1[i]);
+        }
+        if (more) commit(buf ^ 1);
+        __syncthreads();
+    }
+    if (q.keep_touches && (touch_acc ^ touched) == 0x9e3779b9u) sum[0] += 1;
+
+    // the two halves of a c_out tile add their sums in LDS: half 0 writes, half 1 adds
+    if (half == 0) {
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int r = 0; r < R; r++) red[cw][(r * 64 + lane) * C + c] = sum[2 * c + r];
+    }
+    __syncthreads();
+    if (half != 0) {
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int r = 0; r < R; r++) atomicAdd(&red[cw][(r * 64 + lane) * C + c], sum[2 * c + r]);
+    }
+    __syncthreads();
+    // 128 items x (8 tiles x 16 channels): channel fastest across the tiles, 512-byte runs per item
+    const size_t out_plane = (size_t)q.wo * q.ho;
+    const int cot_first = (blockIdx.x % cot_groups) * NWV;
+    for (int e = threadIdx.x; e < NWV * R * 64 * C; e += 64 * NWV * G) {
+        const int c = e % C, tw = (e / C) % NWV, sl = (e / (C * NWV)) % 64, r = e / (C * NWV * 64);
+        const long long s_out = slot_first + sl;
+        const int co = (cot_first + tw) * C + c;
+        if (s_out >= q.slots || co >= q.c_out) continue;
+        const long long item = s_out % q.row_groups + (long long)r * q.row_groups;
+        if (item >= q.n) continue;
+        q.y[((size_t)item * q.c_out + co) * out_plane + (size_t)(s_out / q.row_groups)] = red[tw][(r * 64 + sl) * C + c];
     }
 }
 
@@ -964,12 +1237,27 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
     }
     q.pv_per_block = (pv + splits - 1) / splits;
     splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
-    // (item-innermost launches always go through the accumulating rail kernel)
     const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y && !ROWS_IN_N;
-    if (ROWS_IN_N) {
-        // its lane offsets are 32-bit byte offsets inside one pack of all items
-        if ((unsigned long long)g.act_plane * g.n * 4 >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
-        if (!g.rail) return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets rail with act_item_inner
+    if constexpr (ROWS_IN_N) {
+        static_assert(R == 2 && WK > 0, "item-innermost launches take two items per lane");
+        // the kernel addresses the whole stream buffer with 32-bit byte offsets; y mode only
+        if ((unsigned long long)g.act_words * 4 >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
+        if (!g.rail || g.mode != GEO_SC_ACC_Y) return GEO_SC_ERR_INVALID_ARGUMENT;  // make_geometry sets both with act_item_inner
+        // OR groups of 16 one-wide lines with whole sets of 8 c_out tiles and enough of them to fill the
+        // GPU: the workgroup that stages the activation words of its 8 tiles through LDS
+        if (WK == 1 && g.c_in == kLinLines && g.n_cotile % kLinTiles == 0 && pv % kLinHalves == 0 &&
+            tiles * (g.n_cotile / kLinTiles) >= 128) {
+            q.pv_per_block = pv / kLinHalves;
+            hipLaunchKernelGGL(k_conv_fwd_items_rail_lds, dim3((unsigned)(tiles * (g.n_cotile / kLinTiles))),
+                               dim3(64 * kLinTiles * kLinHalves), 0, s, q);
+            return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+        }
+        // Eight waves per workgroup share the (pack, kernel row) groups of their 128 items x 16 channels
+        // (the 4096 x 4096 layer at batch 1024: 4 or 16 waves 3 - 10 % slower than 8).
+        constexpr int S = 8;
+        q.pv_per_block = (pv + S - 1) / S;
+        hipLaunchKernelGGL((k_conv_fwd_items_rail_wg<WK, CU, S>), dim3((unsigned)blocks), dim3(64 * S), 0, s, q);
+        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     if (!plain) {
         const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
@@ -977,10 +1265,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
     }
     const dim3 grid((unsigned)blocks, (unsigned)(plain ? 1 : splits));
-    if constexpr (ROWS_IN_N) {
-        static_assert(R == 2 && WK > 0, "item-innermost launches take two items per lane");
-        hipLaunchKernelGGL((k_conv_fwd_items_rail<WK, CU>), grid, dim3(64), 0, s, q);
-    } else if (g.rail) {
+    if (g.rail) {
         if constexpr (R == 2 && WK > 0) {
             // two channels per trip for 1-wide kernels: with three, the six address pairs push the 32
             // sums out of the 128 registers
@@ -1048,6 +1333,7 @@ int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* 
     q.n_cotile = g.n_cotile;
     q.act_plane = (unsigned)g.act_plane;
     q.row_groups = 0;
+    q.keep_touches = 0;
     q.slots = 0;
     q.n = g.n;
     q.add_outer = g.add_outer;

@@ -160,6 +160,28 @@ def test_forward_matches_oracle(capi, so, shape_x, shape_w, pad, L, mode):
     assert np.array_equal(got, exp)
 
 
+@pytest.mark.parametrize("shape_x,shape_w,pad,L", [
+    ((300, 16, 1, 40), (20, 16, 1, 40), (0, 0), 128),   # 3 position tiles, second items past the end, 160 groups
+    ((130, 7, 1, 9), (33, 7, 1, 9), (0, 0), 256),       # channel trips 3 2 2, 72 groups, three c_out tiles
+    ((64, 4, 3, 12), (5, 4, 3, 5), (0, 0), 64),         # 3-wide kernel, output (1, 8): lanes span output columns
+    ((2, 3, 1, 2), (1, 3, 1, 2), (0, 0), 32),           # fewer groups than waves in the workgroup
+    ((257, 5, 5, 6), (17, 5, 5, 6), (0, 0), 16),        # 5-wide kernel, odd batch
+    ((2000, 16, 1, 5), (1024, 16, 1, 5), (0, 0), 64),   # groups of 16, 64 c_out tiles: the LDS-staged workgroups
+    ((4100, 16, 1, 2), (520, 16, 1, 2), (0, 0), 32),    # same with two groups only; 33 c_out tiles: not staged
+])
+def test_forward_item_innermost_streams_match_oracle(capi, so, shape_x, shape_w, pad, L):
+    """Single-row outputs (the SC-linear mapping): the workgroup kernel whose waves split the (pack,
+    kernel row) groups and add their partial sums in LDS."""
+    mode = "kaiming" if L >= 128 else "prescribed" if shape_x[0] == 2 else "sparse"
+    x, w = wl.make_inputs(shape_x, shape_w, mode, seed=L + shape_x[0])
+    d = capi.make_desc(shape_x, shape_w, L, pad)
+    assert capi.act_streams(x.cuda(), d).shape[-1] == shape_x[0]     # item-innermost geometry
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad)
+    got = gpu_forward(capi, x, w, L, pad)
+    assert np.array_equal(got, exp)
+    assert np.abs(exp).sum() > 0
+
+
 @pytest.mark.parametrize("loading", [(7, 2, 2, 2), (7, 1, 4, 4), (7, 4, 3, 3), (7, 2, 1, 1)])
 @pytest.mark.parametrize("L", [16, 64, 128])
 def test_forward_progressive_loading_matches_oracle(capi, so, loading, L):
