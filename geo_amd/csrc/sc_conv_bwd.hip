@@ -31,6 +31,8 @@
 // Members of a ragged last channel block that do not exist carry zero weights.
 #include "sc_common.h"
 
+#include <cstdlib>
+
 #include <type_traits>
 
 namespace geo_sc {
@@ -1345,6 +1347,11 @@ BwdLayout bwd_layout(const Geometry& g)
     size_t rows = ((size_t)3 << 30) / per_row;
     if (rows < 1) rows = 1;
     if (rows > (size_t)b.G.n_groups) rows = b.G.n_groups;
+    // GEO_SC_BACKWARD_GROUPS_PER_ROUND caps the add groups per round further (less scratch, more launches)
+    if (const char* cap = getenv("GEO_SC_BACKWARD_GROUPS_PER_ROUND")) {
+        const long v = atol(cap);
+        if (v >= 1 && (size_t)v < rows) rows = (size_t)v;
+    }
     if (rows * b.splits > 65535) rows = 65535 / b.splits;  // grid.z = rows * splits
     if (rows < 1) rows = 1;
     b.rows_per_chunk = (int)rows;

@@ -211,6 +211,10 @@ GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* 
  * gradient on the closed interval.  fp32 throughout, fp32 accumulation.  Either output may
  * be NULL to skip it.  bit_length and the loading fields of `desc` are validated but do not
  * enter the result.
+ * The add groups (kernel rows in mode Y) are processed in rounds of launches of as many groups as
+ * fit about 3 GB of scratch; the environment variable GEO_SC_BACKWARD_GROUPS_PER_ROUND (an integer
+ * >= 1, read at every call) lowers that number and the workspace size with it.  It must not change
+ * between the size query and the call that uses the workspace.
  */
 GEO_SC_API int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
 GEO_SC_API int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float* x, const float* w,

@@ -223,3 +223,79 @@ def test_whole_backward_of_small_or_groups(capi, shape_x, shape_w, pad, mode, zu
     assert torch.equal(gx2, gx) and rel_err(gw2, rw) <= RTOL
     gx3, gw3 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
     assert torch.equal(gx3, gx) and torch.equal(gw3, gw)   # deterministic
+
+
+# ------------------------------------------------------------------ rounds of add groups
+@pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu,cap", [
+    ((3, 12, 7, 9), (6, 12, 3, 5), (1, 2), "y", 1, 2),     # GEMM path (K = 36), 5 kernel rows in rounds of 2, 2, 1
+    ((3, 12, 7, 9), (6, 12, 3, 5), (1, 2), "y", 1, 1),     # one row per round
+    ((2, 7, 8, 8), (12, 7, 3, 3), (1, 1), "z", 1, 3),      # fused small-group kernel, 7 groups in rounds of 3, 3, 1
+    ((2, 10, 6, 5), (40, 10, 3, 2), (1, 0), "yz", 4, 4),   # yz: 3 channel blocks x 2 rows = 6 groups in rounds of 4, 2
+    ((2, 44, 6, 6), (5, 44, 3, 3), (1, 1), "yz", 20, 2),   # yz through the GEMMs (K = 60), ragged last block, rounds of 2
+    ((4, 3, 9, 9), (16, 3, 5, 5), (2, 2), "y", 1, 2),      # weight gradient alone of a first layer (K = 15)
+])
+def test_backward_in_several_rounds_of_add_groups(capi, monkeypatch, shape_x, shape_w, pad, mode, zu, cap):
+    """GEO_SC_BACKWARD_GROUPS_PER_ROUND forces what a 3 GB scratch budget only does for very large
+    layers: the add groups go through the kernels in several rounds, later rounds accumulating into
+    grad_x.  Same gradients as in one round and as the float64 oracle."""
+    from oracle import surrogate
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_x[1] + cap)
+    w = (w * 3).contiguous()
+    w.view(-1)[::7] = 0.0
+    d = capi.make_desc(x.shape, w.shape, 64, pad, accumulate=mode, z_unit=zu)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(6))
+    kw = dict(accumulate=mode, z_unit=zu)
+    one_x, one_w = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
+    bytes_one = capi.backward_workspace_size(d)
+    monkeypatch.setenv("GEO_SC_BACKWARD_GROUPS_PER_ROUND", str(cap))
+    assert capi.backward_workspace_size(d) < bytes_one
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
+    _, gw_alone = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False, **kw)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("GEO_SC_BACKWARD_GROUPS_PER_ROUND")
+    rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
+    assert rel_err(gx, rx) <= RTOL and rel_err(gw, rw) <= RTOL and rel_err(gw_alone, rw) <= RTOL
+    assert rel_err(gx, one_x) <= 1e-6 and rel_err(gw, one_w) <= 1e-6
+
+
+# ------------------------------------------------------------------ full sizes
+def _fp64_reference_on_gpu(x, w, g, pad):
+    """float64 autograd over the restated surrogate, evaluated on the GPU (the CPU would take minutes)."""
+    from oracle import surrogate
+    xr = x.cuda().double().requires_grad_(True)
+    wr = w.cuda().double().requires_grad_(True)
+    xp = torch.nn.functional.pad(xr, (pad, pad, pad, pad))
+    p, n = surrogate.surrogate_rails(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)))
+    (p - n).backward(g.cuda().double())
+    return xr.grad, wr.grad
+
+
+def test_backward_resnet_shape_full_size(capi):
+    """64->64 3x3 at 56x56, batch 128 (K = 192 members, M = 401 408 positions: the weight gradient's
+    reduction over positions is split and the scratch arrays are at their largest)."""
+    x, w, pad, _ = wl.named("C5", "q7")
+    w = (w * 8).contiguous()
+    g = torch.randn((128, 64, 56, 56), generator=torch.Generator().manual_seed(3))
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 256, (pad, pad))
+    rx, rw = _fp64_reference_on_gpu(x, w, g, pad)
+    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
+    print(f"C5 backward: grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
+    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    gx2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 256, (pad, pad))
+    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)   # deterministic
+
+
+def test_backward_linear_4096_shape(capi):
+    """The 4096 -> 4096 SC linear layer through its conv mapping (N, 16, 1, 256) * (4096, 16, 1, 256): 256
+    add groups of 16 members, 8192 rails (the fused small-group kernel, one launch per 256 rails); batch 64
+    of the 1024 so that the float64 reference stays small."""
+    x, w, pad, _ = wl.named("C4", "q7")
+    x = x[:64].contiguous()
+    w = (w * 16).contiguous()
+    g = torch.randn((64, 4096, 1, 1), generator=torch.Generator().manual_seed(5))
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad))
+    rx, rw = _fp64_reference_on_gpu(x, w, g, pad)
+    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
+    print(f"C4 backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
+    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
