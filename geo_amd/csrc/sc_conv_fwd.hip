@@ -770,7 +770,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         const int go = g / q.add_inner, gi = g - go * q.add_inner;
         const int ch0 = go * q.or_ch_per_group;
         const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
-        u32x16 p0 = 0u, p1 = 0u, n0 = 0u, n1 = 0u;
+        u32x16 p0, p1, n0, n1;  // written by the group's first line
+        bool first = true;
         const uint32_t* ap0 = act_n + (size_t)p * q.act_plane + (size_t)gi * q.add_stride + (size_t)ch0 * q.or_stride;
         const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
                             (size_t)gi * chs * q.w_k;
@@ -778,8 +779,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
         for (int row = 0; row < q.or_rows; row++) {
             const uint32_t* ap = ap0 + row;  // next kernel row: one word further
-            auto channels = [&](auto cu_tag) {
+            auto channels_of = [&](auto cu_tag, auto first_tag) {
                 constexpr int N = decltype(cu_tag)::value;
+                constexpr bool FIRST = decltype(first_tag)::value;
                 uint32_t aw[N][NW];
 #pragma unroll
                 for (int cu = 0; cu < N; cu++)
@@ -796,11 +798,22 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
                 for (int cu = 0; cu < N; cu++)
 #pragma unroll
-                    for (int u = 0; u < WK; u++)
-                        rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u], aw[cu][u + 1]);
+                    for (int u = 0; u < WK; u++) {
+                        if (FIRST && cu == 0 && u == 0)
+                            rail_line_first(p0, p1, n0, n1, wv[0], iv[0], aw[0][0], aw[0][1]);
+                        else
+                            rail_line(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u], aw[cu][u + 1]);
+                    }
                 wp += N * WK * C;
                 ip += N * WK * (C / 2);
                 ap += N * q.or_stride;
+            };
+            auto channels = [&](auto cu_tag) {
+                if (first)
+                    channels_of(cu_tag, std::true_type());
+                else
+                    channels_of(cu_tag, std::false_type());
+                first = false;
             };
             int ci = 0;
             for (; ci + CU <= chs; ci += CU) channels(std::integral_constant<int, CU>());
@@ -809,8 +822,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
 #pragma unroll
         for (int i = 0; i < C; i++) {
-            sum[i] += __popc(p0[i]) - __popc(n0[i]);
-            sum[C + i] += __popc(p1[i]) - __popc(n1[i]);
+            popc_diff(sum[i], p0[i], n0[i]);
+            popc_diff(sum[C + i], p1[i], n1[i]);
         }
     }
 
