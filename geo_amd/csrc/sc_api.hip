@@ -106,7 +106,9 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
     // batch and input size (a buffer serves every geometry of the same weights); the launches with two
     // output rows (or, item-innermost, two batch items) per lane read it: the rail-skipping kernels.
     g->wgt_rail = d->w_k == 1 || d->w_k == 3 || d->w_k == 5;
-    g->rail = g->wgt_rail && !g->thin && (wo >= 2 || g->act_item_inner);
+    // (the rail-skipping kernels address the activation stream buffer with 32-bit byte offsets)
+    g->rail = g->wgt_rail && !g->thin && (wo >= 2 || g->act_item_inner) &&
+              (unsigned long long)g->act_words * 4 < 0xffffffffull;
     const size_t lines = (size_t)g->packs * d->h_k * g->k_or;
     g->wgt_words = lines * g->n_cotile * 2 * kCoTile;
     g->wgt_rail_off = g->wgt_rail_idx_off = g->wgt_flag_off = 0;

@@ -736,6 +736,11 @@ __global__ __launch_bounds__(64 * NWV * NPT) __attribute__((amdgpu_waves_per_eu(
 // The rail-skipping form of k_conv_fwd_split<2, WK, 1, false>: launches split over blockIdx.y and
 // the accumulation modes other than y, position-major activation streams, two output rows per lane.
 // Partial sums are added to the zeroed y with integer atomics.
+// The add groups of the other modes are short (z mode: 9 lines of a 3 x 3 kernel), so what happens
+// per group is kept scalar and small: the (pack, outer, inner) group counters advance by increments (no
+// divisions), the weight lines of a c_out tile follow each other in loop order (both pointers only
+// advance), and the activation words come through buffer loads (resource over the stream buffer, one
+// 32-bit byte offset per lane and row, the group's and channel's offset as the scalar operand).
 template <int WK, int CU>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_conv_fwd_split_rail(FwdParams q)
 {
@@ -749,13 +754,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const int a0 = (int)(t % q.row_groups) * R;
     const long long n = t / q.row_groups;
     const unsigned item_stride = (unsigned)q.packs * q.act_plane;
-    unsigned off[NW];
+    // byte offsets of the lane's rows in the stream buffer (the launcher keeps the buffer under 4 GB);
+    // rows past the end (partial last group) are clamped to valid ones: they only feed outputs that are
+    // never stored
+    unsigned voff[NW];
 #pragma unroll
     for (int j = 0; j < NW; j++) {
         const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
-        off[j] = (unsigned)row * q.hi;
+        voff[j] = 4u * ((unsigned)n * item_stride + (unsigned)b + (unsigned)row * q.hi);
     }
-    const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
+    const __amdgpu_buffer_rsrc_t act = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(q.act), 0, (int)(4u * (unsigned)q.n * item_stride), 0x00020000);
+    const unsigned plane_b = 4u * q.act_plane, add_b = 4u * q.add_stride, or_b = 4u * q.or_stride;
 
     int sum[2 * C];  // [2 c + r]
 #pragma unroll
@@ -765,20 +775,28 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const int pv_begin = blockIdx.y * q.pv_per_block;
     const int pv_end = min(q.packs * groups, pv_begin + q.pv_per_block);
     const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    // group counters of pv_begin; the loop advances them
+    int p = pv_begin / groups;
+    int go = (pv_begin - p * groups) / q.add_inner;
+    int gi = pv_begin - p * groups - go * q.add_inner;
+    const uint32_t* wp;
+    const uint32_t* ip;
+    {
+        const int ch0 = go * q.or_ch_per_group;
+        const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
+        const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
+                            (size_t)gi * chs * q.w_k;
+        wp = q.wgt_rail + line * C;
+        ip = q.wgt_rail_idx + line * (C / 2);
+    }
     for (int pv = pv_begin; pv < pv_end; pv++) {
-        const int p = pv / groups, g = pv - p * groups;
-        const int go = g / q.add_inner, gi = g - go * q.add_inner;
         const int ch0 = go * q.or_ch_per_group;
         const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
         u32x16 p0, p1, n0, n1;  // written by the group's first line
         bool first = true;
-        const uint32_t* ap0 = act_n + (size_t)p * q.act_plane + (size_t)gi * q.add_stride + (size_t)ch0 * q.or_stride;
-        const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
-                            (size_t)gi * chs * q.w_k;
-        const uint32_t* wp = q.wgt_rail + line * C;
-        const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
+        const unsigned group_off = (unsigned)p * plane_b + (unsigned)gi * add_b + (unsigned)ch0 * or_b;
         for (int row = 0; row < q.or_rows; row++) {
-            const uint32_t* ap = ap0 + row;  // next kernel row: one word further
+            unsigned ch_off = group_off + 4u * (unsigned)row;  // next kernel row: one word further
             auto channels_of = [&](auto cu_tag, auto first_tag) {
                 constexpr int N = decltype(cu_tag)::value;
                 constexpr bool FIRST = decltype(first_tag)::value;
@@ -786,7 +804,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
                 for (int cu = 0; cu < N; cu++)
 #pragma unroll
-                    for (int j = 0; j < NW; j++) aw[cu][j] = ap[cu * q.or_stride + off[j]];
+                    for (int j = 0; j < NW; j++)
+                        aw[cu][j] = __builtin_amdgcn_raw_buffer_load_b32(act, (int)voff[j],
+                                                                         (int)(ch_off + (unsigned)cu * or_b), 0);
                 uint32_t wv[N * WK][C], iv[N * WK][C / 2];
 #pragma unroll
                 for (int l = 0; l < N * WK; l++) {
@@ -806,7 +826,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                     }
                 wp += N * WK * C;
                 ip += N * WK * (C / 2);
-                ap += N * q.or_stride;
+                ch_off += (unsigned)N * or_b;
             };
             auto channels = [&](auto cu_tag) {
                 if (first)
@@ -824,6 +844,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int i = 0; i < C; i++) {
             popc_diff(sum[i], p0[i], n0[i]);
             popc_diff(sum[C + i], p1[i], n1[i]);
+        }
+        // next group: inner add group, then outer, then pack
+        if (++gi == q.add_inner) {
+            gi = 0;
+            if (++go == q.add_outer) {
+                go = 0;
+                p++;
+            }
         }
     }
 
