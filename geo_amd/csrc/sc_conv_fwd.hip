@@ -638,14 +638,17 @@ __global__ __launch_bounds__(64 * NWV * NPT) __attribute__((amdgpu_waves_per_eu(
     const int a0 = (int)(t % q.row_groups) * R;
     const long long n = t / q.row_groups;
     const unsigned item_stride = (unsigned)q.packs * q.act_plane;
-    unsigned off[NW];
+    // byte offsets of the lane's four rows in the stream buffer (under 4 GB: the launcher checks), read
+    // with buffer loads: the chunk's and channel's offset is the scalar operand
+    unsigned voff[NW];
 #pragma unroll
     for (int j = 0; j < NW; j++) {
         const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
-        off[j] = (unsigned)row * q.hi;
+        voff[j] = 4u * ((unsigned)n * item_stride + (unsigned)b + (unsigned)row * q.hi);
     }
-    const unsigned ch_stride = (unsigned)q.wi * q.hi;
-    const uint32_t* act_n = q.act + (size_t)n * item_stride + b;
+    const unsigned ch_b = 4u * (unsigned)q.wi * q.hi;
+    const __amdgpu_buffer_rsrc_t act = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(q.act), 0, (int)(4u * (unsigned)q.n * item_stride), 0x00020000);
     const int chunks_per_pass = q.c_in / CH;
     // this launch row's share of the (pack, kernel row) passes; with more than one row the partial sums
     // are added to the zeroed y with integer atomics
@@ -661,11 +664,14 @@ __global__ __launch_bounds__(64 * NWV * NPT) __attribute__((amdgpu_waves_per_eu(
     uint4 fetched[CPW];
     auto fetch = [&](int pass, int cc) {
         const int p = pass / q.h_k, v = pass - p * q.h_k;
-        const uint32_t* ap = act_n + (size_t)p * q.act_plane + v + (size_t)(cc * CH + wave) * ch_stride;
+        const unsigned so = 4u * ((unsigned)p * q.act_plane + (unsigned)v) + (unsigned)(cc * CH + wave) * ch_b;
 #pragma unroll
         for (int i = 0; i < CPW; i++) {
-            const uint32_t* ac = ap + (size_t)(NWV * i) * ch_stride;
-            fetched[i] = make_uint4(ac[off[0]], ac[off[1]], ac[off[2]], ac[off[3]]);
+            const int sc = (int)(so + (unsigned)(NWV * i) * ch_b);
+            fetched[i] = make_uint4(__builtin_amdgcn_raw_buffer_load_b32(act, (int)voff[0], sc, 0),
+                                    __builtin_amdgcn_raw_buffer_load_b32(act, (int)voff[1], sc, 0),
+                                    __builtin_amdgcn_raw_buffer_load_b32(act, (int)voff[2], sc, 0),
+                                    __builtin_amdgcn_raw_buffer_load_b32(act, (int)voff[3], sc, 0));
         }
     };
     auto commit = [&](int buf) {
