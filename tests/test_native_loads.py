@@ -41,6 +41,13 @@ def test_host_side_validation_without_gpu():
         assert e.value.status == status
     with pytest.raises(capi.GeoScError):
         capi.workspace_size(capi.make_desc((2, 3, 8, 8), (4, 3, 3, 3), 64, load_width=0))
+    # stream layout query: single-row outputs of 1/3/5-wide kernels with several items are item-innermost
+    import ctypes as ct
+    from geo_amd import _native
+    inner = ct.c_int(-1)
+    for sx, sw, want in (((5, 4, 3, 6), (2, 4, 3, 3), 1), ((5, 4, 8, 6), (2, 4, 3, 3), 0), ((1, 4, 3, 6), (2, 4, 3, 3), 0)):
+        assert _native.lib().geo_sc_act_stream_layout(ct.byref(capi.make_desc(sx, sw, 64)), ct.byref(inner)) == 0
+        assert inner.value == want, (sx, sw)
     # workspace of the headline shape: tables + weight streams + activation streams
     d = capi.make_desc((256, 128, 16, 16), (128, 128, 3, 3), 128, (1, 1))
     assert capi.workspace_size(d) >= 4 * (256 * 4 * 128 * 18 * 18 + 2 * 4 * 3 * 384 * 128)
