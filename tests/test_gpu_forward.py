@@ -182,6 +182,25 @@ def test_forward_item_innermost_streams_match_oracle(capi, so, shape_x, shape_w,
     assert np.abs(exp).sum() > 0
 
 
+@pytest.mark.parametrize("shape_x,shape_w,L", [
+    ((2000, 16, 1, 5), (1024, 16, 1, 5), 64),     # the LDS-staged workgroups
+    ((130, 7, 1, 9), (33, 7, 1, 9), 128),         # the general workgroup kernel
+])
+def test_item_innermost_streams_with_loading_and_7bit_activations(capi, so, shape_x, shape_w, L):
+    """The single-row kernels behind the other ways into the forward: progressive loading (weights and
+    activations with different waits) and the uint8 entry point (activations k / 128)."""
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=L)
+    w = (w * 4).clamp(-0.99, 0.99).contiguous()
+    kw = dict(total_width=7, load_width=2, load_wait_w=2, load_wait_a=3)
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, (0, 0), **kw)
+    assert np.abs(exp).sum() > 0
+    got = gpu_forward(capi, x, w, L, (0, 0), **kw)
+    assert np.array_equal(got, exp)
+    k = (x * 128).round().to(torch.uint8)
+    got_q7 = capi.conv2d_add_partial_forward_q7(k.cuda(), w.cuda(), L, (0, 0), **kw)
+    assert np.array_equal(got_q7.cpu().numpy(), exp)
+
+
 @pytest.mark.parametrize("loading", [(7, 2, 2, 2), (7, 1, 4, 4), (7, 4, 3, 3), (7, 2, 1, 1)])
 @pytest.mark.parametrize("L", [16, 64, 128])
 def test_forward_progressive_loading_matches_oracle(capi, so, loading, L):
