@@ -883,6 +883,71 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
     }
 }
 
+// a[i] += b_1[i] + ... + b_{n-1}[i] for n arrays `stride` floats apart (a is the first), four floats
+// per thread, the arrays added in their order: the dcol slices of the fused kernel's column blocks.
+// count and stride are multiples of 4.
+__global__ __launch_bounds__(256) void k_sum_slices(float* __restrict__ a, size_t count, int n, size_t stride)
+{
+    const size_t n4 = count / 4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 256) {
+        float4 acc = ((const float4*)a)[i];
+        for (int s0 = 1; s0 < n; s0 += 8) {
+            float4 v[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) v[q] = ((const float4*)(a + (size_t)(s0 + q < n ? s0 + q : 0) * stride))[i];
+#pragma unroll
+            for (int q = 0; q < 8; q++)
+                if (s0 + q < n) {
+                    acc.x += v[q].x;
+                    acc.y += v[q].y;
+                    acc.z += v[q].z;
+                    acc.w += v[q].w;
+                }
+        }
+        ((float4*)a)[i] = acc;
+    }
+}
+
+// k_reduce_wgrad for at most four partial sums per group: a thread per (k, co) entry, a block per 256
+// entries of one group; the blocks of all groups for the same entries are neighbours in the grid
+// (blockIdx.x = entry block * n_groups_here + group), so that in y accumulation, where the weights of
+// consecutive groups are consecutive in memory, their 4-byte stores meet in the cache.
+__global__ __launch_bounds__(256) void k_reduce_wgrad_few(const float* __restrict__ part, const float* __restrict__ w,
+                                                          float* __restrict__ gw, int g0, int ng, int splits, int c_out,
+                                                          Groups G, size_t g_stride)
+{
+    const int K = G.n_members;
+    const int total = K * c_out;
+    const long long stride = (long long)K * 2 * c_out;
+    const int eb = blockIdx.x / ng, gi = blockIdx.x - eb * ng;
+    const float* partg = part + (size_t)gi * g_stride;
+    const int e = eb * 256 + threadIdx.x;
+    if (e >= total) return;
+    const int co = e % c_out, k = e / c_out;
+    const Member mb = member_of(G, g0 + gi, k);
+    if (!mb.ok) return;
+    float vp[4], vn[4];
+#pragma unroll
+    for (int s0 = 0; s0 < 4; s0++) {
+        const long long o = (s0 < splits ? s0 : 0) * stride + (long long)k * 2 * c_out + co;
+        vp[s0] = partg[o];
+        vn[s0] = partg[o + c_out];
+    }
+    float sp = vp[0], sn = vn[0];
+#pragma unroll
+    for (int s0 = 1; s0 < 4; s0++)
+        if (s0 < splits) {
+            sp += vp[s0];
+            sn += vn[s0];
+        }
+    const long long wi = (((long long)co * G.c_in + mb.ci) * G.w_k + mb.u) * G.h_k + mb.v;
+    const float wv = w[wi];
+    float r = 0.0f;
+    if (wv >= 0.0f && wv <= 100.0f) r += sp;
+    if (wv >= -100.0f && wv <= 0.0f) r += sn;
+    gw[wi] = r;
+}
+
 // Weight gradient of layers with small OR groups (K <= 16 members, 2 * c_out <= 128: first layers,
 // 3 -> 32 channels with 5 x 5 kernels has K = 15) when no input gradient is asked for.  Per tile of
 // 64 output positions the workgroup gathers the im2col columns into LDS, forms Z = col^T wcat with
@@ -1011,41 +1076,86 @@ __global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__
 }
 
 // Whole backward of layers with small OR groups (K <= 32 members: z accumulation has K = W * H,
-// yz with small channel blocks K = z_unit * W) in one kernel.  With few members per group the
-// general path's scratch array E[g][m][j] is c_in (z) times larger than the problem's tensors and
-// its GEMMs use a fraction of each MFMA; here a workgroup loops over tiles of 32 output positions
-// of one group, gathers the im2col columns into LDS, forms Z = col^T wcat with MFMAs, turns it
-// into E = g exp(-Z) in LDS and feeds both Gw += col E (accumulators live over all tiles) and
-// dcol = wd^T E^T from it; only dcol (the size of col) reaches memory, for the common col2im.
-// The weights of both products sit in registers for the life of the workgroup.
+// yz with small channel blocks K = z_unit * W, the SC linear layer K = 16) in one kernel.  With few
+// members per group the general path's scratch array E[g][m][j] is c_in (z) times larger than the
+// problem's tensors and its GEMMs use a fraction of each MFMA; here a workgroup loops over tiles of
+// 32 output positions of one group, gathers the im2col columns into LDS, forms Z = col^T wcat with
+// MFMAs, turns it into E = g exp(-Z) in LDS and feeds both Gw += col E (accumulators live over all
+// tiles) and dcol = wd^T E^T from it; only dcol (the size of col) reaches memory, for the common
+// col2im.  The weights of both products sit in registers for the life of the workgroup.
 //   KS: k-steps of the first product (ceil(K / 2), rounded up to 5, 8, 12 or 16)
-//   NB: 32-column blocks of E per wave; a launch covers NB * 128 columns from j_begin, wider
-//       layers take several launches, later ones adding to dcol
+//   NB: 32-column blocks of E per wave; a workgroup covers NB * 128 columns, wider layers take
+//       several column blocks, each writing a slice dcol[block][g][k][m] of its own that
+//       k_sum_slices adds in a fixed order
 //   DX: the input gradient is wanted
-// A workgroup handles tiles s, s + S, ... of group g0 + blockIdx.y and writes one partial sum
-// part[g][s][k][j] for the common split reduction.
+// A workgroup handles tiles s, s + S, ... of one column block of group g0 + blockIdx.y and writes
+// its columns of one partial sum part[g][s][k][j] for the common split reduction.
+//
+// The vector ALU shares its issue slots with the MFMAs, so every instruction per element of E counts:
+// the upstream gradient comes in the register order of the first product's result (k_tile_grad: four
+// 16-byte loads per 32 x 32 block, no address arithmetic per element), E is stored transposed
+// (E^T[j][m], rows of kFusedLd floats) with 16-byte stores, and no element is range-checked: rows
+// beyond M hold zeros in col and in the gradient, columns beyond 2 * c_out meet zero weights in the
+// input-gradient product and are never stored by the weight-gradient one.
 constexpr int kFusedK = 32;
 constexpr int kFusedTile = 32;
+constexpr int kFusedLd = 36;  // floats per LDS row of a tile: 16-byte aligned rows, conflict-free MFMA operand reads
+
+// Upstream gradient in tiles of 32 positions x 32 columns, each stored in the register order of a
+// 32 x 32 MFMA result: gtt[(tile * n_blocks + block) * 1024 + lane * 16 + r] = g[m][co] with
+// m = 32 tile + 8 (r / 4) + 4 (lane / 32) + r % 4 and column 32 block + lane % 32; rows beyond M and
+// columns beyond the last one are zero.  With dedupe (c_out a multiple of 32) the blocks run over
+// c_out and serve both rails, otherwise over the 2 * c_out rails (column j -> channel j mod c_out).
+// g is [n][c_out][npos]; blockIdx = (tile, block).
+__global__ __launch_bounds__(256) void k_tile_grad(const float* __restrict__ g, float* __restrict__ gtt, int M, int c_out,
+                                                   int npos, int n_blocks, int dedupe)
+{
+    __shared__ float t[32][33];  // [position][column]
+    const int m0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int n_cols = dedupe ? c_out : 2 * c_out;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    // lanes along the positions where an item has many of them, along the channels otherwise
+    const bool along_m = npos >= 8;
+    for (int q = ty; q < 32; q += 8) {
+        const int mi = along_m ? tx : q, ci = along_m ? q : tx;
+        const int m = m0 + mi, c = c0 + ci;
+        const int co = c >= c_out ? c - c_out : c;
+        float v = 0.0f;
+        if (m < M && c < n_cols) {
+            const int n = m / npos, pos = m - n * npos;
+            v = g[((size_t)n * c_out + co) * npos + pos];
+        }
+        t[mi][ci] = v;
+    }
+    __syncthreads();
+    const int o = threadIdx.x * 4, lane = o >> 4, r = o & 15;
+    const int i = 8 * (r >> 2) + 4 * (lane >> 5), l32 = lane & 31;
+    float4 v = make_float4(t[i][l32], t[i + 1][l32], t[i + 2][l32], t[i + 3][l32]);
+    *(float4*)(gtt + ((size_t)blockIdx.x * n_blocks + blockIdx.y) * 1024 + o) = v;
+}
+
 template <int KS, int NB, bool DX>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_bwd_small_k(const float* __restrict__ x, const float* __restrict__ wcat,
-                                                     const float* __restrict__ wd, const float* __restrict__ gt,
-                                                     const int* __restrict__ base, const int* __restrict__ arow,
-                                                     const int* __restrict__ bcol, float* __restrict__ part,
-                                                     float* __restrict__ dcol, Groups G, int g0, int M, int w_in, int h_in,
-                                                     int c_out, int j_begin, int splits, int store_part, int dcol_add,
-                                                     size_t w_stride, size_t part_stride, size_t dcol_stride)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_bwd_small_k(
+    const float* __restrict__ x, const float* __restrict__ wcat, const float* __restrict__ wd,
+    const float* __restrict__ gtt, const int* __restrict__ base, const int* __restrict__ arow,
+    const int* __restrict__ bcol, float* __restrict__ part, float* __restrict__ dcol, Groups G, int g0, int M, int w_in,
+    int h_in, int c_out, int jblocks, int splits, int store_part, int gt_blocks, int gt_dedupe, size_t w_stride,
+    size_t part_stride, size_t dcol_stride, size_t dcol_slice)
 {
     constexpr int KP = KS <= 8 ? 16 : 32;       // member rows held in LDS and in the weight gradient
-    constexpr int TM = kFusedTile;
-    constexpr int JW = NB * 128;                // columns of E per launch
+    constexpr int TM = kFusedTile, LD = kFusedLd;
+    constexpr int JW = NB * 128;                // columns of E per workgroup
     constexpr int DPARTS = KP == 16 ? 2 : 1;    // waves that share one 16 x 16 block of dcol and split j
     constexpr int DSTEPS = JW / DPARTS / 4;     // 16x16x4 MFMAs per wave and tile in the dcol product
     constexpr int GQ = KP / 8;                  // members gathered per thread
-    __shared__ float cs[KP][TM + 1];            // col tile [k][m]
-    __shared__ float es[TM][JW + 1];            // E tile [m][j]; the odd stride keeps column reads conflict-free
+    __shared__ __attribute__((aligned(16))) float cs[KP][LD];  // col tile [k][m]
+    __shared__ __attribute__((aligned(16))) float es[JW][LD];  // E^T tile [j][m]
     __shared__ float red[2][16][17];            // second j-half's partial dcol blocks (KP == 16)
     const int K = G.n_members, J = 2 * c_out;
     const int g = g0 + blockIdx.y;
+    // blockIdx.x = split * jblocks + column block: the workgroups that gather the same columns of x run together
+    const int split = blockIdx.x / jblocks, jblock = blockIdx.x - split * jblocks;
+    const int j_begin = jblock * JW;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int l32 = lane & 31, lk = lane >> 5, l16 = lane & 15, lq = lane >> 4;
 
@@ -1088,6 +1198,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
         g_u[q4] = e.u;
         g_v[q4] = e.v;
     }
+    // this lane's 16 values of each 32 x 32 block of the upstream gradient: block of tile 0, and the
+    // distance to the next tile of this workgroup
+    const float* gp[NB];
+#pragma unroll
+    for (int y = 0; y < NB; y++) {
+        const int j0 = j_begin + 32 * (NB * wave + y);
+        int blk = gt_dedupe ? (j0 >= c_out ? j0 - c_out : j0) >> 5 : j0 >> 5;
+        if (j0 >= J) blk = 0;  // columns outside the problem: any finite values will do
+        gp[y] = gtt + ((size_t)split * gt_blocks + blk) * 1024 + lane * 16;
+    }
+    const size_t g_step = (size_t)splits * gt_blocks * 1024;
 
     // weight-gradient accumulators: 32 x 32 blocks (lane holds rows 8 (r/4) + 4 lk + r%4 of column l32),
     // or, with at most 16 members, 16 x 16 blocks (rows 4 lq + r of column l16) at half the MFMA time
@@ -1105,10 +1226,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
             for (int r = 0; r < 4; r++) gw_acc4[b][r] = 0.0f;
     }
 
-    float* dg = dcol + (size_t)blockIdx.y * dcol_stride;
+    float* dg = dcol + (size_t)jblock * dcol_slice + (size_t)blockIdx.y * dcol_stride;
     const int n_tiles = (M + TM - 1) / TM;
-    for (int tile = blockIdx.x; tile < n_tiles; tile += splits) {
+    for (int tile = split; tile < n_tiles; tile += splits) {
         const int m0 = tile * TM;
+        // the tile's upstream gradient, asked for before anything waits: it is needed after the first product
+        float4 gv[NB][4];
+#pragma unroll
+        for (int y = 0; y < NB; y++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) gv[y][q] = ((const float4*)gp[y])[q];
+            gp[y] += g_step;
+        }
         __syncthreads();  // the previous tile's products have read cs, es and red
         {
             const bool m_ok = m0 + ml < M;
@@ -1134,48 +1263,53 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
             for (int r = 0; r < 16; r++) z[r] = 0.0f;
 #pragma unroll
             for (int t = 0; t < KS; t++) z = __builtin_amdgcn_mfma_f32_32x32x2f32(cs[2 * t + lk][l32], w_s[y][t], z, 0, 0, 0);
-            // E[m][j] = g[m][co] * exp(-Z), zero outside the problem; loads of g first, no branches
-            const int jl = 32 * (NB * wave + y) + l32, j = j_begin + jl;
-            const int co = j >= c_out ? j - c_out : j;
-            const bool j_ok = j < J;
-            float gv[16];
+            // E^T[j][m] = g[m][co] * exp(-Z): register r of the result is position 8 (r / 4) + 4 lk + r % 4
+            float* er = &es[32 * (NB * wave + y) + l32][4 * lk];
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                gv[r] = gt[(m < M && j_ok) ? (long long)m * c_out + co : 0];
-            }
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int i = 8 * (r >> 2) + 4 * lk + (r & 3);
-                es[i][jl] = (m0 + i < M && j_ok) ? gv[r] * exp_neg(z[r]) : 0.0f;
+            for (int q = 0; q < 4; q++) {
+                float4 e;
+                e.x = gv[y][q].x * exp_neg(z[4 * q + 0]);
+                e.y = gv[y][q].y * exp_neg(z[4 * q + 1]);
+                e.z = gv[y][q].z * exp_neg(z[4 * q + 2]);
+                e.w = gv[y][q].w * exp_neg(z[4 * q + 3]);
+                *(float4*)(er + 8 * q) = e;
             }
         }
         __syncthreads();
-        // Gw[k][j] += sum_m col[k][m] * E[m][j] on this wave's column blocks
+        // Gw[k][j] += sum_m col[k][m] * E[m][j] on this wave's column blocks; a lane's share of the sum
+        // over m is a run of consecutive positions, read with 16-byte loads
         if constexpr (KP == 32) {
+            float a[16];
 #pragma unroll
-            for (int mm = 0; mm < TM; mm += 2) {
-                const float a = cs[l32][mm + lk];
+            for (int q = 0; q < 4; q++) *(float4*)&a[4 * q] = *(const float4*)&cs[l32][16 * lk + 4 * q];
 #pragma unroll
-                for (int y = 0; y < NB; y++)
-                    gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, es[mm + lk][32 * (NB * wave + y) + l32], gw_acc[y], 0, 0, 0);
+            for (int y = 0; y < NB; y++) {
+                float b[16];
+#pragma unroll
+                for (int q = 0; q < 4; q++) *(float4*)&b[4 * q] = *(const float4*)&es[32 * (NB * wave + y) + l32][16 * lk + 4 * q];
+#pragma unroll
+                for (int st = 0; st < 16; st++) gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[st], b[st], gw_acc[y], 0, 0, 0);
             }
         } else {
+            float a[8];
 #pragma unroll
-            for (int mm = 0; mm < TM; mm += 4) {
-                const float a = cs[l16][mm + lq];
+            for (int q = 0; q < 2; q++) *(float4*)&a[4 * q] = *(const float4*)&cs[l16][8 * lq + 4 * q];
 #pragma unroll
-                for (int b = 0; b < 2 * NB; b++)
-                    gw_acc4[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, es[mm + lq][32 * NB * wave + 16 * b + l16], gw_acc4[b], 0, 0, 0);
+            for (int bq = 0; bq < 2 * NB; bq++) {
+                float b[8];
+#pragma unroll
+                for (int q = 0; q < 2; q++) *(float4*)&b[4 * q] = *(const float4*)&es[32 * NB * wave + 16 * bq + l16][8 * lq + 4 * q];
+#pragma unroll
+                for (int st = 0; st < 8; st++) gw_acc4[bq] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[st], b[st], gw_acc4[bq], 0, 0, 0);
             }
         }
         if (DX) {
             // dcol[k][m] = sum_j wd[j][k] * E[m][j]: one 16 x 16 block per wave (v_mfma_f32_16x16x4_f32:
             // lane l feeds A[i = l%16][k' = l/16] and B[k' = l/16][j = l%16], holds D[4 (l/16) + r][l%16])
             floatx4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+            const float* eb = &es[jd0 + lq][16 * mb + l16];
 #pragma unroll
-            for (int t = 0; t < DSTEPS; t++)
-                d = __builtin_amdgcn_mfma_f32_16x16x4f32(w_d[t], es[16 * mb + l16][jd0 + 4 * t + lq], d, 0, 0, 0);
+            for (int t = 0; t < DSTEPS; t++) d = __builtin_amdgcn_mfma_f32_16x16x4f32(w_d[t], eb[4 * t * LD], d, 0, 0, 0);
             if (DPARTS == 2) {
                 if (jpart == 1) {
 #pragma unroll
@@ -1192,16 +1326,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int k = 16 * kb + 4 * lq + r;
-                    if (k < K && m < M) {
-                        float* pd = dg + (size_t)k * M + m;
-                        *pd = dcol_add ? *pd + d[r] : d[r];
-                    }
+                    if (k < K && m < M) dg[(size_t)k * M + m] = d[r];
                 }
             }
         }
     }
     if (store_part) {
-        float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)blockIdx.x * K * J;
+        float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)split * K * J;
         if constexpr (KP == 32) {
 #pragma unroll
             for (int y = 0; y < NB; y++) {
@@ -1285,8 +1416,13 @@ struct BwdLayout {
     Groups G;
     bool small_k;        // OR groups of at most 16 members and 2 * c_out <= 128: fused weight-gradient kernel
     bool fused_k;        // OR groups of at most 32 members: whole backward in one kernel, no col / E scratch
-    int fused_splits;    // its workgroups per add group
+    int fused_jw;        // columns of E per workgroup of that kernel
+    int fused_jblocks;   // its column blocks: each writes a dcol slice of its own
+    int fused_splits;    // its workgroups per add group and column block
+    int gt_dedupe;       // its upstream-gradient tiles serve both rails (c_out a multiple of 32)
+    int gt_blocks;       // 32-column blocks of those tiles
     int rows_per_chunk;  // add groups processed by one round of launches
+    int dcol_slices;     // partial dcol arrays per round (column blocks of the fused kernel), rows_per_chunk * col_v apart
     size_t col_v, e_v, part_v, w_v;  // floats per add group of each scratch array
     size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, off_gt, bytes;
 };
@@ -1316,10 +1452,14 @@ BwdLayout bwd_layout(const Geometry& g)
     const int K = b.G.n_members;
     b.small_k = K <= kSmallK && 2 * g.c_out <= kTile;
     b.fused_k = K <= kFusedK;
+    b.fused_jw = 2 * g.c_out <= 128 ? 128 : 256;
+    b.fused_jblocks = (2 * g.c_out + b.fused_jw - 1) / b.fused_jw;
+    b.gt_dedupe = g.c_out % 32 == 0;
+    b.gt_blocks = b.gt_dedupe ? g.c_out / 32 : (2 * g.c_out + 31) / 32;
     {
         // about eight workgroups per CU in all, each looping over its share of the tiles
         const long long n_tiles = (b.m_total + kFusedTile - 1) / kFusedTile;
-        long long want = 2048 / b.G.n_groups;
+        long long want = 2048 / ((long long)b.G.n_groups * b.fused_jblocks);
         if (want > n_tiles) want = n_tiles;
         if (want > 65535) want = 65535;
         b.fused_splits = (int)(want < 1 ? 1 : want);
@@ -1342,8 +1482,9 @@ BwdLayout bwd_layout(const Geometry& g)
     b.w_v = pad64((size_t)K * 2 * g.c_out);
     // the fused kernel needs neither col nor E
     const size_t col_alloc = b.fused_k ? 0 : b.col_v, e_alloc = b.fused_k ? 0 : b.e_v;
+    b.dcol_slices = b.fused_k ? b.fused_jblocks : 1;
     // all groups in one round of launches unless that needs more than ~3 GB of scratch
-    const size_t per_row = sizeof(float) * (col_alloc + b.col_v + e_alloc + b.part_v + 2 * b.w_v);
+    const size_t per_row = sizeof(float) * (col_alloc + b.dcol_slices * b.col_v + e_alloc + b.part_v + 2 * b.w_v);
     size_t rows = ((size_t)3 << 30) / per_row;
     if (rows < 1) rows = 1;
     if (rows > (size_t)b.G.n_groups) rows = b.G.n_groups;
@@ -1358,12 +1499,18 @@ BwdLayout bwd_layout(const Geometry& g)
     size_t o = 0;
     b.off_col = o;  o += align256(sizeof(float) * rows * col_alloc);
     b.off_e = o;    o += align256(sizeof(float) * rows * e_alloc);
-    b.off_dcol = o; o += align256(sizeof(float) * rows * b.col_v);
+    b.off_dcol = o; o += align256(sizeof(float) * rows * b.col_v * b.dcol_slices);
     b.off_part = o; o += align256(sizeof(float) * rows * b.part_v);
     b.off_wcat = o; o += align256(sizeof(float) * rows * b.w_v);
     b.off_wd = o;   o += align256(sizeof(float) * rows * b.w_v);
     b.off_pos = o;  o += 3 * align256(sizeof(int) * (size_t)b.m_total);
-    b.off_gt = o;   o += align256(sizeof(float) * (size_t)b.m_total * g.c_out);
+    {
+        // [m][c_out], or the fused kernel's tiles of 32 positions x 32 columns
+        const size_t tiled = (size_t)((b.m_total + kFusedTile - 1) / kFusedTile) * b.gt_blocks * 1024;
+        const size_t plain = (size_t)b.m_total * g.c_out;
+        b.off_gt = o;
+        o += align256(sizeof(float) * (b.fused_k && tiled > plain ? tiled : plain));
+    }
     b.bytes = o;
     return b;
 }
@@ -1397,14 +1544,21 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     const int m_blocks = grid1d(M);
     hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
                        g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
+    const bool wgrad_only = !gx && gw && L.small_k;
+    const bool fused = L.fused_k && !wgrad_only;
     {
         const int npos = g.wo * g.ho;
-        if (g.n > 65535) return GEO_SC_ERR_UNSUPPORTED;  // grid.z of the transpose
-        hipLaunchKernelGGL(k_transpose_grad, dim3((npos + 31) / 32, (g.c_out + 31) / 32, g.n), dim3(256), 0, s, gy, gt,
-                           g.c_out, npos);
+        if (fused) {
+            hipLaunchKernelGGL(k_tile_grad, dim3((M + kFusedTile - 1) / kFusedTile, L.gt_blocks), dim3(256), 0, s, gy, gt, M,
+                               g.c_out, npos, L.gt_blocks, L.gt_dedupe);
+        } else {
+            if (g.n > 65535) return GEO_SC_ERR_UNSUPPORTED;  // grid.z of the transpose
+            hipLaunchKernelGGL(k_transpose_grad, dim3((npos + 31) / 32, (g.c_out + 31) / 32, g.n), dim3(256), 0, s, gy, gt,
+                               g.c_out, npos);
+        }
     }
     int rc;
-    if (!gx && gw && L.small_k) {
+    if (wgrad_only) {
         // first-layer case: fused im2col + both products, no col / E scratch traffic
         for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
             const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
@@ -1431,25 +1585,27 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         }
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
-    if (L.fused_k && !(!gx && gw && L.small_k)) {
+    if (fused) {
         if (!gx && !gw) return GEO_SC_OK;
         const int plane_blocks = (g.w_in * g.h_in + 255) / 256;
         const int n_planes = g.n * g.c_in;
         const int pb = plane_blocks > 64 ? 64 : plane_blocks;
         const int want = 256 * 16 / pb;
         const int ks = (K + 1) / 2;
-        const int jw = J <= 128 ? 128 : 256;
+        const int jw = L.fused_jw;
+        const size_t slice = (size_t)L.rows_per_chunk * L.col_v;
+        if ((long long)L.fused_splits * L.fused_jblocks > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
         for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
             const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
             int wb = grid1d((long long)K * g.c_out);
             hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
                                g.c_out, G, L.w_v);
-            const dim3 grid(L.fused_splits, nv);
-            for (int jb = 0; jb < J; jb += jw) {
+            const dim3 grid(L.fused_splits * L.fused_jblocks, nv);
+            {
 #define GEO_SC_FUSED_K(KS, NB, DX)                                                                                     \
     hipLaunchKernelGGL((k_bwd_small_k<KS, NB, DX>), grid, dim3(256), 0, s, x, wcat, wd, gt, pos_base, pos_arow,         \
-                       pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, jb, L.fused_splits, gw ? 1 : 0,         \
-                       jb > 0 ? 1 : 0, L.w_v, L.part_v, L.col_v)
+                       pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks, L.fused_splits,        \
+                       gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v, slice)
 #define GEO_SC_FUSED_NB_DX(KS)                                                                                         \
     do {                                                                                                               \
         if (jw == 128) {                                                                                               \
@@ -1465,9 +1621,18 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
 #undef GEO_SC_FUSED_NB_DX
 #undef GEO_SC_FUSED_K
             }
-            if (gw)
-                hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
-                                   L.fused_splits, g.c_out, G, L.part_v);
+            if (gw) {
+                const long long few_blocks = (long long)((K * g.c_out + 255) / 256) * nv;
+                if (L.fused_splits <= 4 && few_blocks <= 0x7fffffffLL)
+                    hipLaunchKernelGGL(k_reduce_wgrad_few, dim3((unsigned)few_blocks), dim3(256), 0, s, part, w, gw, v0, nv,
+                                       L.fused_splits, g.c_out, G, L.part_v);
+                else
+                    hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
+                                       L.fused_splits, g.c_out, G, L.part_v);
+            }
+            if (gx && L.dcol_slices > 1)
+                hipLaunchKernelGGL(k_sum_slices, dim3(grid1d((long long)((size_t)nv * L.col_v / 4))), dim3(256), 0, s, dcol,
+                                   (size_t)nv * L.col_v, L.dcol_slices, slice);
             if (gx)
                 hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx,
                                    v0, nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
