@@ -883,6 +883,93 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
     }
 }
 
+// (ci, u, v) of the flat index i of one output channel's weights
+__device__ __forceinline__ void weight_coords(const Groups& G, int i, int& ci, int& u, int& v)
+{
+    const int t = i / G.h_k;
+    v = i - t * G.h_k;
+    ci = t / G.w_k;
+    u = t - ci * G.w_k;
+}
+
+// wcat of the groups [g0, g0 + ng) for the fused kernel (which forms wd from it): a block moves a
+// tile of 32 output channels x 32 consecutive weights of each through LDS, so that w is read and wcat
+// written in 128-byte runs whatever the accumulation mode (k_weight_operands reads or writes one
+// element per cache line when the members of a group are not neighbours in w).  Only members that
+// exist are written: not for ragged channel blocks.  blockIdx = (weight tile, channel tile).
+__global__ __launch_bounds__(256) void k_weight_cat_tiled(const float* __restrict__ w, float* __restrict__ wcat, int g0,
+                                                          int ng, int c_out, Groups G, size_t g_stride)
+{
+    __shared__ float t[32][33];  // [channel][weight]
+    const int per_channel = G.c_in * G.w_k * G.h_k;
+    const int i0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int q = ty; q < 32; q += 8) {
+        const int co = c0 + q, i = i0 + tx;
+        t[q][tx] = (co < c_out && i < per_channel) ? w[(size_t)co * per_channel + i] : 0.0f;
+    }
+    __syncthreads();
+    for (int q = ty; q < 32; q += 8) {
+        const int i = i0 + q, co = c0 + tx;
+        if (i >= per_channel || co >= c_out) continue;
+        int ci, u, v, g, k;
+        weight_coords(G, i, ci, u, v);
+        group_of(G, ci, u, v, g, k);
+        if (g < g0 || g >= g0 + ng) continue;
+        const float wv = t[tx][q];
+        float* row = wcat + (size_t)(g - g0) * g_stride + (size_t)k * 2 * c_out;
+        row[co] = fminf(fmaxf(wv, 0.0f), 100.0f);
+        row[c_out + co] = -fminf(fmaxf(wv, -100.0f), 0.0f);
+    }
+}
+
+// k_reduce_wgrad with the same tiles: the partial sums part[g][s][k][j] of 32 weights x 32 channels
+// are read in 128-byte runs along the channel, added over the splits in their order, and dL/dw is
+// written in 128-byte runs along the weights of one channel.
+__global__ __launch_bounds__(256) void k_reduce_wgrad_tiled(const float* __restrict__ part, const float* __restrict__ w,
+                                                            float* __restrict__ gw, int g0, int ng, int splits, int c_out,
+                                                            Groups G, size_t g_stride)
+{
+    __shared__ float tp[32][33], tn[32][33];  // [weight][channel]
+    const int per_channel = G.c_in * G.w_k * G.h_k;
+    const long long stride = (long long)G.n_members * 2 * c_out;
+    const int i0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int q = ty; q < 32; q += 8) {
+        const int i = i0 + q, co = c0 + tx;
+        float sp = 0.0f, sn = 0.0f;
+        if (i < per_channel && co < c_out) {
+            int ci, u, v, g, k;
+            weight_coords(G, i, ci, u, v);
+            group_of(G, ci, u, v, g, k);
+            if (g >= g0 && g < g0 + ng) {
+                const float* src = part + (size_t)(g - g0) * g_stride + (size_t)k * 2 * c_out + co;
+                for (int s0 = 0; s0 < splits; s0++) {
+                    sp += src[s0 * stride];
+                    sn += src[s0 * stride + c_out];
+                }
+            }
+        }
+        tp[q][tx] = sp;
+        tn[q][tx] = sn;
+    }
+    __syncthreads();
+    for (int q = ty; q < 32; q += 8) {
+        const int co = c0 + q, i = i0 + tx;
+        if (i >= per_channel || co >= c_out) continue;
+        int ci, u, v, g, k;
+        weight_coords(G, i, ci, u, v);
+        group_of(G, ci, u, v, g, k);
+        if (g < g0 || g >= g0 + ng) continue;
+        const size_t wi = (size_t)co * per_channel + i;
+        const float wv = w[wi];
+        float r = 0.0f;
+        if (wv >= 0.0f && wv <= 100.0f) r += tp[tx][q];
+        if (wv >= -100.0f && wv <= 0.0f) r += tn[tx][q];
+        gw[wi] = r;
+    }
+}
+
 // a[i] += b_1[i] + ... + b_{n-1}[i] for n arrays `stride` floats apart (a is the first), four floats
 // per thread, the arrays added in their order: the dcol slices of the fused kernel's column blocks.
 // count and stride are multiples of 4.
@@ -906,46 +993,6 @@ __global__ __launch_bounds__(256) void k_sum_slices(float* __restrict__ a, size_
         }
         ((float4*)a)[i] = acc;
     }
-}
-
-// k_reduce_wgrad for at most four partial sums per group: a thread per (k, co) entry, a block per 256
-// entries of one group; the blocks of all groups for the same entries are neighbours in the grid
-// (blockIdx.x = entry block * n_groups_here + group), so that in y accumulation, where the weights of
-// consecutive groups are consecutive in memory, their 4-byte stores meet in the cache.
-__global__ __launch_bounds__(256) void k_reduce_wgrad_few(const float* __restrict__ part, const float* __restrict__ w,
-                                                          float* __restrict__ gw, int g0, int ng, int splits, int c_out,
-                                                          Groups G, size_t g_stride)
-{
-    const int K = G.n_members;
-    const int total = K * c_out;
-    const long long stride = (long long)K * 2 * c_out;
-    const int eb = blockIdx.x / ng, gi = blockIdx.x - eb * ng;
-    const float* partg = part + (size_t)gi * g_stride;
-    const int e = eb * 256 + threadIdx.x;
-    if (e >= total) return;
-    const int co = e % c_out, k = e / c_out;
-    const Member mb = member_of(G, g0 + gi, k);
-    if (!mb.ok) return;
-    float vp[4], vn[4];
-#pragma unroll
-    for (int s0 = 0; s0 < 4; s0++) {
-        const long long o = (s0 < splits ? s0 : 0) * stride + (long long)k * 2 * c_out + co;
-        vp[s0] = partg[o];
-        vn[s0] = partg[o + c_out];
-    }
-    float sp = vp[0], sn = vn[0];
-#pragma unroll
-    for (int s0 = 1; s0 < 4; s0++)
-        if (s0 < splits) {
-            sp += vp[s0];
-            sn += vn[s0];
-        }
-    const long long wi = (((long long)co * G.c_in + mb.ci) * G.w_k + mb.u) * G.h_k + mb.v;
-    const float wv = w[wi];
-    float r = 0.0f;
-    if (wv >= 0.0f && wv <= 100.0f) r += sp;
-    if (wv >= -100.0f && wv <= 0.0f) r += sn;
-    gw[wi] = r;
 }
 
 // Weight gradient of layers with small OR groups (K <= 16 members, 2 * c_out <= 128: first layers,
@@ -1136,8 +1183,8 @@ __global__ __launch_bounds__(256) void k_tile_grad(const float* __restrict__ g, 
 
 template <int KS, int NB, bool DX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_bwd_small_k(
-    const float* __restrict__ x, const float* __restrict__ wcat, const float* __restrict__ wd,
-    const float* __restrict__ gtt, const int* __restrict__ base, const int* __restrict__ arow,
+    const float* __restrict__ x, const float* __restrict__ wcat, const float* __restrict__ gtt,
+    const int* __restrict__ base, const int* __restrict__ arow,
     const int* __restrict__ bcol, float* __restrict__ part, float* __restrict__ dcol, Groups G, int g0, int M, int w_in,
     int h_in, int c_out, int jblocks, int splits, int store_part, int gt_blocks, int gt_dedupe, size_t w_stride,
     size_t part_stride, size_t dcol_stride, size_t dcol_slice)
@@ -1159,32 +1206,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int l32 = lane & 31, lk = lane >> 5, l16 = lane & 15, lq = lane >> 4;
 
+    // this group's wcat[k][j_begin .. j_begin + JW) through LDS (the space of es), read in 128-byte
+    // runs; zero outside the problem
+    constexpr int WLD = JW + 1;
+    float* wl = &es[0][0];
+    {
+        const float* wg = wcat + (size_t)blockIdx.y * w_stride;
+        for (int e = threadIdx.x; e < KP * JW; e += 256) {
+            const int k = e / JW, jl = e - k * JW, j = j_begin + jl;
+            const bool ok = k < K && j < J;
+            const float v = wg[ok ? (size_t)k * J + j : 0];
+            wl[k * WLD + jl] = ok ? v : 0.0f;
+        }
+    }
+    __syncthreads();
     // weights of the first product, B operand of step t: wcat[k = 2 t + lk][j]
-    const float* wg = wcat + (size_t)blockIdx.y * w_stride;
     float w_s[NB][KS];
 #pragma unroll
     for (int y = 0; y < NB; y++)
 #pragma unroll
-        for (int t = 0; t < KS; t++) {
-            const int k = 2 * t + lk, j = j_begin + 32 * (NB * wave + y) + l32;
-            const bool ok = k < K && j < J;
-            const float v = wg[ok ? (size_t)k * J + j : 0];
-            w_s[y][t] = ok ? v : 0.0f;
-        }
-    // dcol: wave -> (member block kb, position block mb, j part); A operand of step t: wd[j][k = 16 kb + l16]
+        for (int t = 0; t < KS; t++) w_s[y][t] = wl[(2 * t + lk) * WLD + 32 * (NB * wave + y) + l32];
+    // dcol: wave -> (member block kb, position block mb, j part); A operand of step t: wd[j][k = 16 kb + l16],
+    // which is wcat[k][j] with the negative rail (j >= c_out) negated (it enters dL/dx with a minus sign)
     const int kb = KP == 32 ? wave >> 1 : 0, mb = wave & 1, jpart = KP == 32 ? 0 : wave >> 1;
     const int jd0 = jpart * (JW / DPARTS);
     float w_d[DX ? DSTEPS : 1];
     if (DX) {
-        const float* wdg = wd + (size_t)blockIdx.y * w_stride;
 #pragma unroll
         for (int t = 0; t < DSTEPS; t++) {
-            const int j = j_begin + jd0 + 4 * t + lq, k = 16 * kb + l16;
-            const bool ok = k < K && j < J;
-            const float v = wdg[ok ? (size_t)j * K + k : 0];
-            w_d[t] = ok ? v : 0.0f;
+            const int jl = jd0 + 4 * t + lq;
+            const float v = wl[(16 * kb + l16) * WLD + jl];
+            w_d[t] = j_begin + jl >= c_out ? -v : v;
         }
     }
+    // (the tile loop's first barriers come before anything is written to es)
     // im2col gather: thread -> position (t & 31) of the tile, members (t >> 5) + 8 q
     const int ml = threadIdx.x & 31, slot = threadIdx.x >> 5;
     int g_off[GQ], g_u[GQ], g_v[GQ];
@@ -1597,13 +1652,20 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         if ((long long)L.fused_splits * L.fused_jblocks > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
         for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
             const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
-            int wb = grid1d((long long)K * g.c_out);
-            hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
-                               g.c_out, G, L.w_v);
+            // channel blocks with a ragged end have members that do not exist: their zeros come from the plain kernel
+            const bool ragged = G.mode == GEO_SC_ACC_YZ && g.c_in % G.zu != 0;
+            const dim3 w_tiles((g.c_in * g.w_k * g.h_k + 31) / 32, (g.c_out + 31) / 32);
+            if (ragged) {
+                int wb = grid1d((long long)K * g.c_out);
+                hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
+                                   g.c_out, G, L.w_v);
+            } else {
+                hipLaunchKernelGGL(k_weight_cat_tiled, w_tiles, dim3(256), 0, s, w, wcat, v0, nv, g.c_out, G, L.w_v);
+            }
             const dim3 grid(L.fused_splits * L.fused_jblocks, nv);
             {
 #define GEO_SC_FUSED_K(KS, NB, DX)                                                                                     \
-    hipLaunchKernelGGL((k_bwd_small_k<KS, NB, DX>), grid, dim3(256), 0, s, x, wcat, wd, gt, pos_base, pos_arow,         \
+    hipLaunchKernelGGL((k_bwd_small_k<KS, NB, DX>), grid, dim3(256), 0, s, x, wcat, gt, pos_base, pos_arow,             \
                        pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks, L.fused_splits,        \
                        gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v, slice)
 #define GEO_SC_FUSED_NB_DX(KS)                                                                                         \
@@ -1622,10 +1684,10 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
 #undef GEO_SC_FUSED_K
             }
             if (gw) {
-                const long long few_blocks = (long long)((K * g.c_out + 255) / 256) * nv;
-                if (L.fused_splits <= 4 && few_blocks <= 0x7fffffffLL)
-                    hipLaunchKernelGGL(k_reduce_wgrad_few, dim3((unsigned)few_blocks), dim3(256), 0, s, part, w, gw, v0, nv,
-                                       L.fused_splits, g.c_out, G, L.part_v);
+                // few partial sums (wide layers): coalesced tiles; many: the kernel that adds eight splits side by side
+                if (L.fused_splits <= 4)
+                    hipLaunchKernelGGL(k_reduce_wgrad_tiled, w_tiles, dim3(256), 0, s, part, w, gw, v0, nv, L.fused_splits,
+                                       g.c_out, G, L.part_v);
                 else
                     hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
                                        L.fused_splits, g.c_out, G, L.part_v);
