@@ -1412,6 +1412,294 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
     }
 }
 
+// The fused kernel on the bf16 matrix cores, for K <= 16 members and more than 128 rails.  The fp32
+// MFMAs of k_bwd_small_k run on the vector ALU's multipliers: while one executes, no wave of the SIMD
+// issues vector instructions, and the kernel's time is the sum of its MFMA and vector work.  The bf16
+// MFMAs have a pipe of their own.  Here every operand is split into three bf16 terms as in
+// k_gemm_split (six term products per product, fp32 accumulation): the weights once per workgroup,
+// col once per tile, E once per element (eleven vector instructions per pair), and all three
+// products take 72 bf16 MFMAs per wave and tile (1152 cycles of the matrix pipe, beside the vector
+// work) where the fp32 kernel takes 80 fp32 ones (3072 cycles of the vector pipe).
+//   first product   32x32x16: A = col[m][k] (csz), B = wcat[k][j] (registers)
+//   weight gradient 16x16x32: A = col[k][m] (csg), B = E[m][j] read from E^T[j][m]: 8 consecutive m
+//   input gradient  16x16x32: A = wd[k][j] (registers), B = E[m][j] for 8 consecutive j: eight 2-byte
+//                   reads down a column of E^T (rows of kBfEw words keep them free of bank conflicts)
+// Same grid, arguments, tiles and outputs as k_bwd_small_k<8, 2, DX>.
+constexpr int kBfEw = 18;  // words per row of E^T: 32 bf16 and padding
+constexpr int kBfCw = 20;  // words per row of col[k][m]: 16-byte aligned rows
+
+template <bool DX>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k_bwd_small_k_bf16(
+    const float* __restrict__ x, const float* __restrict__ wcat, const float* __restrict__ gtt,
+    const int* __restrict__ base, const int* __restrict__ arow, const int* __restrict__ bcol, float* __restrict__ part,
+    float* __restrict__ dcol, Groups G, int g0, int M, int w_in, int h_in, int c_out, int jblocks, int splits,
+    int store_part, int gt_blocks, int gt_dedupe, size_t w_stride, size_t part_stride, size_t dcol_stride,
+    size_t dcol_slice)
+{
+    constexpr int KP = 16, TM = kFusedTile, JW = 256, EW = kBfEw, CW = kBfCw, NT = 512;
+    // col of two tiles in turn: the next tile's is written while this tile's products run
+    __shared__ __attribute__((aligned(16))) uint4 csz[2][3][2][TM];      // first product: (term, k half, m) -> 8 bf16 along k
+    __shared__ __attribute__((aligned(16))) unsigned csg[2][3][KP][CW];  // weight gradient: [term][k][m], two m per word
+    __shared__ __attribute__((aligned(16))) unsigned est[3][JW][EW];  // E^T: [term][j][m], two m per word
+    __shared__ float red[3][2][16][17];                               // the other j quarters' partial dcol blocks
+    const int K = G.n_members, J = 2 * c_out;
+    const int g = g0 + blockIdx.y;
+    const int split = blockIdx.x / jblocks, jblock = blockIdx.x - split * jblocks;
+    const int j_begin = jblock * JW;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int l32 = lane & 31, lk = lane >> 5, l16 = lane & 15, lq = lane >> 4;
+    // smallest terms first; 0 = hi, 1 = mid, 2 = lo
+    constexpr int ta[6] = {2, 0, 1, 1, 0, 0}, tb[6] = {0, 2, 1, 0, 1, 0};
+
+    // this group's wcat[k][j_begin .. j_begin + JW) through LDS (the space of est); zero outside the problem
+    constexpr int WLD = JW + 1;
+    float* wl = (float*)&est[0][0][0];
+    {
+        const float* wg = wcat + (size_t)blockIdx.y * w_stride;
+        for (int e = threadIdx.x; e < KP * JW; e += NT) {
+            const int k = e / JW, jl = e - k * JW, j = j_begin + jl;
+            const bool ok = k < K && j < J;
+            const float v = wg[ok ? (size_t)k * J + j : 0];
+            wl[k * WLD + jl] = ok ? v : 0.0f;
+        }
+    }
+    __syncthreads();
+    // first product, B operand: lane -> column 32 wave + l32, k = 8 lk .. + 7
+    bf16x8 wz[3];
+    {
+        unsigned h[4], m[4], l[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float* src = wl + (8 * lk + 2 * c) * WLD + 32 * wave + l32;
+            split3(src[0], src[WLD], h[c], m[c], l[c]);
+        }
+        wz[0] = __builtin_bit_cast(bf16x8, make_uint4(h[0], h[1], h[2], h[3]));
+        wz[1] = __builtin_bit_cast(bf16x8, make_uint4(m[0], m[1], m[2], m[3]));
+        wz[2] = __builtin_bit_cast(bf16x8, make_uint4(l[0], l[1], l[2], l[3]));
+    }
+    // input gradient: wave -> (position block mb, j quarter jpart); A operand of step st: wd[j][k = l16] for
+    // j = jd0 + 32 st + 8 lq .. + 7, which is wcat[k][j] with the negative rail (j >= c_out) negated
+    const int mb = wave & 1, jpart = wave >> 1;
+    const int jd0 = jpart * (JW / 4);
+    bf16x8 wdr[DX ? 2 : 1][3];
+    if (DX) {
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            unsigned h[4], m[4], l[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int jl = jd0 + 32 * st + 8 * lq + 2 * c;
+                float v0 = wl[l16 * WLD + jl], v1 = wl[l16 * WLD + jl + 1];
+                if (j_begin + jl >= c_out) v0 = -v0;
+                if (j_begin + jl + 1 >= c_out) v1 = -v1;
+                split3(v0, v1, h[c], m[c], l[c]);
+            }
+            wdr[st][0] = __builtin_bit_cast(bf16x8, make_uint4(h[0], h[1], h[2], h[3]));
+            wdr[st][1] = __builtin_bit_cast(bf16x8, make_uint4(m[0], m[1], m[2], m[3]));
+            wdr[st][2] = __builtin_bit_cast(bf16x8, make_uint4(l[0], l[1], l[2], l[3]));
+        }
+    }
+    // (the tile loop's first barriers come before anything is written to est)
+
+    // im2col gather by the first four waves: thread -> position (t & 31) of the tile, members 2 (t >> 5) and
+    // 2 (t >> 5) + 1
+    const int ml = threadIdx.x & 31, kg = (threadIdx.x >> 5) & 7;
+    const bool gathers = threadIdx.x < 256;
+    int g_off[2], g_u[2], g_v[2];
+    bool g_ok[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+        const int k = 2 * kg + q;
+        const Member e = member_of(G, g, k < K ? k : 0);
+        g_ok[q] = gathers && k < K && e.ok;
+        g_off[q] = (e.ci * w_in + e.u) * h_in + e.v;
+        g_u[q] = e.u;
+        g_v[q] = e.v;
+    }
+    // this lane's 16 values of the wave's 32 x 32 block of the upstream gradient: offset in tile `split`, and
+    // the distance to the next tile of this workgroup
+    size_t g_at;
+    {
+        const int j0 = j_begin + 32 * wave;
+        int blk = gt_dedupe ? (j0 >= c_out ? j0 - c_out : j0) >> 5 : j0 >> 5;
+        if (j0 >= J) blk = 0;  // columns outside the problem: any finite values will do
+        g_at = ((size_t)split * gt_blocks + blk) * 1024 + lane * 16;
+    }
+    const size_t g_step = (size_t)splits * gt_blocks * 1024;
+
+    floatx4 gw_acc4[2];
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) gw_acc4[b][r] = 0.0f;
+
+    float* dg = dcol + (size_t)jblock * dcol_slice + (size_t)blockIdx.y * dcol_stride;
+    const int n_tiles = (M + TM - 1) / TM;
+    // The gather runs a tile ahead and its table entries two: a tile's columns of x are asked for at the
+    // top of the tile before and its table entries at the top of the one before that, so that no tile
+    // waits for two dependent loads in a row.
+    struct Where {
+        int r0, c0, b0;
+        bool ok;
+    };
+    auto where = [&](int tile) {
+        Where p;
+        p.ok = gathers && tile < n_tiles && tile * TM + ml < M;
+        const int mc = p.ok ? tile * TM + ml : 0;
+        p.r0 = arow[mc];
+        p.c0 = bcol[mc];
+        p.b0 = base[mc];
+        return p;
+    };
+    auto fetch = [&](const Where& p, float (&v)[2], bool (&ok)[2]) {
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int rr = p.r0 + g_u[q], cc = p.c0 + g_v[q];
+            ok[q] = p.ok && g_ok[q] && cc >= 0 && cc < h_in && rr >= 0 && rr < w_in;
+            v[q] = x[ok[q] ? p.b0 + g_off[q] : 0];
+        }
+    };
+    float x_next[2], x_after[2];
+    bool ok_next[2], ok_after[2];
+    Where w_after;
+    auto commit = [&](int buf, const float (&v)[2], const bool (&ok)[2]) {
+        unsigned t3[3];
+        split3(ok[0] ? v[0] : 0.0f, ok[1] ? v[1] : 0.0f, t3[0], t3[1], t3[2]);
+#pragma unroll
+        for (int t = 0; t < 3; t++) {
+            ((unsigned*)&csz[buf][t][kg >> 2][ml])[kg & 3] = t3[t];
+            ((unsigned short*)&csg[buf][t][2 * kg][0])[ml] = (unsigned short)t3[t];
+            ((unsigned short*)&csg[buf][t][2 * kg + 1][0])[ml] = (unsigned short)(t3[t] >> 16);
+        }
+    };
+    {
+        const Where w0 = where(split);
+        fetch(w0, x_next, ok_next);
+        if (gathers) commit(0, x_next, ok_next);
+        const Where w1 = where(split + splits);
+        fetch(w1, x_next, ok_next);
+        w_after = where(split + 2 * splits);
+    }
+    __syncthreads();  // the first tile's col is in place, and every wave has taken its weights out of est's space
+    int buf = 0;
+    for (int tile = split; tile < n_tiles; tile += splits, buf ^= 1) {
+        const int m0 = tile * TM;
+        float4 gv[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) gv[q] = ((const float4*)(gtt + g_at))[q];
+        g_at += g_step;
+        fetch(w_after, x_after, ok_after);
+        w_after = where(tile + 3 * splits);
+        {
+            // Z[m][j] = sum_k col[k][m] * wcat[k][j] for the wave's 32 x 32 block; then E^T[j][m] =
+            // g[m][co] * exp(-Z), split into its terms: register r is position 8 (r / 4) + 4 lk + r % 4
+            bf16x8 az[3];
+#pragma unroll
+            for (int t = 0; t < 3; t++) az[t] = __builtin_bit_cast(bf16x8, csz[buf][t][lk][l32]);
+            floatx16 z;
+#pragma unroll
+            for (int r = 0; r < 16; r++) z[r] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < 6; t++) z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(az[ta[t]], wz[tb[t]], z, 0, 0, 0);
+            const int j = 32 * wave + l32;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float e0 = gv[q].x * exp_neg(z[4 * q + 0]), e1 = gv[q].y * exp_neg(z[4 * q + 1]);
+                const float e2 = gv[q].z * exp_neg(z[4 * q + 2]), e3 = gv[q].w * exp_neg(z[4 * q + 3]);
+                unsigned h0, m0w, l0, h1, m1w, l1;
+                split3(e0, e1, h0, m0w, l0);
+                split3(e2, e3, h1, m1w, l1);
+                *(uint2*)&est[0][j][4 * q + 2 * lk] = make_uint2(h0, h1);
+                *(uint2*)&est[1][j][4 * q + 2 * lk] = make_uint2(m0w, m1w);
+                *(uint2*)&est[2][j][4 * q + 2 * lk] = make_uint2(l0, l1);
+            }
+        }
+        __syncthreads();
+        {
+            // Gw[k][j] += sum_m col[k][m] * E[m][j]: two 16-column blocks of the wave, lane -> m = 8 lq .. + 7
+            bf16x8 ag[3];
+#pragma unroll
+            for (int t = 0; t < 3; t++) ag[t] = __builtin_bit_cast(bf16x8, *(const uint4*)&csg[buf][t][l16][4 * lq]);
+            bf16x8 bg[2][3];
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int t = 0; t < 3; t++) {
+                    const unsigned* row = &est[t][32 * wave + 16 * b + l16][4 * lq];
+                    const uint2 p0 = *(const uint2*)row, p1 = *(const uint2*)(row + 2);
+                    bg[b][t] = __builtin_bit_cast(bf16x8, make_uint4(p0.x, p0.y, p1.x, p1.y));
+                }
+#pragma unroll
+            for (int t = 0; t < 6; t++)
+#pragma unroll
+                for (int b = 0; b < 2; b++)
+                    gw_acc4[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ag[ta[t]], bg[b][tb[t]], gw_acc4[b], 0, 0, 0);
+        }
+        // the next tile's col, into the buffer whose readers finished before the last barrier
+        if (gathers) commit(buf ^ 1, x_next, ok_next);
+        floatx4 d[2];
+        if (DX) {
+            // dcol[k][m] = sum_j wd[j][k] * E[m][j]: one 16 x 16 block per wave over its quarter of j, lane ->
+            // position 16 mb + l16, j = jd0 + 32 st + 8 lq .. + 7; the two steps in accumulators of their own
+            const unsigned short* eh = (const unsigned short*)&est[0][jd0 + 8 * lq][0] + 16 * mb + l16;
+            bf16x8 bd[2][3];
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int t = 0; t < 3; t++) {
+                    unsigned wv[4];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const unsigned short* pe = eh + ((t * JW + 32 * st + 2 * c) * EW) * 2;
+                        wv[c] = (unsigned)pe[0] | ((unsigned)pe[2 * EW] << 16);
+                    }
+                    bd[st][t] = __builtin_bit_cast(bf16x8, make_uint4(wv[0], wv[1], wv[2], wv[3]));
+                }
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) d[st][r] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < 6; t++)
+#pragma unroll
+                for (int st = 0; st < 2; st++)
+                    d[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wdr[st][ta[t]], bd[st][tb[t]], d[st], 0, 0, 0);
+            if (jpart > 0) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) red[jpart - 1][mb][4 * lq + r][l16] = d[0][r] + d[1][r];
+            }
+        }
+        // every wave has read this tile's E and col, and written the next tile's col and its share of red
+        __syncthreads();
+        if (DX && jpart == 0) {
+            const int m = m0 + 16 * mb + l16;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int k = 4 * lq + r;
+                const float sum = ((d[0][r] + d[1][r]) + red[0][mb][k][l16]) + (red[1][mb][k][l16] + red[2][mb][k][l16]);
+                if (k < K && m < M) dg[(size_t)k * M + m] = sum;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            x_next[q] = x_after[q];
+            ok_next[q] = ok_after[q];
+        }
+    }
+    if (store_part) {
+        float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)split * K * J;
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int j = j_begin + 32 * wave + 16 * b + l16;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int k = 4 * lq + r;
+                if (k < K && j < J) pg[(size_t)k * J + j] = gw_acc4[b][r];
+            }
+        }
+    }
+}
+
 int grid1d(long long total)
 {
     long long blocks = (total + 255) / 256;
@@ -1676,7 +1964,18 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             if (gx) GEO_SC_FUSED_K(KS, 2, true); else GEO_SC_FUSED_K(KS, 2, false);                                    \
         }                                                                                                              \
     } while (0)
-                if (ks <= 5) GEO_SC_FUSED_NB_DX(5);
+                if (ks <= 8 && jw == 256) {
+                    if (gx)
+                        hipLaunchKernelGGL(k_bwd_small_k_bf16<true>, grid, dim3(512), 0, s, x, wcat, gt, pos_base, pos_arow,
+                                           pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks,
+                                           L.fused_splits, gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v,
+                                           slice);
+                    else
+                        hipLaunchKernelGGL(k_bwd_small_k_bf16<false>, grid, dim3(512), 0, s, x, wcat, gt, pos_base, pos_arow,
+                                           pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks,
+                                           L.fused_splits, gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v,
+                                           slice);
+                } else if (ks <= 5) GEO_SC_FUSED_NB_DX(5);
                 else if (ks <= 8) GEO_SC_FUSED_NB_DX(8);
                 else if (ks <= 12) GEO_SC_FUSED_NB_DX(12);
                 else GEO_SC_FUSED_NB_DX(16);
