@@ -31,6 +31,7 @@
 // Members of a ragged last channel block that do not exist carry zero weights.
 #include "sc_common.h"
 
+#include <cstdint>
 #include <cstdlib>
 
 #include <type_traits>
@@ -769,6 +770,59 @@ __global__ __launch_bounds__(256) void k_im2col_rows(const float* __restrict__ x
     }
 }
 
+// Four consecutive values of a row of floats starting `sh` (0..3) floats into the aligned quad a,
+// continued in the next quad b.
+__device__ __forceinline__ float4 shifted_quad(const float4& a, const float4& b, int sh)
+{
+    float4 r;
+    r.x = sh == 0 ? a.x : sh == 1 ? a.y : sh == 2 ? a.z : a.w;
+    r.y = sh == 0 ? a.y : sh == 1 ? a.z : sh == 2 ? a.w : b.x;
+    r.z = sh == 0 ? a.z : sh == 1 ? a.w : sh == 2 ? b.x : b.y;
+    r.w = sh == 0 ? a.w : sh == 1 ? b.x : sh == 2 ? b.y : b.z;
+    return r;
+}
+
+// k_im2col_rows with four positions per thread, for image rows of a multiple of four elements on both
+// sides (h_in, ho) and a 16-byte aligned x: the four positions are neighbours in one output row, so a
+// member's four values are four consecutive elements of one input row, cut out of one or two aligned
+// quads (the kernel tap shifts them by v - pad_h) and stored as one quad: a quarter of the loads,
+// stores and table reads of the one-position kernel.
+__global__ __launch_bounds__(256) void k_im2col_rows_v4(const float* __restrict__ x, float* __restrict__ col,
+                                                        const int* __restrict__ base, const int* __restrict__ arow,
+                                                        const int* __restrict__ bcol, int g0, int m_total, Groups G,
+                                                        int w_in, int h_in, size_t g_stride)
+{
+    const int g = g0 + blockIdx.z;
+    const int k0 = blockIdx.y * kIm2colMembers;
+    const int k1 = min(G.n_members, k0 + kIm2colMembers);
+    float* colg = col + (size_t)blockIdx.z * g_stride;
+    const float4* x4 = (const float4*)x;
+    const int quads = m_total >> 2;
+    for (int mq = blockIdx.x * 256 + threadIdx.x; mq < quads; mq += gridDim.x * 256) {
+        const int m = mq << 2;
+        const int r0 = arow[m], c0 = bcol[m], b0 = base[m];
+        float4 vals[kIm2colMembers];
+        Member e = member_of(G, g, k0);
+#pragma unroll
+        for (int q = 0; q < kIm2colMembers; q++) {
+            const int r = r0 + e.u, c = c0 + e.v;  // c: column of the first of the four values
+            const int sh = c & 3, ca = c - sh;     // the aligned quads at columns ca and ca + 4 hold them
+            const bool row_ok = k0 + q < k1 && e.ok && r >= 0 && r < w_in;
+            const bool ok_a = row_ok && ca >= 0 && ca < h_in;
+            const bool ok_b = row_ok && sh != 0 && ca + 4 >= 0 && ca + 4 < h_in;
+            const int at = (b0 + (e.ci * w_in + e.u) * h_in + e.v - sh) >> 2;  // quad index of column ca of that row
+            float4 a = x4[ok_a ? at : 0], b = x4[ok_b ? at + 1 : 0];
+            if (!ok_a) a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (!ok_b) b = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            vals[q] = shifted_quad(a, b, sh);
+            next_member(G, e);
+        }
+#pragma unroll
+        for (int q = 0; q < kIm2colMembers; q++)
+            if (k0 + q < k1) *(float4*)(colg + (size_t)(k0 + q) * m_total + m) = vals[q];
+    }
+}
+
 // Weight operands of groups g0 + blockIdx.y:
 //   wcat[g][k][j]: j < c_out -> clamp(w,0,100), j >= c_out -> -clamp(w,-100,0)   (utils_functional.py:611-612)
 //   wd[g][j][k]  : the same with the negative rail negated (it enters dL/dx with a minus sign)
@@ -880,6 +934,58 @@ __global__ __launch_bounds__(256) void k_col2im_rows(const float* __restrict__ d
             }
             dst[e] = g0 == 0 ? s : dst[e] + s;
         }
+    }
+}
+
+// k_col2im_rows with four elements of an input row per thread, for image rows of a multiple of four
+// elements on both sides, kernels of at most eight columns and 16-byte aligned buffers: a tap's four
+// terms are four consecutive elements of one dcol row, cut out of one or two aligned quads.  One
+// grid-stride loop over the quads of all planes.
+__global__ __launch_bounds__(256) void k_col2im_rows_v4(const float* __restrict__ dcol, float* __restrict__ gx, int g0,
+                                                        int ng, long long m_total, int n_planes, Groups G, int w_in,
+                                                        int h_in, int pad_w, int pad_h, int wo, int ho, size_t g_stride)
+{
+    const int plane = w_in * h_in, plane_quads = plane >> 2;
+    const int k_step = (G.mode == GEO_SC_ACC_Z || G.mode == GEO_SC_ACC_FULL) ? G.h_k : 1;
+    const long long total = (long long)n_planes * plane_quads;
+    for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
+        const int nc = (int)(idx / plane_quads), eq = (int)(idx - (long long)nc * plane_quads);
+        const int n = nc / G.c_in, ci = nc - n * G.c_in;
+        float4* dst = (float4*)(gx + (size_t)nc * plane);
+        const float* src = dcol + (size_t)n * wo * ho;
+        const int e = eq << 2;
+        const int p = e / h_in, qq = e - p * h_in;  // the thread's elements are (p, qq .. qq + 3)
+        float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int v = 0; v < G.h_k; v++) {
+            int g, k;
+            group_of(G, ci, 0, v, g, k);
+            if (g < g0 || g >= g0 + ng) continue;
+            const int b = qq + pad_h - v;  // output column of the first element's term
+            const int sh = b & 3, ba = b - sh;
+            const bool ok_a = ba >= 0 && ba < ho, ok_b = sh != 0 && ba + 4 >= 0 && ba + 4 < ho;
+            const float* sg = src + (size_t)(g - g0) * g_stride + (size_t)k * m_total;
+            for (int u = 0; u < G.w_k; u++) {
+                const int a = p + pad_w - u;
+                const bool row_ok = a >= 0 && a < wo;
+                const float4* row = (const float4*)(sg + (size_t)u * k_step * m_total + (row_ok ? a : 0) * ho);
+                float4 qa = row[(row_ok && ok_a) ? ba >> 2 : 0], qb = row[(row_ok && ok_b) ? (ba >> 2) + 1 : 0];
+                if (!(row_ok && ok_a)) qa = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (!(row_ok && ok_b)) qb = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                const float4 t = shifted_quad(qa, qb, sh);
+                s.x += t.x;
+                s.y += t.y;
+                s.z += t.z;
+                s.w += t.w;
+            }
+        }
+        if (g0 != 0) {
+            const float4 o = dst[eq];
+            s.x += o.x;
+            s.y += o.y;
+            s.z += o.z;
+            s.w += o.w;
+        }
+        dst[eq] = s;
     }
 }
 
@@ -1885,6 +1991,10 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     int* pos_bcol = pos_arow + pos_stride;
     float* gt = (float*)(ws + L.off_gt);
     const int m_blocks = grid1d(M);
+    // four elements per thread in im2col / col2im where rows of the input and of the output are whole quads
+    const bool quad_rows = g.h_in % 4 == 0 && g.ho % 4 == 0;
+    const bool im2col_v4 = quad_rows && ((uintptr_t)x & 15) == 0;
+    const bool col2im_v4 = quad_rows && g.h_k <= 8 && gx && ((uintptr_t)gx & 15) == 0;
     hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
                        g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
     const bool wgrad_only = !gx && gw && L.small_k;
@@ -1994,7 +2104,10 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             if (gx && L.dcol_slices > 1)
                 hipLaunchKernelGGL(k_sum_slices, dim3(grid1d((long long)((size_t)nv * L.col_v / 4))), dim3(256), 0, s, dcol,
                                    (size_t)nv * L.col_v, L.dcol_slices, slice);
-            if (gx)
+            if (gx && col2im_v4)
+                hipLaunchKernelGGL(k_col2im_rows_v4, dim3(grid1d((long long)n_planes * (g.w_in * g.h_in / 4))), dim3(256), 0, s, dcol, gx,
+                                   v0, nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
+            else if (gx)
                 hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx,
                                    v0, nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
         }
@@ -2002,9 +2115,16 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     }
     for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
         const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
-        hipLaunchKernelGGL(k_im2col_rows,
-                           dim3(m_blocks > 1024 ? 1024 : m_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
-                           dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, G, g.w_in, g.h_in, L.col_v);
+        if (im2col_v4) {
+            const int q_blocks = grid1d(M / 4);
+            hipLaunchKernelGGL(k_im2col_rows_v4,
+                               dim3(q_blocks > 1024 ? 1024 : q_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
+                               dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, G, g.w_in, g.h_in, L.col_v);
+        } else {
+            hipLaunchKernelGGL(k_im2col_rows,
+                               dim3(m_blocks > 1024 ? 1024 : m_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
+                               dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, G, g.w_in, g.h_in, L.col_v);
+        }
         {
             int wb = grid1d((long long)K * g.c_out);
             hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
@@ -2047,8 +2167,12 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         const int n_planes = g.n * g.c_in;
         const int pb = plane_blocks > 64 ? 64 : plane_blocks;
         const int want = 256 * 16 / pb;  // a few thousand blocks in all
-        hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx, v0,
-                           nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
+        if (col2im_v4)
+            hipLaunchKernelGGL(k_col2im_rows_v4, dim3(grid1d((long long)n_planes * (g.w_in * g.h_in / 4))), dim3(256), 0, s, dcol, gx, v0,
+                               nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
+        else
+            hipLaunchKernelGGL(k_col2im_rows, dim3(n_planes < want ? n_planes : want, pb), dim3(256), 0, s, dcol, gx, v0,
+                               nv, L.m_total, n_planes, G, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho, L.col_v);
     }
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }

@@ -68,6 +68,11 @@ GEMM_CASES = [
     ((4, 24, 10, 10), (20, 24, 2, 2), (0, 0), 3.0),   # K = 48, 40 rails: 64-wide column tiles
     ((4, 11, 20, 20), (16, 11, 3, 3), (1, 1), 2.0),   # K = 33: 1600 positions split over workgroups, a 1-member tail chunk
     ((1, 40, 4, 6), (3, 40, 1, 3), (0, 1), 2.0),      # K = 40 with 24 positions and 6 rails: one partly filled tile, unaligned rails
+    # image rows of whole quads on both sides: the four-position im2col / col2im kernels, taps shifted by -2..2, -3..3
+    ((2, 12, 8, 12), (6, 12, 3, 5), (1, 2), 2.0),
+    ((2, 12, 4, 8), (4, 12, 3, 7), (1, 3), 2.0),
+    ((1, 12, 3, 16), (3, 12, 3, 9), (1, 4), 2.0),     # nine kernel columns: four-position im2col, one-position col2im
+    ((1, 12, 6, 8), (4, 12, 3, 2), (1, 0), 2.0),      # output rows of 7: the one-position kernels
 ]
 
 
