@@ -171,7 +171,7 @@ int forward_impl(const geo_sc_conv_desc* desc, const void* x, const float* w, in
     uint32_t* wgt = (uint32_t*)(ws + g.off_wgt);
     uint32_t* act = (uint32_t*)(ws + g.off_act);
     if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
-    if ((rc = launch_weight_streams(g, w, wgt, tables, s)) != GEO_SC_OK) return rc;
+    if ((rc = launch_weight_streams(g, w, wgt, tables, s, g.rail)) != GEO_SC_OK) return rc;
     if ((rc = launch_rail_pack(g, wgt, s, true)) != GEO_SC_OK) return rc;
     rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)x, act, tables, s)
             : launch_act_streams(g, (const float*)x, act, tables, s);

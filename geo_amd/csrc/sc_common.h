@@ -80,8 +80,10 @@ int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s);
 int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s);
 int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* streams, const uint32_t* tables,
                           hipStream_t s);
+// rail_only: the caller's convolution kernel reads the rail-packed copy only; a generator that writes that
+// copy itself may then leave the two-rail lines unwritten
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
-                          hipStream_t s);
+                          hipStream_t s, bool rail_only = false);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
 // fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.wgt_rail;
 // with from_generator also where launch_weight_streams has written that part itself)

@@ -202,56 +202,70 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __r
     }
 }
 
-// The same streams for kernels that are long in dim 3 (h_k >= 16, e.g. the SC-linear mapping with
-// h_k = 256): a workgroup takes one (c_out tile, member k) and 16 consecutive kernel rows, so that
-// the 16 rows of one output channel are one 64-byte run of w, shared by the workgroup's four waves
-// through the vector cache (4096 x 4096 linear layer: 1.46 GB fetched -> the 67 MB of the tensor).
+// Weight streams of kernels long in dim 3 (the SC linear layer's 1 x 256 rows): a block takes a
+// tile of 16 output channels x 16 OR members x 16 kernel rows.  The weights come in through LDS (w is
+// read in 64-byte runs along the kernel row), then a thread keeps one (channel, member) and walks the
+// 16 rows: the lines of consecutive members are neighbours in the rail-packed copy, so a block writes
+// it in 1 KB runs.  rail_words / rail_fields: the rail-packed copy in the same pass (these tensors are
+// large: a separate pass would read all lines back): [c_out tile][line][channel], the non-zero rail's
+// word and the 16-bit M0 field of the channel's rail.  two_rail = 0 leaves the two-rail lines unwritten
+// (a caller whose convolution kernel reads the rail-packed copy only).
 __global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float* __restrict__ w,
                                                                     uint32_t* __restrict__ streams,
                                                                     const uint32_t* __restrict__ tables, GenParams gp,
                                                                     int c_out, int c_in, int w_k, int h_k, int n_cotile,
                                                                     int v_chunks, uint32_t* __restrict__ rail_words,
                                                                     uint16_t* __restrict__ rail_fields,
-                                                                    size_t rail_lines)
+                                                                    size_t rail_lines, int two_rail)
 {
     extern __shared__ uint32_t lds[];
     load_tables_to_lds(lds, tables, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
+    float* wt = reinterpret_cast<float*>(lds + gp.L + gp.L * gp.wpc);  // [row][member][channel], rows of 17
     const int k_or = c_in * w_k;
+    const int k_chunks = (k_or + 15) / 16;
     const size_t pack_stride = (size_t)h_k * k_or * n_cotile * 2 * kCoTile;
     const float Lf = (float)gp.L, top = (float)(gp.L - 1);
-    const size_t n_blocks = (size_t)v_chunks * k_or * n_cotile;
-    const int co_l = threadIdx.x & 15, v_l = threadIdx.x >> 4;
+    const size_t n_blocks = (size_t)v_chunks * k_chunks * n_cotile;
+    const int co_l = threadIdx.x & 15, k_l = threadIdx.x >> 4;
     for (size_t blk = blockIdx.x; blk < n_blocks; blk += gridDim.x) {
         const int cot = (int)(blk % n_cotile);
         const size_t r = blk / n_cotile;
-        const int k = (int)(r % k_or);
-        const int v = (int)(r / k_or) * 16 + v_l;
-        const int co = cot * kCoTile + co_l;
-        const int ci = k / w_k, u = k % w_k;
-        if (v >= h_k) continue;
-        int cp = 0, cn = 0;
-        if (co < c_out) {
-            const float t = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v] * Lf;
-            cp = (int)ceilf(fminf(fmaxf(t, 0.0f), top));
-            cn = (int)ceilf(-fminf(fmaxf(t, -top), 0.0f));
+        const int k0 = (int)(r % k_chunks) * 16, v0 = (int)(r / k_chunks) * 16;
+        __syncthreads();  // the previous tile has been read
+        // element e = (channel e / 256, member (e / 16) % 16, row e % 16): 16 consecutive threads read 64 bytes
+#pragma unroll 4
+        for (int i = 0; i < 16; i++) {
+            const int vl = threadIdx.x & 15, kl = threadIdx.x >> 4;
+            const int co = cot * kCoTile + i, k = k0 + kl, v = v0 + vl;
+            const bool ok = co < c_out && k < k_or && v < h_k;
+            const float val = w[ok ? ((size_t)co * k_or + k) * h_k + v : 0];
+            wt[(vl * 16 + kl) * 17 + i] = ok ? val : 0.0f;
         }
+        __syncthreads();
+        const int k = k0 + k_l;
+        if (k >= k_or) continue;
         const int op = (int)posp1[(67 + k) % (gp.L - 1)];
         const int on = (int)posp1[(37 + k) % (gp.L - 1)];
-        const size_t base = (((size_t)v * k_or + k) * n_cotile + cot) * (2 * kCoTile) + co_l;
-        for (int pk = 0; pk < gp.packs; pk++) {
-            const uint32_t wp = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
-            const uint32_t wn = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
-            streams[pk * pack_stride + base] = wp;
-            streams[pk * pack_stride + base + kCoTile] = wn;
-            if (rail_words) {
-                // the rail-packed copy in the same pass (these tensors are large: a separate pass
-                // would read all lines back): [c_out tile][line][channel], the non-zero rail's word
-                // and the 16-bit M0 field of the channel's rail
-                const size_t dst = ((size_t)cot * rail_lines + ((size_t)pk * h_k + v) * k_or + k) * kCoTile + co_l;
-                rail_words[dst] = wp | wn;
-                rail_fields[dst] = (uint16_t)(0xC000u | ((cn ? 2u * kCoTile : 0u) + 2u * co_l));
+        for (int vl = 0; vl < 16 && v0 + vl < h_k; vl++) {
+            const int v = v0 + vl;
+            const float t = wt[(vl * 16 + k_l) * 17 + co_l] * Lf;
+            const int cp = (int)ceilf(fminf(fmaxf(t, 0.0f), top));
+            const int cn = (int)ceilf(-fminf(fmaxf(t, -top), 0.0f));
+            const size_t base = (((size_t)v * k_or + k) * n_cotile + cot) * (2 * kCoTile) + co_l;
+            for (int pk = 0; pk < gp.packs; pk++) {
+                const uint32_t wp = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
+                const uint32_t wn = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+                if (two_rail) {
+                    streams[pk * pack_stride + base] = wp;
+                    streams[pk * pack_stride + base + kCoTile] = wn;
+                }
+                if (rail_words) {
+                    const size_t dst = ((size_t)cot * rail_lines + ((size_t)pk * h_k + v) * k_or + k) * kCoTile + co_l;
+                    rail_words[dst] = wp | wn;
+                    rail_fields[dst] = (uint16_t)(0xC000u | ((cn ? 2u * kCoTile : 0u) + 2u * co_l));
+                }
             }
         }
     }
@@ -558,7 +572,7 @@ int launch_act_streams_q7(const Geometry& g, const uint8_t* x, uint32_t* streams
 }
 
 int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
-                          hipStream_t s)
+                          hipStream_t s, bool rail_only)
 {
     if (g.generator != GEO_SC_GEN_LFSR) {
         const size_t n_el = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
@@ -576,13 +590,15 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     if (weight_rows_generator(g)) {
-        const int v_chunks = (g.h_k + 15) / 16;
-        const size_t n_blocks = (size_t)v_chunks * g.k_or * g.n_cotile;
-        hipLaunchKernelGGL(k_weight_streams_rows, dim3((unsigned)(n_blocks > 256 * 8 ? 256 * 8 : n_blocks)),
-                           dim3(kGenThreads), table_bytes(g.L), s, w, streams, tables, gp, g.c_out, g.c_in, g.w_k,
-                           g.h_k, g.n_cotile, v_chunks, g.wgt_rail ? streams + g.wgt_rail_off : nullptr,
+        const int v_chunks = (g.h_k + 15) / 16, k_chunks = (g.k_or + 15) / 16;
+        const size_t n_blocks = (size_t)v_chunks * k_chunks * g.n_cotile;
+        const bool two_rail = !(rail_only && g.wgt_rail);
+        hipLaunchKernelGGL(k_weight_streams_rows, dim3((unsigned)(n_blocks > 256 * 16 ? 256 * 16 : n_blocks)),
+                           dim3(kGenThreads), table_bytes(g.L) + 16 * 16 * 17 * sizeof(float), s, w, streams, tables, gp,
+                           g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile, v_chunks,
+                           g.wgt_rail ? streams + g.wgt_rail_off : nullptr,
                            g.wgt_rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
-                           g.wgt_rail_lines);
+                           g.wgt_rail_lines, two_rail ? 1 : 0);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
