@@ -264,13 +264,13 @@ def test_backward_in_several_rounds_of_add_groups(capi, monkeypatch, shape_x, sh
 
 
 # ------------------------------------------------------------------ full sizes
-def _fp64_reference_on_gpu(x, w, g, pad):
+def _fp64_reference_on_gpu(x, w, g, pad, mode="y", z_unit=1):
     """float64 autograd over the restated surrogate, evaluated on the GPU (the CPU would take minutes)."""
     from oracle import surrogate
     xr = x.cuda().double().requires_grad_(True)
     wr = w.cuda().double().requires_grad_(True)
     xp = torch.nn.functional.pad(xr, (pad, pad, pad, pad))
-    p, n = surrogate.surrogate_rails(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)))
+    p, n = surrogate.surrogate_rails(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)), mode, z_unit)
     (p - n).backward(g.cuda().double())
     return xr.grad, wr.grad
 
@@ -292,7 +292,7 @@ def test_backward_resnet_shape_full_size(capi):
 
 def test_backward_linear_4096_shape(capi):
     """The 4096 -> 4096 SC linear layer through its conv mapping (N, 16, 1, 256) * (4096, 16, 1, 256): 256
-    add groups of 16 members, 8192 rails (the fused small-group kernel, one launch per 256 rails); batch 64
+    add groups of 16 members, 8192 rails (the fused small-group kernel, 32 column blocks of 256 rails); batch 64
     of the 1024 so that the float64 reference stays small."""
     x, w, pad, _ = wl.named("C4", "q7")
     x = x[:64].contiguous()
@@ -304,3 +304,21 @@ def test_backward_linear_4096_shape(capi):
     print(f"C4 backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
     assert ex <= RTOL and ew <= RTOL, (ex, ew)
     assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
+
+
+@pytest.mark.parametrize("mode,zu", [("z", 1), ("yz", 4), ("yz", 8)])
+def test_backward_small_groups_at_the_headline_shape(capi, mode, zu):
+    """128->128 3x3 at 16x16 with z accumulation (128 groups of 9 members) and yz accumulation with 4 and 8
+    channels per group (96 groups of 12, 48 of 24): the fused small-group kernels (bf16 matrix cores up to 16
+    members, fp32 beyond) at a batch of 64 of the 256, against float64 autograd on the GPU."""
+    x, w, pad, _ = wl.named("C3", "q7")
+    x = x[:64].contiguous()
+    w = (w * 8).contiguous()
+    g = torch.randn((64, 128, 16, 16), generator=torch.Generator().manual_seed(7))
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad), accumulate=mode, z_unit=zu)
+    rx, rw = _fp64_reference_on_gpu(x, w, g, pad, mode, zu)
+    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
+    print(f"{mode} z_unit {zu} backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
+    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    gx2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad), accumulate=mode, z_unit=zu)
+    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)   # deterministic
