@@ -70,6 +70,13 @@ struct GemmParams {
     // EPI_EXP_TIMES_G: c[i][j] = g[i * c_out + (j % c_out)] * exp(-acc), g = upstream gradient stored [m][c_out]
     const float* __restrict__ g;
     int c_out, npos;
+    // A as a view of the shifted input planes instead of a materialised col (kernels with VA): row r of
+    // batch member z starts a_rows[z * a_rows_batch + r] elements into `a`, and position m of that row lies
+    // m + (m / a_item) * a_skip elements further (a_item positions per item, a_skip elements between the
+    // items' runs); lda and a_batch_stride are not used.
+    const long long* __restrict__ a_rows;
+    long long a_rows_batch;
+    int a_item, a_skip;
     // tile extent per workgroup in i and j: kTile, or kTile / 2 in at most one of them (set by
     // launch_gemm): the four waves then line up along the other dimension
     int tile_i, tile_j;
@@ -428,9 +435,108 @@ struct SplitStager {
     }
 };
 
+// The same stager for an A operand that is a view of the shifted input planes (GemmParams::a_rows): the
+// rows start where a table says, and the positions of one item are a_skip elements away from the next
+// item's.  As the K-major operand of the first product the positions are the rows' elements (a lane keeps
+// its own position, shifted once); as the I-major operand of the weight-gradient product they are the k
+// dimension: a thread's eight positions and a whole chunk lie inside one item (a_item is a multiple of
+// kChunk), and the pointer jumps by a_skip when it passes an item's end.
+template <bool KMAJOR>
+struct ViewStager {
+    const float* base;
+    const long long* rows;  // K-major: the table of this batch member (uniform)
+    const float* p;         // I-major: this thread's first element
+    int off;                // K-major: this thread's element of every row
+    int kr;                 // K-major: first row of this thread's half of the current chunk
+    int in_item, item, skip;
+    int half, ii;
+
+    __device__ __forceinline__ void init(const GemmParams& q, int batch, int i0, int k_begin, int I, int wave)
+    {
+        const int t = threadIdx.x;
+        base = q.a;
+        rows = q.a_rows + batch * q.a_rows_batch;
+        item = q.a_item;
+        skip = q.a_skip;
+        if (KMAJOR) {
+            half = wave >> 1;
+            ii = t & 127;
+            const int m = min(i0 + ii, I - 1);
+            off = m + (m / item) * skip;
+            kr = k_begin + 8 * half;
+        } else {
+            ii = t >> 1;
+            half = t & 1;
+            const int m = k_begin + 8 * half;
+            in_item = m % item;
+            p = base + rows[min(i0 + ii, I - 1)] + m + (long long)(m / item) * skip;
+        }
+    }
+    __device__ __forceinline__ void advance()
+    {
+        if (KMAJOR) {
+            kr += kChunk;
+        } else {
+            p += kChunk;
+            in_item += kChunk;
+            if (in_item >= item) {
+                in_item -= item;
+                p += skip;
+            }
+        }
+    }
+    __device__ __forceinline__ void fetch_whole(float (&r)[8])
+    {
+        if (KMAJOR) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = (base + rows[kr + c])[off];
+        } else {
+            const float4 v0 = *(const float4*)p, v1 = *(const float4*)(p + 4);
+            r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+            r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+        }
+        advance();
+    }
+    __device__ __forceinline__ void fetch(float (&r)[8], int k_left)
+    {
+        const bool tail = k_left < kChunk;
+        if (KMAJOR) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                // rows past the end of a partial chunk read the chunk's first row instead
+                const int row = (tail && 8 * half + c >= k_left) ? kr - 8 * half : kr + c;
+                r[c] = (base + rows[row])[off];
+            }
+        } else {
+            if (!tail) {
+                const float4 v0 = *(const float4*)p, v1 = *(const float4*)(p + 4);
+                r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+                r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; c++) r[c] = p[8 * half + c < k_left ? c : -8 * half];
+            }
+        }
+        advance();
+    }
+    __device__ __forceinline__ void commit(uint4 (*s)[2][kLdx], float (&r)[8], int k_left) const
+    {
+        if (k_left < kChunk) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = 8 * half + c < k_left ? r[c] : 0.0f;
+        }
+        unsigned hi[4], mid[4], lo[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) split3(r[2 * c], r[2 * c + 1], hi[c], mid[c], lo[c]);
+        s[0][half][ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        s[1][half][ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        s[2][half][ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    }
+};
+
 // v_mfma_f32_32x32x16_bf16: lane l feeds A[i = l%32][k = 8 (l/32) .. + 7] and B[those k][j = l%32]:
 // the 16 bytes at s[term][l/32][i]; results as in the fp32 instruction.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int NX, int NY>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int NX, int NY, bool VA>
 __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)[3][2][kLdx], uint4 (*bs)[3][2][kLdx],
                                                 int i0, int j0, int batch, int split, int k_begin, int k_end, int wi,
                                                 int wj, int l32, int lk, int wave)
@@ -443,9 +549,12 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
 
-    SplitStager<A_KMAJOR> sa;
+    typename std::conditional<VA, ViewStager<A_KMAJOR>, SplitStager<A_KMAJOR>>::type sa;
     SplitStager<B_KMAJOR> sb;
-    sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
+    if constexpr (VA)
+        sa.init(q, batch, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
+    else
+        sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
     sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
     // Two chunks ahead: while chunk c is multiplied out of LDS, chunk c + 1 sits in one register set
     // (its loads issued a whole trip ago) and the loads of chunk c + 2 go out into the other.
@@ -581,7 +690,7 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
 }
 
 // Operands with 16-byte aligned rows and chunks (launch_gemm checks).
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VA = false>
 // three waves per SIMD (at most 168 registers; three workgroups' LDS fit a CU)
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void k_gemm_split(GemmParams q)
 {
@@ -602,7 +711,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const bool y0 = j0 + wj < q.J, y1 = !narrow_i && j0 + wj + 32 < q.J;
     const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
 #define GEO_SC_GEMM_WAVE(NX, NY)                                                                                        \
-    gemm_wave_split<A_KMAJOR, B_KMAJOR, EPI, NX, NY>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk, wave)
+    gemm_wave_split<A_KMAJOR, B_KMAJOR, EPI, NX, NY, VA>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk, wave)
     switch (blocks_xy) {
     case 3: GEO_SC_GEMM_WAVE(2, 2); break;
     case 2: GEO_SC_GEMM_WAVE(2, 1); break;
@@ -820,6 +929,52 @@ __global__ __launch_bounds__(256) void k_im2col_rows_v4(const float* __restrict_
 #pragma unroll
         for (int q = 0; q < kIm2colMembers; q++)
             if (k0 + q < k1) *(float4*)(colg + (size_t)(k0 + q) * m_total + m) = vals[q];
+    }
+}
+
+// The input as col without the copies: planes xs[v][ci][n][r][b] = x~[n, ci, r, b + v] over the padded
+// rows r (w_in + 2 pad_w of them) and the output columns b, one per kernel column v and channel.  Member
+// (ci, u, v) at position m = (n, a, b) is xs[v][ci][n][a + u][b]: row (ci, u) of col for kernel column v is
+// the plane (v, ci) read from u * ho elements in, with the positions of item n shifted by
+// n * (w_k - 1) * ho -- a third of col's bytes for a 3-wide kernel, and the rows of one channel share
+// their cache lines.  Four columns per thread (ho and h_in multiples of four, 16-byte aligned x), as in
+// k_im2col_rows_v4.  `total` quads; the (w_k - 1) * ho elements behind the last plane are never read.
+__global__ __launch_bounds__(256) void k_shift_planes(const float* __restrict__ x, float* __restrict__ xs, long long total,
+                                                      int n_items, int c_in, int w_in, int h_in, int pad_w, int pad_h,
+                                                      int ho)
+{
+    const int wp = w_in + 2 * pad_w, hq = ho >> 2;
+    const float4* x4 = (const float4*)x;
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)gridDim.x * 256) {
+        // e = (((v * c_in + ci) * n_items + n) * wp + r) * hq + quad
+        long long t = e;
+        const int bq = (int)(t % hq);
+        t /= hq;
+        const int r = (int)(t % wp);
+        t /= wp;
+        const int n = (int)(t % n_items);
+        t /= n_items;
+        const int ci = (int)(t % c_in), v = (int)(t / c_in);
+        const int row = r - pad_w, c = 4 * bq + v - pad_h;  // input row, and input column of the first of the four
+        const int sh = c & 3, ca = c - sh;
+        const bool row_ok = row >= 0 && row < w_in;
+        const bool ok_a = row_ok && ca >= 0 && ca < h_in, ok_b = row_ok && sh != 0 && ca + 4 >= 0 && ca + 4 < h_in;
+        const long long at = ((((long long)n * c_in + ci) * w_in + row) * h_in + ca) >> 2;
+        float4 a = x4[ok_a ? at : 0], b = x4[ok_b ? at + 1 : 0];
+        if (!ok_a) a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (!ok_b) b = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        ((float4*)xs)[e] = shifted_quad(a, b, sh);
+    }
+}
+
+// rows[g - g0][k]: where row k of group g's col starts in the planes of k_shift_planes (elements).
+__global__ __launch_bounds__(256) void k_view_rows(long long* __restrict__ rows, int g0, int ng, Groups G, long long plane,
+                                                   int ho, int k_pad)
+{
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < ng * k_pad; e += gridDim.x * 256) {
+        const int gi = e / k_pad, k = e - gi * k_pad;
+        const Member mb = member_of(G, g0 + gi, k < G.n_members ? k : G.n_members - 1);
+        rows[e] = ((long long)mb.v * G.c_in + mb.ci) * plane + (long long)mb.u * ho;
     }
 }
 
@@ -1813,7 +1968,9 @@ int grid1d(long long total)
     return (int)(blocks < 1 ? 1 : blocks);
 }
 
-template <bool AK, bool BK, int EPI>
+// VA: the A operand is a view of the shifted input planes (GemmParams::a_rows); the caller has checked that
+// its rows and chunks are 16-byte aligned.
+template <bool AK, bool BK, int EPI, bool VA = false>
 int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
 {
     GemmParams q = q0;
@@ -1844,9 +2001,12 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
     auto rows_aligned = [&](const float* base, long long ld, long long batch_stride) {
         return ld % 4 == 0 && ((uintptr_t)base & 15) == 0 && batch_stride % 4 == 0 && q.k_per_split % 4 == 0;
     };
-    const bool a_vec = AK || rows_aligned(q.a, q.lda, q.a_batch_stride);
+    const bool a_vec = VA || AK || rows_aligned(q.a, q.lda, q.a_batch_stride);
     const bool b_vec = BK || rows_aligned(q.b, q.ldb, q.b_batch_stride);
-    if constexpr (AK && BK) {
+    if constexpr (VA) {
+        if (!b_vec) return GEO_SC_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
+    } else if constexpr (AK && BK) {
         hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI>), grid, dim3(256), 0, s, q);
     } else {
         if (a_vec && b_vec)
@@ -1872,9 +2032,19 @@ struct BwdLayout {
     int gt_blocks;       // 32-column blocks of those tiles
     int rows_per_chunk;  // add groups processed by one round of launches
     int dcol_slices;     // partial dcol arrays per round (column blocks of the fused kernel), rows_per_chunk * col_v apart
+    bool view_col;       // the GEMMs read col as a view of the shifted input planes (k_shift_planes) kept in col's space
+    int view_k_pad;      // entries per group of the view's row table
+    size_t off_rows;     // the row table
     size_t col_v, e_v, part_v, w_v;  // floats per add group of each scratch array
     size_t off_col, off_e, off_dcol, off_part, off_wcat, off_wd, off_pos, off_gt, bytes;
 };
+
+// floats of the shifted input planes (one per kernel column and channel, over the padded rows and the
+// output columns) including the run behind the last plane that a shifted row may touch
+size_t view_floats(const Geometry& g)
+{
+    return (size_t)g.h_k * g.c_in * g.n * (g.w_in + 2 * g.pad_w) * g.ho + (size_t)g.w_k * g.ho;
+}
 
 BwdLayout bwd_layout(const Geometry& g)
 {
@@ -1945,6 +2115,14 @@ BwdLayout bwd_layout(const Geometry& g)
     if (rows * b.splits > 65535) rows = 65535 / b.splits;  // grid.z = rows * splits
     if (rows < 1) rows = 1;
     b.rows_per_chunk = (int)rows;
+    // col as a view: whole quads in every row on both sides, chunks of kChunk positions inside one item, an
+    // even number of rails' worth of columns (16-byte aligned rows of E), every group in one round, members
+    // that all exist, and offsets that fit the stagers' 32-bit position index
+    b.view_k_pad = (K + kChunk - 1) / kChunk * kChunk;
+    b.view_col = !b.fused_k && g.ho % 4 == 0 && g.h_in % 4 == 0 && (g.wo * g.ho) % kChunk == 0 && g.c_out % 2 == 0 &&
+                 rows == (size_t)b.G.n_groups && !(g.mode == GEO_SC_ACC_YZ && g.c_in % g.z_unit != 0) &&
+                 view_floats(g) <= rows * col_alloc &&
+                 (long long)g.n * (g.w_in + 2 * g.pad_w) * g.ho + (long long)g.w_k * g.ho < 0x7fffffffLL;
     size_t o = 0;
     b.off_col = o;  o += align256(sizeof(float) * rows * col_alloc);
     b.off_e = o;    o += align256(sizeof(float) * rows * e_alloc);
@@ -1960,6 +2138,8 @@ BwdLayout bwd_layout(const Geometry& g)
         b.off_gt = o;
         o += align256(sizeof(float) * (b.fused_k && tiled > plain ? tiled : plain));
     }
+    b.off_rows = o;
+    o += align256(sizeof(long long) * (size_t)b.G.n_groups * b.view_k_pad);
     b.bytes = o;
     return b;
 }
@@ -2113,9 +2293,22 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         }
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
+    // col as a view of the shifted input planes (one round holds every group then)
+    const bool view = L.view_col && ((uintptr_t)x & 15) == 0;
+    long long* view_rows = (long long*)(ws + L.off_rows);
+    if (view) {
+        const long long plane = (long long)g.n * (g.w_in + 2 * g.pad_w) * g.ho;
+        const long long quads = (long long)g.h_k * g.c_in * plane / 4;
+        hipLaunchKernelGGL(k_shift_planes, dim3(grid1d(quads)), dim3(256), 0, s, x, col, quads, g.n, g.c_in, g.w_in, g.h_in,
+                           g.pad_w, g.pad_h, g.ho);
+        hipLaunchKernelGGL(k_view_rows, dim3(grid1d((long long)G.n_groups * L.view_k_pad)), dim3(256), 0, s, view_rows, 0,
+                           G.n_groups, G, plane, g.ho, L.view_k_pad);
+    }
     for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
         const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
-        if (im2col_v4) {
+        if (view) {
+            // nothing to copy
+        } else if (im2col_v4) {
             const int q_blocks = grid1d(M / 4);
             hipLaunchKernelGGL(k_im2col_rows_v4,
                                dim3(q_blocks > 1024 ? 1024 : q_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
@@ -2139,7 +2332,10 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         q1.a_batch_stride = (long long)L.col_v; q1.b_batch_stride = (long long)L.w_v;
         q1.c_batch_stride = (long long)L.e_v;
         q1.g = gt; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
-        if ((rc = launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, nv, s)) != GEO_SC_OK) return rc;
+        q1.a_rows = view_rows; q1.a_rows_batch = L.view_k_pad; q1.a_item = g.wo * g.ho; q1.a_skip = (g.w_k - 1) * g.ho;
+        rc = view ? launch_gemm<true, true, EPI_EXP_TIMES_G, true>(q1, nv, s)
+                  : launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, nv, s);
+        if (rc != GEO_SC_OK) return rc;
         if (gw) {
             // partial Gw[v][s][k][j] = sum_{m in split s} col_v[k][m] * E_v[m][j]
             GemmParams q2 = {};
@@ -2149,7 +2345,9 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             q2.splits = L.splits; q2.k_per_split = L.m_per_split; q2.c_split_stride = (long long)K * J;
             q2.a_batch_stride = (long long)L.col_v; q2.b_batch_stride = (long long)L.e_v;
             q2.c_batch_stride = (long long)L.part_v;
-            if ((rc = launch_gemm<false, true, EPI_STORE>(q2, nv, s)) != GEO_SC_OK) return rc;
+            q2.a_rows = view_rows; q2.a_rows_batch = L.view_k_pad; q2.a_item = g.wo * g.ho; q2.a_skip = (g.w_k - 1) * g.ho;
+            rc = view ? launch_gemm<false, true, EPI_STORE, true>(q2, nv, s) : launch_gemm<false, true, EPI_STORE>(q2, nv, s);
+            if (rc != GEO_SC_OK) return rc;
             hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
                                L.splits, g.c_out, G, L.part_v);
         }

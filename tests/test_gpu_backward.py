@@ -195,6 +195,35 @@ def test_weight_gradient_of_small_or_groups(capi, shape_x, shape_w, pad, mode, z
 
 
 @pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu", [
+    # more than 32 members per group (the GEMMs) with image rows of whole quads and items of a multiple of 16
+    # positions: col is read as a view of the shifted input planes, in every accumulation mode
+    ((2, 24, 8, 8), (6, 24, 3, 3), (1, 1), "yz", 12),    # 36 members, 2 channel blocks x 3 rows
+    ((2, 3, 8, 8), (4, 3, 7, 7), (3, 3), "z", 1),        # z mode with a 7 x 7 kernel: 49 members
+    ((2, 4, 8, 8), (6, 4, 3, 3), (1, 1), "full", 1),     # one group of 36 members
+    ((3, 12, 8, 8), (8, 12, 3, 3), (1, 1), "y", 1),      # y mode, 36 members: 2 whole chunks and 4 members
+    ((2, 12, 12, 8), (5, 12, 3, 3), (1, 1), "y", 1),     # odd number of output channels: the materialised col
+])
+def test_backward_through_the_gemms_in_every_mode(capi, shape_x, shape_w, pad, mode, zu):
+    from oracle import surrogate
+    x, w = wl.make_inputs(shape_x, shape_w, "kaiming", seed=shape_x[1] + shape_w[0])
+    w = (w * 2).contiguous()
+    w.view(-1)[::5] = 0.0
+    d = capi.make_desc(x.shape, w.shape, 64, pad)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(6))
+    kw = dict(accumulate=mode, z_unit=zu)
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
+    torch.cuda.synchronize()
+    rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
+    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
+    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    # an input that does not start on a 16-byte boundary takes the materialised col: same bits
+    xo = torch.empty(x.numel() + 1, device="cuda")[1:].view(x.shape)
+    xo.copy_(x)
+    gx2, gw2 = capi.conv2d_add_partial_backward(xo, w.cuda(), g.cuda(), 64, pad, **kw)
+    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)
+
+
+@pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu", [
     ((3, 5, 9, 7), (140, 5, 3, 3), (1, 1), "z", 1),      # 9 members; 280 rails: two column launches, the second adds
     ((2, 4, 8, 8), (70, 4, 5, 5), (2, 2), "z", 1),       # 25 members, 140 rails in one launch
     ((2, 20, 6, 6), (12, 20, 3, 3), (1, 1), "yz", 8),    # 24 members, ragged last channel block
