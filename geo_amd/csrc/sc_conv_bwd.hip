@@ -1256,133 +1256,6 @@ __global__ __launch_bounds__(256) void k_sum_slices(float* __restrict__ a, size_
     }
 }
 
-// Weight gradient of layers with small OR groups (K <= 16 members, 2 * c_out <= 128: first layers,
-// 3 -> 32 channels with 5 x 5 kernels has K = 15) when no input gradient is asked for.  Per tile of
-// 64 output positions the workgroup gathers the im2col columns into LDS, forms Z = col^T wcat with
-// MFMAs, turns it into E = g exp(-Z) in LDS and accumulates Gw += col E in MFMA accumulators that
-// stay live over all tiles of the workgroup; neither col nor E reach memory (at K = 15 they are
-// 80 MB and 335 MB per call).  A workgroup handles tiles s, s + S, ... of group g0 + blockIdx.y
-// and writes one partial sum part[g][s][k][j] for the common split reduction.
-constexpr int kSmallK = 16;
-constexpr int kSmallTile = 64;
-// JB: 32-wide column blocks of the result (ceil(2 * c_out / 32), 1..4), a template parameter so
-// that the MFMAs on the long-lived accumulators are unconditional.
-template <int JB>
-__global__ __launch_bounds__(256) void k_wgrad_small_k(const float* __restrict__ x, const float* __restrict__ wcat,
-                                                       const float* __restrict__ gt, const int* __restrict__ base,
-                                                       const int* __restrict__ arow, const int* __restrict__ bcol,
-                                                       float* __restrict__ part, Groups G, int g0, int M, int w_in,
-                                                       int h_in, int c_out, int splits, size_t w_stride,
-                                                       size_t part_stride)
-{
-    constexpr int NB1 = JB <= 2 ? 1 : 2;  // column blocks of the first product per wave
-    __shared__ __attribute__((aligned(16))) float cs[kSmallK][kSmallTile + 4];  // col tile [k][m]
-    __shared__ __attribute__((aligned(16))) float ws[kSmallK][JB * 32 + 4];      // wcat [k][j], zero padded
-    __shared__ __attribute__((aligned(16))) float es[kSmallTile][JB * 32 + 4];   // E tile [m][j]
-    const int K = G.n_members, J = 2 * c_out;
-    const int g = g0 + blockIdx.y;
-    // the wave index as a scalar: everything derived from it (member indices, which MFMA blocks
-    // exist) stays wave-uniform, so no divergent branches are generated around loads and MFMAs
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int l32 = lane & 31, lk = lane >> 5;
-    // first product: 64 positions x JB column blocks; wave w takes row half w / 2 and column
-    // block(s) w % 2 (JB <= 2) or 2 (w % 2), 2 (w % 2) + 1 (JB > 2)
-    const int i0 = (wave >> 1) * 32;
-    const int cb0 = NB1 == 1 ? (wave & 1) : (wave & 1) * 2;
-
-    const float* wg = wcat + (size_t)blockIdx.y * w_stride;
-    for (int e = threadIdx.x; e < kSmallK * JB * 32; e += 256) {
-        const int k = e / (JB * 32), j = e - k * (JB * 32);
-        ws[k][j] = (k < K && j < J) ? wg[(size_t)k * J + j] : 0.0f;
-    }
-    floatx16 gw_acc[JB];
-#pragma unroll
-    for (int y = 0; y < JB; y++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) gw_acc[y][r] = 0.0f;
-
-    const int n_tiles = (M + kSmallTile - 1) / kSmallTile;
-    for (int tile = blockIdx.x; tile < n_tiles; tile += splits) {
-        const int m0 = tile * kSmallTile;
-        __syncthreads();  // the previous tile's second product has read cs and es
-        {
-            // im2col gather: thread -> position m0 + (t & 63), members wave, wave + 4, wave + 8, wave + 12.
-            // Loads without branches: lanes outside the image read x[0] and are zeroed by a select.
-            const int ml = threadIdx.x & 63;
-            const bool m_ok = m0 + ml < M;
-            const int mc = m_ok ? m0 + ml : 0;
-            const int r0 = arow[mc], c0 = bcol[mc], b0 = base[mc];
-            float vals[4];
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                const int k = wave + 4 * q4;
-                const Member mb = member_of(G, g, k < K ? k : 0);
-                const int rr = r0 + mb.u, cc = c0 + mb.v;
-                const bool ok = m_ok && k < K && mb.ok && cc >= 0 && cc < h_in && rr >= 0 && rr < w_in;
-                const float v = x[ok ? b0 + (mb.ci * w_in + mb.u) * h_in + mb.v : 0];
-                vals[q4] = ok ? v : 0.0f;
-            }
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) cs[wave + 4 * q4][ml] = vals[q4];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int y = 0; y < NB1; y++) {
-            const int cb = cb0 + y;
-            if (cb < JB) {  // wave-uniform
-                // Z[m][j] = sum_k col[k][m] * wcat[k][j] for one 32 x 32 block
-                floatx16 z;
-#pragma unroll
-                for (int r = 0; r < 16; r++) z[r] = 0.0f;
-#pragma unroll
-                for (int kk = 0; kk < kSmallK; kk += 2)
-                    z = __builtin_amdgcn_mfma_f32_32x32x2f32(cs[kk + lk][i0 + l32], ws[kk + lk][cb * 32 + l32], z, 0, 0, 0);
-                // E[m][j] = g[m][co] * exp(-Z), zero outside the problem; loads of g first, no branches
-                const int j = cb * 32 + l32;
-                const int co = j >= c_out ? j - c_out : j;
-                const bool j_ok = j < J;
-                float gv[16];
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int m = m0 + i0 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                    gv[r] = gt[(m < M && j_ok) ? (long long)m * c_out + co : 0];
-                }
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int i = i0 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                    es[i][j] = (m0 + i < M && j_ok) ? gv[r] * exp_neg(z[r]) : 0.0f;
-                }
-            }
-        }
-        __syncthreads();
-        // Gw[k][j] += sum_m col[k][m] * E[m][j]: wave w takes positions 16 w .. 16 w + 15 of the tile
-        const int mw = wave * 16;
-#pragma unroll
-        for (int mm = 0; mm < 16; mm += 2) {
-            const float a = l32 < kSmallK ? cs[l32][mw + mm + lk] : 0.0f;
-#pragma unroll
-            for (int y = 0; y < JB; y++)
-                gw_acc[y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, es[mw + mm + lk][32 * y + l32], gw_acc[y], 0, 0, 0);
-        }
-    }
-    // sum the four waves' accumulators in wave order through LDS (cs/es are free after a barrier)
-    __syncthreads();
-    float (*red)[kSmallK][JB * 32 + 4] = reinterpret_cast<float (*)[kSmallK][JB * 32 + 4]>(&es[0][0]);  // 4 x 16 rows of es
-#pragma unroll
-    for (int y = 0; y < JB; y++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int k = 8 * (r >> 2) + 4 * lk + (r & 3);
-            if (k < kSmallK) red[wave][k][32 * y + l32] = gw_acc[y][r];
-        }
-    __syncthreads();
-    float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)blockIdx.x * K * J;
-    for (int e = threadIdx.x; e < K * J; e += 256) {
-        const int k = e / J, j = e - k * J;
-        pg[e] = ((red[0][k][j] + red[1][k][j]) + red[2][k][j]) + red[3][k][j];
-    }
-}
-
 // Whole backward of layers with small OR groups (K <= 32 members: z accumulation has K = W * H,
 // yz with small channel blocks K = z_unit * W, the SC linear layer K = 16) in one kernel.  With few
 // members per group the general path's scratch array E[g][m][j] is c_in (z) times larger than the
@@ -1689,20 +1562,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
 constexpr int kBfEw = 18;  // words per row of E^T: 32 bf16 and padding
 constexpr int kBfCw = 20;  // words per row of col[k][m]: 16-byte aligned rows
 
-template <bool DX>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k_bwd_small_k_bf16(
+template <int NW, bool DX>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4))) void k_bwd_small_k_bf16(
     const float* __restrict__ x, const float* __restrict__ wcat, const float* __restrict__ gtt,
     const int* __restrict__ base, const int* __restrict__ arow, const int* __restrict__ bcol, float* __restrict__ part,
     float* __restrict__ dcol, Groups G, int g0, int M, int w_in, int h_in, int c_out, int jblocks, int splits,
     int store_part, int gt_blocks, int gt_dedupe, size_t w_stride, size_t part_stride, size_t dcol_stride,
     size_t dcol_slice)
 {
-    constexpr int KP = 16, TM = kFusedTile, JW = 256, EW = kBfEw, CW = kBfCw, NT = 512;
+    constexpr int KP = 16, TM = kFusedTile, JW = 32 * NW, EW = kBfEw, CW = kBfCw, NT = 64 * NW;
+    constexpr int JPARTS = NW / 2;   // waves that share one 16 x 16 block of dcol and split j
+    constexpr int GP = 256 / NT > 1 ? 256 / NT : 1;  // member pairs gathered per thread (256 (position, pair) slots)
     // col of two tiles in turn: the next tile's is written while this tile's products run
     __shared__ __attribute__((aligned(16))) uint4 csz[2][3][2][TM];      // first product: (term, k half, m) -> 8 bf16 along k
     __shared__ __attribute__((aligned(16))) unsigned csg[2][3][KP][CW];  // weight gradient: [term][k][m], two m per word
     __shared__ __attribute__((aligned(16))) unsigned est[3][JW][EW];  // E^T: [term][j][m], two m per word
-    __shared__ float red[3][2][16][17];                               // the other j quarters' partial dcol blocks
+    __shared__ float red[JPARTS > 1 ? JPARTS - 1 : 1][2][16][17];     // the other j parts' partial dcol blocks
     const int K = G.n_members, J = 2 * c_out;
     const int g = g0 + blockIdx.y;
     const int split = blockIdx.x / jblocks, jblock = blockIdx.x - split * jblocks;
@@ -1738,10 +1613,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k
         wz[1] = __builtin_bit_cast(bf16x8, make_uint4(m[0], m[1], m[2], m[3]));
         wz[2] = __builtin_bit_cast(bf16x8, make_uint4(l[0], l[1], l[2], l[3]));
     }
-    // input gradient: wave -> (position block mb, j quarter jpart); A operand of step st: wd[j][k = l16] for
+    // input gradient: wave -> (position block mb, j part jpart of 64 columns); A operand of step st: wd[j][k = l16] for
     // j = jd0 + 32 st + 8 lq .. + 7, which is wcat[k][j] with the negative rail (j >= c_out) negated
     const int mb = wave & 1, jpart = wave >> 1;
-    const int jd0 = jpart * (JW / 4);
+    const int jd0 = jpart * 64;
     bf16x8 wdr[DX ? 2 : 1][3];
     if (DX) {
 #pragma unroll
@@ -1762,20 +1637,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k
     }
     // (the tile loop's first barriers come before anything is written to est)
 
-    // im2col gather by the first four waves: thread -> position (t & 31) of the tile, members 2 (t >> 5) and
-    // 2 (t >> 5) + 1
-    const int ml = threadIdx.x & 31, kg = (threadIdx.x >> 5) & 7;
+    // im2col gather: 256 slots (position t & 31 of the tile, member pair t >> 5: members 2 pair and 2 pair + 1),
+    // taken by the first four waves, or GP per thread in a smaller workgroup
+    const int ml = threadIdx.x & 31;
     const bool gathers = threadIdx.x < 256;
-    int g_off[2], g_u[2], g_v[2];
-    bool g_ok[2];
+    int kg[GP];
+    int g_off[GP][2], g_u[GP][2], g_v[GP][2];
+    bool g_ok[GP][2];
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
-        const int k = 2 * kg + q;
-        const Member e = member_of(G, g, k < K ? k : 0);
-        g_ok[q] = gathers && k < K && e.ok;
-        g_off[q] = (e.ci * w_in + e.u) * h_in + e.v;
-        g_u[q] = e.u;
-        g_v[q] = e.v;
+    for (int gp = 0; gp < GP; gp++) {
+        kg[gp] = ((threadIdx.x >> 5) + gp * (NT / 32)) & 7;
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int k = 2 * kg[gp] + q;
+            const Member e = member_of(G, g, k < K ? k : 0);
+            g_ok[gp][q] = gathers && k < K && e.ok;
+            g_off[gp][q] = (e.ci * w_in + e.u) * h_in + e.v;
+            g_u[gp][q] = e.u;
+            g_v[gp][q] = e.v;
+        }
     }
     // this lane's 16 values of the wave's 32 x 32 block of the upstream gradient: offset in tile `split`, and
     // the distance to the next tile of this workgroup
@@ -1812,25 +1692,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k
         p.b0 = base[mc];
         return p;
     };
-    auto fetch = [&](const Where& p, float (&v)[2], bool (&ok)[2]) {
+    auto fetch = [&](const Where& p, float (&v)[GP][2], bool (&ok)[GP][2]) {
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
-            const int rr = p.r0 + g_u[q], cc = p.c0 + g_v[q];
-            ok[q] = p.ok && g_ok[q] && cc >= 0 && cc < h_in && rr >= 0 && rr < w_in;
-            v[q] = x[ok[q] ? p.b0 + g_off[q] : 0];
-        }
+        for (int gp = 0; gp < GP; gp++)
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const int rr = p.r0 + g_u[gp][q], cc = p.c0 + g_v[gp][q];
+                ok[gp][q] = p.ok && g_ok[gp][q] && cc >= 0 && cc < h_in && rr >= 0 && rr < w_in;
+                v[gp][q] = x[ok[gp][q] ? p.b0 + g_off[gp][q] : 0];
+            }
     };
-    float x_next[2], x_after[2];
-    bool ok_next[2], ok_after[2];
+    float x_next[GP][2], x_after[GP][2];
+    bool ok_next[GP][2], ok_after[GP][2];
     Where w_after;
-    auto commit = [&](int buf, const float (&v)[2], const bool (&ok)[2]) {
-        unsigned t3[3];
-        split3(ok[0] ? v[0] : 0.0f, ok[1] ? v[1] : 0.0f, t3[0], t3[1], t3[2]);
+    auto commit = [&](int buf, const float (&v)[GP][2], const bool (&ok)[GP][2]) {
 #pragma unroll
-        for (int t = 0; t < 3; t++) {
-            ((unsigned*)&csz[buf][t][kg >> 2][ml])[kg & 3] = t3[t];
-            ((unsigned short*)&csg[buf][t][2 * kg][0])[ml] = (unsigned short)t3[t];
-            ((unsigned short*)&csg[buf][t][2 * kg + 1][0])[ml] = (unsigned short)(t3[t] >> 16);
+        for (int gp = 0; gp < GP; gp++) {
+            unsigned t3[3];
+            split3(ok[gp][0] ? v[gp][0] : 0.0f, ok[gp][1] ? v[gp][1] : 0.0f, t3[0], t3[1], t3[2]);
+#pragma unroll
+            for (int t = 0; t < 3; t++) {
+                ((unsigned*)&csz[buf][t][kg[gp] >> 2][ml])[kg[gp] & 3] = t3[t];
+                ((unsigned short*)&csg[buf][t][2 * kg[gp]][0])[ml] = (unsigned short)t3[t];
+                ((unsigned short*)&csg[buf][t][2 * kg[gp] + 1][0])[ml] = (unsigned short)(t3[t] >> 16);
+            }
         }
     };
     {
@@ -1925,7 +1810,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k
 #pragma unroll
                 for (int st = 0; st < 2; st++)
                     d[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wdr[st][ta[t]], bd[st][tb[t]], d[st], 0, 0, 0);
-            if (jpart > 0) {
+            if (JPARTS > 1 && jpart > 0) {
 #pragma unroll
                 for (int r = 0; r < 4; r++) red[jpart - 1][mb][4 * lq + r][l16] = d[0][r] + d[1][r];
             }
@@ -1937,15 +1822,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4))) void k
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int k = 4 * lq + r;
-                const float sum = ((d[0][r] + d[1][r]) + red[0][mb][k][l16]) + (red[1][mb][k][l16] + red[2][mb][k][l16]);
+                float sum = d[0][r] + d[1][r];
+#pragma unroll
+                for (int jp = 1; jp < JPARTS; jp++) sum += red[jp - 1][mb][k][l16];
                 if (k < K && m < M) dg[(size_t)k * M + m] = sum;
             }
         }
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
-            x_next[q] = x_after[q];
-            ok_next[q] = ok_after[q];
-        }
+        for (int gp = 0; gp < GP; gp++)
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                x_next[gp][q] = x_after[gp][q];
+                ok_next[gp][q] = ok_after[gp][q];
+            }
     }
     if (store_part) {
         float* pg = part + (size_t)blockIdx.y * part_stride + (size_t)split * K * J;
@@ -2023,7 +1912,6 @@ struct BwdLayout {
     long long m_total;
     int splits, m_per_split;
     Groups G;
-    bool small_k;        // OR groups of at most 16 members and 2 * c_out <= 128: fused weight-gradient kernel
     bool fused_k;        // OR groups of at most 32 members: whole backward in one kernel, no col / E scratch
     int fused_jw;        // columns of E per workgroup of that kernel
     int fused_jblocks;   // its column blocks: each writes a dcol slice of its own
@@ -2069,9 +1957,9 @@ BwdLayout bwd_layout(const Geometry& g)
         b.G.n_members = g.k_or;
     }
     const int K = b.G.n_members;
-    b.small_k = K <= kSmallK && 2 * g.c_out <= kTile;
     b.fused_k = K <= kFusedK;
-    b.fused_jw = 2 * g.c_out <= 128 ? 128 : 256;
+    // the bf16 kernel (at most 16 members) comes with 2, 4 or 8 waves of 32 columns, the fp32 one with 128 or 256 columns
+    b.fused_jw = 2 * g.c_out <= 64 && K <= 16 ? 64 : 2 * g.c_out <= 128 ? 128 : 256;
     b.fused_jblocks = (2 * g.c_out + b.fused_jw - 1) / b.fused_jw;
     b.gt_dedupe = g.c_out % 32 == 0;
     b.gt_blocks = b.gt_dedupe ? g.c_out / 32 : (2 * g.c_out + 31) / 32;
@@ -2177,8 +2065,7 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     const bool col2im_v4 = quad_rows && g.h_k <= 8 && gx && ((uintptr_t)gx & 15) == 0;
     hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
                        g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
-    const bool wgrad_only = !gx && gw && L.small_k;
-    const bool fused = L.fused_k && !wgrad_only;
+    const bool fused = L.fused_k;
     {
         const int npos = g.wo * g.ho;
         if (fused) {
@@ -2191,33 +2078,6 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         }
     }
     int rc;
-    if (wgrad_only) {
-        // first-layer case: fused im2col + both products, no col / E scratch traffic
-        for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
-            const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
-            int wb = grid1d((long long)K * g.c_out);
-            hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
-                               g.c_out, G, L.w_v);
-            // about eight workgroups per CU in all, each looping over its share of the tiles
-            int active = 2048 / nv;
-            if (active > L.splits) active = L.splits;
-            if (active < 1) active = 1;
-            const dim3 grid(active, nv);
-#define GEO_SC_SMALL_K(JB)                                                                                          \
-    hipLaunchKernelGGL(k_wgrad_small_k<JB>, grid, dim3(256), 0, s, x, wcat, gt, pos_base, pos_arow, pos_bcol, part, G, \
-                       v0, M, g.w_in, g.h_in, g.c_out, active, L.w_v, L.part_v)
-            switch ((J + 31) / 32) {
-            case 1: GEO_SC_SMALL_K(1); break;
-            case 2: GEO_SC_SMALL_K(2); break;
-            case 3: GEO_SC_SMALL_K(3); break;
-            default: GEO_SC_SMALL_K(4); break;
-            }
-#undef GEO_SC_SMALL_K
-            hipLaunchKernelGGL(k_reduce_wgrad, dim3((K * g.c_out + 31) / 32, nv), dim3(256), 0, s, part, w, gw, v0,
-                               active, g.c_out, G, L.part_v);
-        }
-        return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
-    }
     if (fused) {
         if (!gx && !gw) return GEO_SC_OK;
         const int plane_blocks = (g.w_in * g.h_in + 255) / 256;
@@ -2254,21 +2114,22 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             if (gx) GEO_SC_FUSED_K(KS, 2, true); else GEO_SC_FUSED_K(KS, 2, false);                                    \
         }                                                                                                              \
     } while (0)
-                if (ks <= 8 && jw == 256) {
-                    if (gx)
-                        hipLaunchKernelGGL(k_bwd_small_k_bf16<true>, grid, dim3(512), 0, s, x, wcat, gt, pos_base, pos_arow,
-                                           pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks,
-                                           L.fused_splits, gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v,
-                                           slice);
-                    else
-                        hipLaunchKernelGGL(k_bwd_small_k_bf16<false>, grid, dim3(512), 0, s, x, wcat, gt, pos_base, pos_arow,
-                                           pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks,
-                                           L.fused_splits, gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v,
-                                           slice);
-                } else if (ks <= 5) GEO_SC_FUSED_NB_DX(5);
-                else if (ks <= 8) GEO_SC_FUSED_NB_DX(8);
+#define GEO_SC_FUSED_BF16(NW, DX)                                                                                      \
+    hipLaunchKernelGGL((k_bwd_small_k_bf16<NW, DX>), grid, dim3(64 * NW), 0, s, x, wcat, gt, pos_base, pos_arow,        \
+                       pos_bcol, part, dcol, G, v0, M, g.w_in, g.h_in, g.c_out, L.fused_jblocks, L.fused_splits,        \
+                       gw ? 1 : 0, L.gt_blocks, L.gt_dedupe, L.w_v, L.part_v, L.col_v, slice)
+                if (ks <= 8) {
+                    if (jw == 64) {
+                        if (gx) GEO_SC_FUSED_BF16(2, true); else GEO_SC_FUSED_BF16(2, false);
+                    } else if (jw == 128) {
+                        if (gx) GEO_SC_FUSED_BF16(4, true); else GEO_SC_FUSED_BF16(4, false);
+                    } else {
+                        if (gx) GEO_SC_FUSED_BF16(8, true); else GEO_SC_FUSED_BF16(8, false);
+                    }
+                }
                 else if (ks <= 12) GEO_SC_FUSED_NB_DX(12);
                 else GEO_SC_FUSED_NB_DX(16);
+#undef GEO_SC_FUSED_BF16
 #undef GEO_SC_FUSED_NB_DX
 #undef GEO_SC_FUSED_K
             }
