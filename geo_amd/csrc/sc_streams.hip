@@ -112,13 +112,14 @@ __device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, const uint32_t
 // keep their place in the seed numbering (sc.cpp:409-413).  Layout [n][P][c_in][Wi][Hi], or
 // with ITEM_INNER [P][c_in][Wi][Hi][n]; threads run along the innermost axis of the output.
 // XT: float (the activation itself) or uint8_t (the 7-bit integer k, activation k / 128).
-template <bool ITEM_INNER, typename XT>
+template <bool ITEM_INNER, typename XT, int V = 1>
 __global__ __launch_bounds__(kGenThreads) void k_act_streams(const XT* __restrict__ x,
                                                             uint32_t* __restrict__ streams,
                                                             const uint32_t* __restrict__ tables, GenParams gp, int n,
                                                             int c_in, int w_in, int h_in, int pad_w, int pad_h,
                                                             uint32_t seed_wrap)
 {
+    static_assert(V == 1 || (V == 4 && !ITEM_INNER), "four elements per thread along the item's flat index only");
     extern __shared__ uint32_t lds[];
     load_tables_to_lds(lds, tables, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
@@ -127,38 +128,66 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const XT* __restric
     const uint32_t plane = (uint32_t)c_in * wi * hi;
     const size_t total = (size_t)n * plane;
     const float Lf = (float)gp.L, top = (float)(gp.L - 1);
-    for (size_t e = (size_t)blockIdx.x * kGenThreads + threadIdx.x; e < total; e += (size_t)gridDim.x * kGenThreads) {
-        uint32_t item, i;
+    // V = 4: a thread takes four consecutive elements of one item (the launcher checks plane % 4 == 0 and the
+    // buffer's alignment) and stores their words of a pack as one 16-byte quad
+    for (size_t e = ((size_t)blockIdx.x * kGenThreads + threadIdx.x) * V; e < total;
+         e += (size_t)gridDim.x * kGenThreads * V) {
+        uint32_t item, i0;
         if (ITEM_INNER) {
-            i = (uint32_t)(e / (uint32_t)n);
-            item = (uint32_t)(e - (size_t)i * n);
+            i0 = (uint32_t)(e / (uint32_t)n);
+            item = (uint32_t)(e - (size_t)i0 * n);
         } else {
             item = (uint32_t)(e / plane);
-            i = (uint32_t)(e - (size_t)item * plane);
+            i0 = (uint32_t)(e - (size_t)item * plane);
         }
-        const uint32_t q = i % (uint32_t)hi;
-        const uint32_t r = i / (uint32_t)hi;
-        const uint32_t p = r % (uint32_t)wi;
-        const uint32_t c = r / (uint32_t)wi;
-        const int ps = (int)p - pad_w, qs = (int)q - pad_h;
-        int code = 0;
-        if (ps >= 0 && ps < w_in && qs >= 0 && qs < h_in) {
-            const float v = sizeof(XT) == 1 ? (float)x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs] * 0.0078125f
-                                            : (float)x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs];
-            // ceil(clamp(x*L, 0, L-1))  (sc.cpp:301)
-            code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
+        int code[V], o[V];
+        // coordinates and seed index of the first element by division, of the next ones by stepping
+        uint32_t q = i0 % (uint32_t)hi;
+        const uint32_t r0 = i0 / (uint32_t)hi;
+        uint32_t p = r0 % (uint32_t)wi, c = r0 / (uint32_t)wi;
+        uint32_t iw = i0 % seed_wrap, sm = iw % (uint32_t)(gp.L - 1);
+#pragma unroll
+        for (int j = 0; j < V; j++) {
+            const int ps = (int)p - pad_w, qs = (int)q - pad_h;
+            code[j] = 0;
+            if (ps >= 0 && ps < w_in && qs >= 0 && qs < h_in) {
+                const float v = sizeof(XT) == 1
+                                    ? (float)x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs] * 0.0078125f
+                                    : (float)x[(((size_t)item * c_in + c) * w_in + ps) * h_in + qs];
+                // ceil(clamp(x*L, 0, L-1))  (sc.cpp:301)
+                code[j] = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
+            }
+            // seed index: flat position in the item, restarting per channel group when seed_wrap is
+            // smaller than the item (sc_cuda_kernel.cu:1080)
+            o[j] = (int)posp1[sm];
+            if (V > 1) {
+                if (++q == (uint32_t)hi) {
+                    q = 0;
+                    if (++p == (uint32_t)wi) {
+                        p = 0;
+                        ++c;
+                    }
+                }
+                ++sm;
+                if (++iw == seed_wrap) iw = sm = 0;
+                if (sm == (uint32_t)(gp.L - 1)) sm = 0;
+            }
         }
-        // seed index: flat position in the item, restarting per channel group when seed_wrap is
-        // smaller than the item (sc_cuda_kernel.cu:1080)
-        const int o = (int)posp1[(i % seed_wrap) % (uint32_t)(gp.L - 1)];
         if (ITEM_INNER) {
-            uint32_t* dst = streams + (size_t)i * n + item;
+            uint32_t* dst = streams + (size_t)i0 * n + item;
             for (int pk = 0; pk < gp.packs; pk++)
-                dst[(size_t)pk * plane * n] = code ? stream_word(thr, code, o, pk, gp) : 0u;
+                dst[(size_t)pk * plane * n] = code[0] ? stream_word(thr, code[0], o[0], pk, gp) : 0u;
         } else {
-            uint32_t* dst = streams + (size_t)item * gp.packs * plane + i;
-            for (int pk = 0; pk < gp.packs; pk++)
-                dst[(size_t)pk * plane] = code ? stream_word(thr, code, o, pk, gp) : 0u;
+            uint32_t* dst = streams + (size_t)item * gp.packs * plane + i0;
+            for (int pk = 0; pk < gp.packs; pk++) {
+                uint32_t wv[V];
+#pragma unroll
+                for (int j = 0; j < V; j++) wv[j] = code[j] ? stream_word(thr, code[j], o[j], pk, gp) : 0u;
+                if constexpr (V == 4)
+                    *(uint4*)(dst + (size_t)pk * plane) = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+                else
+                    dst[(size_t)pk * plane] = wv[0];
+            }
         }
     }
 }
@@ -554,6 +583,9 @@ static int launch_act_streams_t(const Geometry& g, const XT* x, uint32_t* stream
     if (g.act_item_inner)
         hipLaunchKernelGGL((k_act_streams<true, XT>), dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
                            streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
+    else if (g.act_plane % 4 == 0 && ((uintptr_t)streams & 15) == 0)
+        hipLaunchKernelGGL((k_act_streams<false, XT, 4>), dim3(grid_for(total / 4)), dim3(kGenThreads), table_bytes(g.L),
+                           s, x, streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     else
         hipLaunchKernelGGL((k_act_streams<false, XT>), dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s,
                            x, streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
