@@ -77,6 +77,11 @@ struct GemmParams {
     const long long* __restrict__ a_rows;
     long long a_rows_batch;
     int a_item, a_skip;
+    // B as a view of E shifted by whole image rows (kernels with VB; the input-gradient product summed over
+    // the kernel rows u): k = u * sh_j + j, and column i = (n, p, b) of B is row (n, p + sh_pad - u, b) of E
+    // (sh_j floats per row of E, ldb apart) where that output row exists, zero elsewhere (read from sh_zero).
+    const float* __restrict__ sh_zero;
+    int sh_j, sh_wo, sh_ho, sh_win, sh_pad;
     // tile extent per workgroup in i and j: kTile, or kTile / 2 in at most one of them (set by
     // launch_gemm): the four waves then line up along the other dimension
     int tile_i, tile_j;
@@ -534,9 +539,79 @@ struct ViewStager {
     }
 };
 
+// Stager of the B operand of the input-gradient product when it sums over the kernel rows inside the GEMM
+// (GemmParams::sh_*): the k dimension runs over (u, j), and for kernel row u the column (n, p, b) of B is
+// the row (n, p + pad - u, b) of E.  I-major: a thread keeps one column and eight consecutive j; when j passes
+// the end of a row of E the thread moves to the row of the next u.  Columns whose output row does not exist
+// for a u read a block of zeros instead (no select on the loaded data, so nothing waits for the load).
+// sh_j is a multiple of kChunk: no chunk straddles two u, and there are no partial chunks.
+struct ShiftStager {
+    const float* e_rows;   // E of this batch member
+    const float* zero;
+    const float* p;
+    long long ld;
+    int j, u, prow, wo;  // j: this thread's first column of E in the current chunk; prow: p + pad
+    long long row0;                 // (n * wo + prow + pad) * ho + b: the row of E for u = 0
+    int half, ii, sh_j, ho;
+
+    __device__ __forceinline__ void point()
+    {
+        const int r = prow - u;  // prow already holds p + pad
+        p = (r >= 0 && r < wo) ? e_rows + (row0 - (long long)u * ho) * ld + j : zero;
+    }
+    __device__ __forceinline__ void init(const GemmParams& q, int batch, int j0, int k_begin, int Jn, int)
+    {
+        const int t = threadIdx.x;
+        ii = t >> 1;
+        half = t & 1;
+        e_rows = q.b + batch * q.b_batch_stride;
+        zero = q.sh_zero;
+        ld = q.ldb;
+        sh_j = q.sh_j;
+        wo = q.sh_wo;
+        ho = q.sh_ho;
+        const int m = min(j0 + ii, Jn - 1);
+        const int per_item = q.sh_win * q.sh_ho;
+        const int n = m / per_item, rem = m - n * per_item;
+        const int pr = rem / q.sh_ho, b = rem - pr * q.sh_ho;
+        prow = pr + q.sh_pad;
+        row0 = ((long long)n * wo + prow) * ho + b;
+        const int k = k_begin + 8 * half;
+        u = k / sh_j;
+        j = k - u * sh_j;
+        point();
+    }
+    __device__ __forceinline__ void advance()
+    {
+        j += kChunk;
+        if (j >= sh_j) {
+            j -= sh_j;
+            ++u;
+        }
+        point();
+    }
+    __device__ __forceinline__ void fetch_whole(float (&r)[8])
+    {
+        const float4 v0 = *(const float4*)p, v1 = *(const float4*)(p + 4);
+        r[0] = v0.x; r[1] = v0.y; r[2] = v0.z; r[3] = v0.w;
+        r[4] = v1.x; r[5] = v1.y; r[6] = v1.z; r[7] = v1.w;
+        advance();
+    }
+    __device__ __forceinline__ void fetch(float (&r)[8], int) { fetch_whole(r); }
+    __device__ __forceinline__ void commit(uint4 (*s)[2][kLdx], float (&r)[8], int) const
+    {
+        unsigned hi[4], mid[4], lo[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) split3(r[2 * c], r[2 * c + 1], hi[c], mid[c], lo[c]);
+        s[0][half][ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        s[1][half][ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        s[2][half][ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    }
+};
+
 // v_mfma_f32_32x32x16_bf16: lane l feeds A[i = l%32][k = 8 (l/32) .. + 7] and B[those k][j = l%32]:
 // the 16 bytes at s[term][l/32][i]; results as in the fp32 instruction.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int NX, int NY, bool VA>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int NX, int NY, bool VA, bool VB>
 __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)[3][2][kLdx], uint4 (*bs)[3][2][kLdx],
                                                 int i0, int j0, int batch, int split, int k_begin, int k_end, int wi,
                                                 int wj, int l32, int lk, int wave)
@@ -550,12 +625,15 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
             for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
 
     typename std::conditional<VA, ViewStager<A_KMAJOR>, SplitStager<A_KMAJOR>>::type sa;
-    SplitStager<B_KMAJOR> sb;
+    typename std::conditional<VB, ShiftStager, SplitStager<B_KMAJOR>>::type sb;
     if constexpr (VA)
         sa.init(q, batch, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
     else
         sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
-    sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
+    if constexpr (VB)
+        sb.init(q, batch, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
+    else
+        sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
     // Two chunks ahead: while chunk c is multiplied out of LDS, chunk c + 1 sits in one register set
     // (its loads issued a whole trip ago) and the loads of chunk c + 2 go out into the other.
     float ra[2][8], rb[2][8];
@@ -690,7 +768,7 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
 }
 
 // Operands with 16-byte aligned rows and chunks (launch_gemm checks).
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VA = false>
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VA = false, bool VB = false>
 // three waves per SIMD (at most 168 registers; three workgroups' LDS fit a CU)
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void k_gemm_split(GemmParams q)
 {
@@ -711,7 +789,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const bool y0 = j0 + wj < q.J, y1 = !narrow_i && j0 + wj + 32 < q.J;
     const int blocks_xy = (x0 && y0) ? 2 * (int)x1 + (int)y1 : -1;
 #define GEO_SC_GEMM_WAVE(NX, NY)                                                                                        \
-    gemm_wave_split<A_KMAJOR, B_KMAJOR, EPI, NX, NY, VA>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk, wave)
+    gemm_wave_split<A_KMAJOR, B_KMAJOR, EPI, NX, NY, VA, VB>(q, as, bs, i0, j0, batch, split, k_begin, k_end, wi, wj, l32, lk, wave)
     switch (blocks_xy) {
     case 3: GEO_SC_GEMM_WAVE(2, 2); break;
     case 2: GEO_SC_GEMM_WAVE(2, 1); break;
@@ -1228,6 +1306,66 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad_tiled(const float* __restr
         if (wv >= 0.0f && wv <= 100.0f) r += tp[tx][q];
         if (wv >= -100.0f && wv <= 0.0f) r += tn[tx][q];
         gw[wi] = r;
+    }
+}
+
+// 64 zeros (a fill kernel rather than a memset, so that a caller may capture the launch sequence in a graph)
+__global__ __launch_bounds__(64) void k_zero_block(float* __restrict__ p) { p[threadIdx.x] = 0.0f; }
+
+// The A operand of the input-gradient product summed over the kernel rows inside the GEMM (y
+// accumulation: group = kernel column v, members (ci, u)): wdx[g][(u * 2 c_out + j)][ci] = wd[g][j][(ci, u)],
+// i.e. clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one.
+__global__ __launch_bounds__(256) void k_weight_dx_operand(const float* __restrict__ w, float* __restrict__ wdx, int g0,
+                                                           int c_out, int c_in, int w_k, int h_k, size_t g_stride)
+{
+    const int J = 2 * c_out;
+    const int total = w_k * J * c_in;
+    float* dst = wdx + (size_t)blockIdx.y * g_stride;
+    const int v = g0 + blockIdx.y;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int ci = e % c_in, r = e / c_in;
+        const int j = r % J, u = r / J;
+        const int co = j >= c_out ? j - c_out : j;
+        const float wv = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v];
+        dst[e] = j < c_out ? fminf(fmaxf(wv, 0.0f), 100.0f) : fminf(fmaxf(wv, -100.0f), 0.0f);
+    }
+}
+
+// dL/dx[n][ci][p][q] = sum over the kernel columns v of d[v][ci][(n, p, q + pad_h - v)] where that output
+// column exists: what is left of col2im when the GEMM has summed the kernel rows.  Four elements of an
+// input row per thread (rows of whole quads on both sides, 16-byte aligned buffers), one grid-stride loop
+// over the quads of dL/dx.
+__global__ __launch_bounds__(256) void k_shift_sum_v4(const float* __restrict__ d, float* __restrict__ gx, long long quads,
+                                                      int n_items, int c_in, int w_in, int h_in, int h_k, int pad_h,
+                                                      int ho)
+{
+    const int hq = h_in >> 2;
+    const long long per_v = (long long)c_in * n_items * w_in * ho;
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < quads; e += (long long)gridDim.x * 256) {
+        // e = ((n * c_in + ci) * w_in + p) * hq + quad
+        long long t = e;
+        const int qq = (int)(t % hq) << 2;
+        t /= hq;
+        const int p = (int)(t % w_in);
+        t /= w_in;
+        const int ci = (int)(t % c_in), n = (int)(t / c_in);
+        const float* row = d + (((long long)ci * n_items + n) * w_in + p) * ho;
+        float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int v = 0; v < h_k; v++) {
+            const int b = qq + pad_h - v;
+            const int sh = b & 3, ba = b - sh;
+            const bool ok_a = ba >= 0 && ba < ho, ok_b = sh != 0 && ba + 4 >= 0 && ba + 4 < ho;
+            const float4* r4 = (const float4*)(row + v * per_v);
+            float4 qa = r4[ok_a ? ba >> 2 : 0], qb = r4[ok_b ? (ba >> 2) + 1 : 0];
+            if (!ok_a) qa = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (!ok_b) qb = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            const float4 tq = shifted_quad(qa, qb, sh);
+            s.x += tq.x;
+            s.y += tq.y;
+            s.z += tq.z;
+            s.w += tq.w;
+        }
+        ((float4*)gx)[e] = s;
     }
 }
 
@@ -1859,7 +1997,7 @@ int grid1d(long long total)
 
 // VA: the A operand is a view of the shifted input planes (GemmParams::a_rows); the caller has checked that
 // its rows and chunks are 16-byte aligned.
-template <bool AK, bool BK, int EPI, bool VA = false>
+template <bool AK, bool BK, int EPI, bool VA = false, bool VB = false>
 int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
 {
     GemmParams q = q0;
@@ -1892,7 +2030,10 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
     };
     const bool a_vec = VA || AK || rows_aligned(q.a, q.lda, q.a_batch_stride);
     const bool b_vec = BK || rows_aligned(q.b, q.ldb, q.b_batch_stride);
-    if constexpr (VA) {
+    if constexpr (VB) {
+        // (the caller has checked the view's alignment: rows of E and the runs of eight columns)
+        hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, false, true>), grid, dim3(256), 0, s, q);
+    } else if constexpr (VA) {
         if (!b_vec) return GEO_SC_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
     } else if constexpr (AK && BK) {
@@ -1920,6 +2061,8 @@ struct BwdLayout {
     int gt_blocks;       // 32-column blocks of those tiles
     int rows_per_chunk;  // add groups processed by one round of launches
     int dcol_slices;     // partial dcol arrays per round (column blocks of the fused kernel), rows_per_chunk * col_v apart
+    bool dx_rows;        // the input-gradient GEMM sums the kernel rows itself (E read as a view shifted by image rows)
+    size_t off_zero;     // a block of zeros for that view
     bool view_col;       // the GEMMs read col as a view of the shifted input planes (k_shift_planes) kept in col's space
     int view_k_pad;      // entries per group of the view's row table
     size_t off_rows;     // the row table
@@ -2011,6 +2154,13 @@ BwdLayout bwd_layout(const Geometry& g)
                  rows == (size_t)b.G.n_groups && !(g.mode == GEO_SC_ACC_YZ && g.c_in % g.z_unit != 0) &&
                  view_floats(g) <= rows * col_alloc &&
                  (long long)g.n * (g.w_in + 2 * g.pad_w) * g.ho + (long long)g.w_k * g.ho < 0x7fffffffLL;
+    // the kernel rows summed inside the input-gradient GEMM: y accumulation (group = kernel column, members =
+    // (channel, kernel row)), whole quads in the rows of input and output, whole chunks of rails, every group in
+    // one round, and the per-column result inside dcol's space
+    b.dx_rows = !b.fused_k && g.mode == GEO_SC_ACC_Y && g.ho % 4 == 0 && g.h_in % 4 == 0 && g.h_k <= 8 &&
+                (2 * g.c_out) % kChunk == 0 && rows == (size_t)b.G.n_groups &&
+                (size_t)g.h_k * g.c_in * g.n * g.w_in * g.ho <= rows * b.col_v &&
+                (long long)g.n * g.w_in * g.ho < 0x7fffffffLL && (long long)g.w_k * 2 * g.c_out < 0x7fffffffLL;
     size_t o = 0;
     b.off_col = o;  o += align256(sizeof(float) * rows * col_alloc);
     b.off_e = o;    o += align256(sizeof(float) * rows * e_alloc);
@@ -2028,6 +2178,8 @@ BwdLayout bwd_layout(const Geometry& g)
     }
     b.off_rows = o;
     o += align256(sizeof(long long) * (size_t)b.G.n_groups * b.view_k_pad);
+    b.off_zero = o;
+    o += 256;
     b.bytes = o;
     return b;
 }
@@ -2213,6 +2365,31 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
                                L.splits, g.c_out, G, L.part_v);
         }
         if (!gx) continue;
+        if (L.dx_rows && ((uintptr_t)gx & 15) == 0) {
+            // d[v][ci][(n, p, b)] = sum_(u, j) wd_v[j][(ci, u)] * E_v[(n, p + pad - u, b)][j]: the kernel rows
+            // summed inside the GEMM (three times the k of the product per (ci, u), a third of its rows and of
+            // its output), then the kernel columns by k_shift_sum_v4
+            float* zero = (float*)(ws + L.off_zero);
+            hipLaunchKernelGGL(k_zero_block, dim3(1), dim3(64), 0, s, zero);
+            const int k3 = g.w_k * J;
+            int wb = grid1d((long long)k3 * g.c_in);
+            hipLaunchKernelGGL(k_weight_dx_operand, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wd, v0, g.c_out,
+                               g.c_in, g.w_k, g.h_k, L.w_v);
+            const long long m2 = (long long)g.n * g.w_in * g.ho;
+            GemmParams q3 = {};
+            q3.a = wd; q3.b = e; q3.c = dcol;
+            q3.I = g.c_in; q3.J = (int)m2; q3.K = k3;
+            q3.lda = g.c_in; q3.ldb = J; q3.ldc = m2;
+            q3.splits = 1; q3.k_per_split = k3; q3.c_split_stride = 0;
+            q3.a_batch_stride = (long long)L.w_v; q3.b_batch_stride = (long long)L.e_v;
+            q3.c_batch_stride = (long long)g.c_in * m2;
+            q3.sh_zero = zero; q3.sh_j = J; q3.sh_wo = g.wo; q3.sh_ho = g.ho; q3.sh_win = g.w_in; q3.sh_pad = g.pad_w;
+            if ((rc = launch_gemm<true, false, EPI_STORE, false, true>(q3, nv, s)) != GEO_SC_OK) return rc;
+            const long long quads = (long long)g.n * g.c_in * g.w_in * g.h_in / 4;
+            hipLaunchKernelGGL(k_shift_sum_v4, dim3(grid1d(quads)), dim3(256), 0, s, dcol, gx, quads, g.n, g.c_in, g.w_in,
+                               g.h_in, g.h_k, g.pad_h, g.ho);
+            continue;
+        }
         // dcol[v][k][m] = sum_j wd_v[j][k] * E_v[m][j]
         GemmParams q3 = {};
         q3.a = wd; q3.b = e; q3.c = dcol;

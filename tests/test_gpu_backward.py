@@ -73,6 +73,11 @@ GEMM_CASES = [
     ((2, 12, 4, 8), (4, 12, 3, 7), (1, 3), 2.0),
     ((1, 12, 3, 16), (3, 12, 3, 9), (1, 4), 2.0),     # nine kernel columns: four-position im2col, one-position col2im
     ((1, 12, 6, 8), (4, 12, 3, 2), (1, 0), 2.0),      # output rows of 7: the one-position kernels
+    # a multiple of 8 output channels on top: the input-gradient GEMM sums the kernel rows itself
+    ((2, 12, 8, 12), (8, 12, 5, 5), (2, 2), 2.0),     # 5 x 5, same-size output
+    ((2, 20, 9, 8), (8, 20, 2, 1), (0, 0), 2.0),      # no padding: 8 output rows from 9 input rows
+    ((1, 12, 6, 8), (16, 12, 3, 3), (1, 2), 2.0),     # more output rows (8) than input rows (6)
+    ((3, 16, 4, 4), (24, 16, 3, 3), (1, 1), 2.0),     # 16 positions per item, 48 rails
 ]
 
 
