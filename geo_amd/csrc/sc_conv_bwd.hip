@@ -1701,7 +1701,7 @@ constexpr int kBfEw = 18;  // words per row of E^T: 32 bf16 and padding
 constexpr int kBfCw = 20;  // words per row of col[k][m]: 16-byte aligned rows
 
 template <int NW, bool DX>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4))) void k_bwd_small_k_bf16(
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW == 8 ? 4 : 3))) void k_bwd_small_k_bf16(
     const float* __restrict__ x, const float* __restrict__ wcat, const float* __restrict__ gtt,
     const int* __restrict__ base, const int* __restrict__ arow, const int* __restrict__ bcol, float* __restrict__ part,
     float* __restrict__ dcol, Groups G, int g0, int M, int w_in, int h_in, int c_out, int jblocks, int splits,
