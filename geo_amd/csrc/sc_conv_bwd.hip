@@ -2215,9 +2215,13 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     const bool quad_rows = g.h_in % 4 == 0 && g.ho % 4 == 0;
     const bool im2col_v4 = quad_rows && ((uintptr_t)x & 15) == 0;
     const bool col2im_v4 = quad_rows && g.h_k <= 8 && gx && ((uintptr_t)gx & 15) == 0;
-    hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
-                       g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
     const bool fused = L.fused_k;
+    // col as a view of the shifted input planes (one round holds every group then)
+    const bool view = L.view_col && ((uintptr_t)x & 15) == 0;
+    // the position tables serve the gathers of im2col and of the fused kernels
+    if (fused || !view)
+        hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
+                           g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
     {
         const int npos = g.wo * g.ho;
         if (fused) {
@@ -2306,8 +2310,6 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         }
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
-    // col as a view of the shifted input planes (one round holds every group then)
-    const bool view = L.view_col && ((uintptr_t)x & 15) == 0;
     long long* view_rows = (long long*)(ws + L.off_rows);
     if (view) {
         const long long plane = (long long)g.n * (g.w_in + 2 * g.pad_w) * g.ho;
