@@ -209,6 +209,9 @@ def test_weight_gradient_of_small_or_groups(capi, shape_x, shape_w, pad, mode, z
     ((2, 12, 12, 8), (5, 12, 3, 3), (1, 1), "y", 1),     # odd number of output channels: the materialised col
 ])
 def test_backward_through_the_gemms_in_every_mode(capi, shape_x, shape_w, pad, mode, zu):
+    """The GEMM path with its operands read as views (col from the shifted input planes, in y mode also E
+    shifted by image rows inside the input-gradient product) against the float64 oracle in every accumulation
+    mode, and bit for bit against the materialised col, which an input off its 16-byte alignment takes."""
     from oracle import surrogate
     x, w = wl.make_inputs(shape_x, shape_w, "kaiming", seed=shape_x[1] + shape_w[0])
     w = (w * 2).contiguous()
