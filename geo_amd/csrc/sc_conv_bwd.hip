@@ -34,6 +34,7 @@
 #include <cstdint>
 #include <cstdlib>
 
+#include <algorithm>
 #include <type_traits>
 
 namespace geo_sc {
@@ -188,38 +189,49 @@ struct Stager {
 // upstream gradient: they go out 16 at a time from clamped addresses, then the exponentials, then
 // stores under the range conditions (a load inside a per-element branch is waited for element by
 // element: 64 memory latencies in a row).
-template <int EPI, int NX, int NY>
+template <int EPI, int NX, int NY, int MAXB = 2, bool WHOLE = false>
 __device__ __forceinline__ void store_tile(const GemmParams& q, const floatx16 (&acc)[NX ? NX : 1][NY ? NY : 1],
                                            float* __restrict__ out, int iw, int jw, int l32, int lk)
 {
+    // blocks in batches of up to MAXB: the gradient loads of a whole batch are in flight together.
+    // WHOLE: the wave's blocks lie inside the result, no range conditions.
+    constexpr int NB = NX * NY, NYd = NY ? NY : 1;
+    constexpr int BB = (MAXB >= 4 && NB % 4 == 0) ? 4 : (MAXB >= 3 && NB % 3 == 0) ? 3 : (MAXB >= 2 && NB % 2 == 0) ? 2 : 1;
 #pragma unroll
-    for (int x = 0; x < NX; x++)
+    for (int b0 = 0; b0 < NB; b0 += BB) {
+        float gv[BB][16];
+        if (EPI == EPI_EXP_TIMES_G) {
 #pragma unroll
-        for (int y = 0; y < NY; y++) {
-            const int j = jw + y * 32 + l32;
-            const bool j_ok = j < q.J;
-            const int ib = iw + x * 32 + 4 * lk;
-            float v[16];
-#pragma unroll
-            for (int r = 0; r < 16; r++) v[r] = acc[x][y][r];
-            if (EPI == EPI_EXP_TIMES_G) {
-                const int jc = j_ok ? j : q.J - 1;
+            for (int bb = 0; bb < BB; bb++) {
+                const int x = (b0 + bb) / NYd, y = (b0 + bb) % NYd;
+                const int j = jw + y * 32 + l32, ib = iw + x * 32 + 4 * lk;
+                const int jc = (WHOLE || j < q.J) ? j : q.J - 1;
                 const int co = jc >= q.c_out ? jc - q.c_out : jc;
-                float gv[16];
+                const float* gp = q.g + (long long)ib * q.c_out + co;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const int i = min(ib + 8 * (r >> 2) + (r & 3), q.I - 1);
-                    gv[r] = q.g[(long long)i * q.c_out + co];
+                    const int di = 8 * (r >> 2) + (r & 3);
+                    gv[bb][r] = WHOLE ? gp[di * q.c_out] : q.g[(long long)min(ib + di, q.I - 1) * q.c_out + co];
                 }
-#pragma unroll
-                for (int r = 0; r < 16; r++) v[r] = gv[r] * exp_neg(v[r]);
-            }
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int i = ib + 8 * (r >> 2) + (r & 3);
-                if (j_ok && i < q.I) out[(long long)i * q.ldc + j] = v[r];
             }
         }
+#pragma unroll
+        for (int bb = 0; bb < BB; bb++) {
+            const int x = (b0 + bb) / NYd, y = (b0 + bb) % NYd;
+            const int j = jw + y * 32 + l32, ib = iw + x * 32 + 4 * lk;
+            const bool j_ok = WHOLE || j < q.J;
+            float* op = out + (long long)ib * q.ldc + j;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int di = 8 * (r >> 2) + (r & 3);
+                const float v = EPI == EPI_EXP_TIMES_G ? gv[bb][r] * exp_neg(acc[x][y][r]) : acc[x][y][r];
+                if (WHOLE)
+                    op[(long long)di * q.ldc] = v;
+                else if (j_ok && ib + di < q.I)
+                    out[(long long)(ib + di) * q.ldc + j] = v;
+            }
+        }
+    }
 }
 
 // The K loop and the epilogue of one wave that owns the first NX x NY of its 2 x 2 blocks of
@@ -368,18 +380,16 @@ struct SplitStager {
     int off;          // K-major: this thread's i (clamped)
     int half, ii;
 
-    __device__ __forceinline__ void init(const float* base, long long ld_, int i0, int k_begin, int I, int wave)
+    // (ii_, half_): the row of the tile and the k half this thread stages (stage_slot)
+    __device__ __forceinline__ void init(const float* base, long long ld_, int i0, int k_begin, int I, int ii_, int half_)
     {
-        const int t = threadIdx.x;
         ld = ld_;
+        ii = ii_;
+        half = half_;
         if (KMAJOR) {
-            half = wave >> 1;
-            ii = t & 127;
             off = min(i0 + ii, I - 1);
             p = base + (long long)(k_begin + 8 * half) * ld;
         } else {
-            ii = t >> 1;
-            half = t & 1;
             p = base + (long long)min(i0 + ii, I - 1) * ld + k_begin + 8 * half;
         }
     }
@@ -456,22 +466,19 @@ struct ViewStager {
     int in_item, item, skip;
     int half, ii;
 
-    __device__ __forceinline__ void init(const GemmParams& q, int batch, int i0, int k_begin, int I, int wave)
+    __device__ __forceinline__ void init(const GemmParams& q, int batch, int i0, int k_begin, int I, int ii_, int half_)
     {
-        const int t = threadIdx.x;
         base = q.a;
         rows = q.a_rows + batch * q.a_rows_batch;
         item = q.a_item;
         skip = q.a_skip;
+        ii = ii_;
+        half = half_;
         if (KMAJOR) {
-            half = wave >> 1;
-            ii = t & 127;
             const int m = min(i0 + ii, I - 1);
             off = m + (m / item) * skip;
             kr = k_begin + 8 * half;
         } else {
-            ii = t >> 1;
-            half = t & 1;
             const int m = k_begin + 8 * half;
             in_item = m % item;
             p = base + rows[min(i0 + ii, I - 1)] + m + (long long)(m / item) * skip;
@@ -559,11 +566,10 @@ struct ShiftStager {
         const int r = prow - u;  // prow already holds p + pad
         p = (r >= 0 && r < wo) ? e_rows + (row0 - (long long)u * ho) * ld + j : zero;
     }
-    __device__ __forceinline__ void init(const GemmParams& q, int batch, int j0, int k_begin, int Jn, int)
+    __device__ __forceinline__ void init(const GemmParams& q, int batch, int j0, int k_begin, int Jn, int ii_, int half_)
     {
-        const int t = threadIdx.x;
-        ii = t >> 1;
-        half = t & 1;
+        ii = ii_;
+        half = half_;
         e_rows = q.b + batch * q.b_batch_stride;
         zero = q.sh_zero;
         ld = q.ldb;
@@ -626,14 +632,19 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
 
     typename std::conditional<VA, ViewStager<A_KMAJOR>, SplitStager<A_KMAJOR>>::type sa;
     typename std::conditional<VB, ShiftStager, SplitStager<B_KMAJOR>>::type sb;
+    // K-major operand: waves 0, 1 stage the first k half of the 128 rows, waves 2, 3 the second;
+    // I-major operand: two threads per row, one k half each
+    const int t = threadIdx.x;
+    const int a_ii = A_KMAJOR ? (t & 127) : (t >> 1), a_half = A_KMAJOR ? (wave >> 1) : (t & 1);
+    const int b_ii = (B_KMAJOR && !VB) ? (t & 127) : (t >> 1), b_half = (B_KMAJOR && !VB) ? (wave >> 1) : (t & 1);
     if constexpr (VA)
-        sa.init(q, batch, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
+        sa.init(q, batch, i0, k_begin, min(q.I, i0 + q.tile_i), a_ii, a_half);
     else
-        sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i), wave);
+        sa.init(q.a + batch * q.a_batch_stride, q.lda, i0, k_begin, min(q.I, i0 + q.tile_i), a_ii, a_half);
     if constexpr (VB)
-        sb.init(q, batch, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
+        sb.init(q, batch, j0, k_begin, min(q.J, j0 + q.tile_j), b_ii, b_half);
     else
-        sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j), wave);
+        sb.init(q.b + batch * q.b_batch_stride, q.ldb, j0, k_begin, min(q.J, j0 + q.tile_j), b_ii, b_half);
     // Two chunks ahead: while chunk c is multiplied out of LDS, chunk c + 1 sits in one register set
     // (its loads issued a whole trip ago) and the loads of chunk c + 2 go out into the other.
     float ra[2][8], rb[2][8];
@@ -798,6 +809,188 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     default: GEO_SC_GEMM_WAVE(0, 0); break;
     }
 #undef GEO_SC_GEMM_WAVE
+}
+
+// ---- the split kernel with eight waves per workgroup and a tile of 64 NX x 256 ----
+// What the 128 x 128 kernel waits for is its operands: every tile streams 128 + 128 rows of fp32 per 128 x 128
+// results through L2, and three workgroups per CU ask for more than the caches deliver.  Here one workgroup
+// per CU (2 x 4 waves, 32 NX x 64 results each; 2 waves per SIMD with up to 256 registers) multiplies
+// 64 NX x 256: per result a half (NX = 4) to three quarters (NX = 2) of the operand traffic.  A wave reads
+// the fragments of one term product at a time (NX + 2 reads for 2 NX MFMAs), so that the second wave of the
+// SIMD and the wave's own next reads fill the matrix pipe's shadow; the three-way split of the next chunk
+// is written between the MFMAs as in the small kernel.
+// With nobody else on the CU, a tile's first loads and its epilogue would run with the matrix pipe idle, so
+// the workgroups are persistent: workgroup w takes the tiles w, w + gridDim.x, ... and treats their chunks
+// as one stream - while the last chunks of a tile are multiplied, the first chunks of the next are already
+// loaded, split and written to LDS, and the epilogue runs with those loads in flight.
+// Whole tiles and whole, non-empty chunk ranges only (launch_gemm checks); the stagers and the epilogue
+// are the small kernel's.
+constexpr int kBigJ = 256;
+constexpr int kBigWorkgroups = 256;  // one per CU of an MI355X
+// rows of a tile for a result with I rows: 256, 192 or 128 (NX = 4, 3, 2); 0: I is no multiple of any
+inline int big_rows(int I) { return I % 256 == 0 ? 256 : I % 192 == 0 ? 192 : I % 128 == 0 ? 128 : 0; }
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VA, bool VB, int NX>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_gemm_big(GemmParams q)
+{
+    constexpr int RA = 64 * NX, LA = RA + 4, LB = kBigJ + 4;
+    __shared__ uint4 as[2][3][2][LA];
+    __shared__ uint4 bs[2][3][2][LB];
+    const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63;
+    const int wi = (wave >> 2) * (32 * NX), wj = (wave & 3) * 64;
+    const int l32 = lane & 31, lk = lane >> 5;
+    // Staging slots: 2 RA (row, k half) pairs of A and 512 of B for 512 threads; with NX < 4 the threads
+    // beyond A's pairs stage a pair a second time (same data to the same place).
+    constexpr bool BK = B_KMAJOR && !VB;
+    const int wa = wave % (RA / 32), ta = t % (2 * RA);
+    const int a_ii = A_KMAJOR ? (wa % NX) * 64 + lane : ta >> 1, a_half = A_KMAJOR ? wa / NX : ta & 1;
+    const int b_ii = BK ? (t & 255) : (t >> 1), b_half = BK ? (wave >> 2) : (t & 1);
+    typename std::conditional<VA, ViewStager<A_KMAJOR>, SplitStager<A_KMAJOR>>::type sa;
+    typename std::conditional<VB, ShiftStager, SplitStager<B_KMAJOR>>::type sb;
+
+    const int n_tiles = q.ni * q.nj * q.nz;
+    // the tile whose chunks are being loaded: the stagers point into it, left_f of its chunks are still to load
+    int w_f = blockIdx.x, left_f;
+    auto open_tile = [&]() {
+        int it, jt, z;
+        gemm_tile_of(q, w_f, it, jt, z);
+        const int batch = z / q.splits, split = z - batch * q.splits;
+        const int k_begin = split * q.k_per_split;
+        left_f = (min(q.K, k_begin + q.k_per_split) - k_begin) / kChunk;
+        if constexpr (VA)
+            sa.init(q, batch, it * RA, k_begin, q.I, a_ii, a_half);
+        else
+            sa.init(q.a + batch * q.a_batch_stride, q.lda, it * RA, k_begin, q.I, a_ii, a_half);
+        if constexpr (VB)
+            sb.init(q, batch, jt * kBigJ, k_begin, q.J, b_ii, b_half);
+        else
+            sb.init(q.b + batch * q.b_batch_stride, q.ldb, jt * kBigJ, k_begin, q.J, b_ii, b_half);
+    };
+    // the next chunk of the stream into a register set; nothing once the last tile is through
+    auto fetch_next = [&](float (&ra)[8], float (&rb)[8]) {
+        if (left_f == 0) {
+            if (w_f + (int)gridDim.x >= n_tiles) return;
+            w_f += gridDim.x;
+            open_tile();
+        }
+        sa.fetch_whole(ra);
+        sb.fetch_whole(rb);
+        --left_f;
+    };
+    // the tile being multiplied
+    int w_m = blockIdx.x, left_m, i0_m, j0_m;
+    float* out_m;
+    auto describe_m = [&]() {
+        int it, jt, z;
+        gemm_tile_of(q, w_m, it, jt, z);
+        const int batch = z / q.splits, split = z - batch * q.splits;
+        const int k_begin = split * q.k_per_split;
+        left_m = (min(q.K, k_begin + q.k_per_split) - k_begin) / kChunk;
+        i0_m = it * RA;
+        j0_m = jt * kBigJ;
+        out_m = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
+    };
+
+    floatx16 acc[NX][2];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int x = 0; x < NX; x++)
+#pragma unroll
+            for (int y = 0; y < 2; y++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[x][y][r] = 0.0f;
+    };
+    zero_acc();
+    open_tile();
+    describe_m();
+
+    // Register set c % 2 holds stream chunk c until it is split and written to LDS buffer c % 2, one trip
+    // before it is multiplied; its loads go out two trips before that.
+    float ra[2][8], rb[2][8];
+    fetch_next(ra[0], rb[0]);
+    fetch_next(ra[1], rb[1]);
+    {
+        unsigned hi[8], mid[8], lo[8];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            split3(ra[0][2 * c], ra[0][2 * c + 1], hi[c], mid[c], lo[c]);
+            split3(rb[0][2 * c], rb[0][2 * c + 1], hi[4 + c], mid[4 + c], lo[4 + c]);
+        }
+        as[0][0][a_half][a_ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        as[0][1][a_half][a_ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        as[0][2][a_half][a_ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        bs[0][0][b_half][b_ii] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        bs[0][1][b_half][b_ii] = make_uint4(mid[4], mid[5], mid[6], mid[7]);
+        bs[0][2][b_half][b_ii] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+    }
+    fetch_next(ra[0], rb[0]);
+    __syncthreads();
+
+    // One trip: stream chunk c out of LDS buffer S, chunk c + 1 (register set S ^ 1) split and written to
+    // the other buffer, the loads of chunk c + 3 into that register set.  Past the end of the stream the
+    // split works on stale registers and its result is never read.
+    auto trip = [&](auto set) {
+        constexpr int S = decltype(set)::value, R = S ^ 1;
+        constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};  // smallest terms first; 0 = hi
+        unsigned hi[8], mid[8], lo[8];
+        float r0[8], r1[8];
+        auto step = [&](int n) {
+            const int pr = n / 3, st = n % 3;
+            const float* src = pr < 4 ? ra[R] : rb[R];
+            const int e = 2 * (pr & 3);
+            if (st == 0) {
+                hi[pr] = pack_bf16(src[e], src[e + 1]);
+                r0[pr] = src[e] - __uint_as_float(hi[pr] << 16);
+                r1[pr] = src[e + 1] - __uint_as_float(hi[pr] & 0xffff0000u);
+            } else if (st == 1) {
+                mid[pr] = pack_bf16(r0[pr], r1[pr]);
+                r0[pr] -= __uint_as_float(mid[pr] << 16);
+                r1[pr] -= __uint_as_float(mid[pr] & 0xffff0000u);
+            } else {
+                lo[pr] = pack_bf16(r0[pr], r1[pr]);
+            }
+        };
+#pragma unroll
+        for (int p6 = 0; p6 < 6; p6++) {
+            bf16x8 a[NX], b[2];
+#pragma unroll
+            for (int x = 0; x < NX; x++) a[x] = __builtin_bit_cast(bf16x8, as[S][pa[p6]][lk][wi + 32 * x + l32]);
+#pragma unroll
+            for (int y = 0; y < 2; y++) b[y] = __builtin_bit_cast(bf16x8, bs[S][pb[p6]][lk][wj + 32 * y + l32]);
+#pragma unroll
+            for (int m = 0; m < 2 * NX; m++) {
+                acc[m >> 1][m & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m >> 1], b[m & 1], acc[m >> 1][m & 1], 0, 0, 0);
+                // 24 steps over the trip's 12 NX MFMAs
+                const int gm = p6 * 2 * NX + m;
+#pragma unroll
+                for (int n = 2 * gm / NX; n < 2 * (gm + 1) / NX; n++) step(n);
+            }
+        }
+        as[R][0][a_half][a_ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        as[R][1][a_half][a_ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        as[R][2][a_half][a_ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        bs[R][0][b_half][b_ii] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        bs[R][1][b_half][b_ii] = make_uint4(mid[4], mid[5], mid[6], mid[7]);
+        bs[R][2][b_half][b_ii] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        fetch_next(ra[R], rb[R]);
+        __syncthreads();
+    };
+    // after a trip: was that the tile's last chunk?  Then its results go out; true when it was the last tile.
+    auto tile_done = [&]() -> bool {
+        if (--left_m > 0) return false;
+        store_tile<EPI, NX, 2, 4, true>(q, acc, out_m, i0_m + wi, j0_m + wj, l32, lk);
+        if (w_m + (int)gridDim.x >= n_tiles) return true;
+        w_m += gridDim.x;
+        describe_m();
+        zero_acc();
+        return false;
+    };
+    for (;;) {
+        trip(std::integral_constant<int, 0>());
+        if (tile_done()) break;
+        trip(std::integral_constant<int, 1>());
+        if (tile_done()) break;
+    }
 }
 
 // gt[n*npos + pos][co] = g[n][co][pos]: the upstream gradient with the channel innermost, so that the
@@ -2001,6 +2194,41 @@ template <bool AK, bool BK, int EPI, bool VA = false, bool VB = false>
 int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
 {
     GemmParams q = q0;
+    if constexpr (VA || VB) {
+        // Whole tiles of 64 NX x 256, whole chunks in every split, no empty split and tiles for at least
+        // three quarters of the CUs: the eight-wave kernel (the callers have checked the views' alignment).
+        const int nx = big_rows(q.I) / 64;
+        const bool b_ok = VB || BK || (q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0);
+        if (nx && q.J % kBigJ == 0 && q.K % kChunk == 0 && q.k_per_split % kChunk == 0 && b_ok &&
+            (long long)(q.splits - 1) * q.k_per_split < q.K &&
+            (long long)(q.I / (64 * nx)) * (q.J / kBigJ) * q.splits * batch >= 3 * kBigWorkgroups / 4) {
+            q.tile_i = 64 * nx;
+            q.tile_j = kBigJ;
+            q.ni = q.I / q.tile_i;
+            q.nj = q.J / q.tile_j;
+            q.nz = q.splits * batch;
+            if ((long long)q.ni * q.nj <= 16) {
+                q.cluster_of = 2;
+                q.cluster = q.ni * q.nj;
+            } else if (q.nj <= q.ni) {
+                q.cluster_of = 0;
+                q.cluster = q.nj;
+            } else {
+                q.cluster_of = 1;
+                q.cluster = q.ni;
+            }
+            const long long n_wg = (long long)q.ni * q.nj * q.nz;
+            if (n_wg > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
+            const dim3 grid((unsigned)std::min<long long>(n_wg, kBigWorkgroups));
+            if (nx == 4)
+                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 4>), grid, dim3(512), 0, s, q);
+            else if (nx == 3)
+                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 3>), grid, dim3(512), 0, s, q);
+            else
+                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 2>), grid, dim3(512), 0, s, q);
+            return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+        }
+    }
     // A dimension of at most 192 whose last (or only) 128-tile would be at most half full takes tiles of
     // 64: the 2 x 2 wave arrangement would leave half of the waves of such a tile without work (one
     // dimension only, j first).
@@ -2117,8 +2345,12 @@ BwdLayout bwd_layout(const Geometry& g)
     // split the m-reduction of the weight gradient so that all groups' tiles together make about one
     // round of workgroups (three per CU): more splits only add partial sums to write and reduce (C3: 0.85 ms
     // with two rounds, 0.82 with one, 0.85 with a third of one)
-    const long long tiles = (long long)((K + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
-    long long want = 768 / (tiles * b.G.n_groups);
+    // (one per CU where the eight-wave kernel will take that product: the shapes that read col as a view)
+    const bool quads = g.ho % 4 == 0 && g.h_in % 4 == 0 && (g.wo * g.ho) % kChunk == 0 && g.c_out % 2 == 0;
+    const int big_i = !b.fused_k && quads && (2 * g.c_out) % kBigJ == 0 ? big_rows(K) : 0;
+    const long long tiles = big_i ? (long long)(K / big_i) * (2 * g.c_out / kBigJ)
+                                  : (long long)((K + kTile - 1) / kTile) * ((2 * g.c_out + kTile - 1) / kTile);
+    long long want = (big_i ? kBigWorkgroups : 768) / (tiles * b.G.n_groups);
     if (want < 1) want = 1;
     long long per = (b.m_total + want - 1) / want;
     per = (per + kChunk - 1) / kChunk * kChunk;

@@ -343,6 +343,26 @@ def test_backward_linear_4096_shape(capi):
     assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
 
 
+def test_backward_through_the_eight_wave_gemm(capi):
+    """256->128 3x3 at 16x16, batch 64: all three products take the eight-wave kernel with tiles of 256 rows
+    (at the headline shape they take 256, 192 and 128 rows), 192 tiles each.  Against float64 autograd on the
+    GPU, and bit for bit against the 128 x 128 kernel, which the two products that read col take when the
+    input is off its 16-byte alignment."""
+    x, w = wl.make_inputs((64, 256, 16, 16), (128, 256, 3, 3), "kaiming", seed=11)
+    w = (w * 4).contiguous()
+    g = torch.randn((64, 128, 16, 16), generator=torch.Generator().manual_seed(8))
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (1, 1))
+    rx, rw = _fp64_reference_on_gpu(x, w, g, 1)
+    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
+    print(f"256->128 backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
+    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
+    xo = torch.empty(x.numel() + 1, device="cuda")[1:].view(x.shape)
+    xo.copy_(x)
+    gx2, gw2 = capi.conv2d_add_partial_backward(xo, w.cuda(), g.cuda(), 128, (1, 1))
+    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)
+
+
 @pytest.mark.parametrize("mode,zu", [("z", 1), ("yz", 4), ("yz", 8)])
 def test_backward_small_groups_at_the_headline_shape(capi, mode, zu):
     """128->128 3x3 at 16x16 with z accumulation (128 groups of 9 members) and yz accumulation with 4 and 8
