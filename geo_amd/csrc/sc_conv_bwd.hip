@@ -393,6 +393,8 @@ struct SplitStager {
             p = base + (long long)min(i0 + ii, I - 1) * ld + k_begin + 8 * half;
         }
     }
+    // past a chunk that another thread stages
+    __device__ __forceinline__ void skip_chunk() { p += KMAJOR ? (long long)kChunk * ld : (long long)kChunk; }
     // a whole chunk, no branches
     __device__ __forceinline__ void fetch_whole(float (&r)[8])
     {
@@ -497,6 +499,7 @@ struct ViewStager {
             }
         }
     }
+    __device__ __forceinline__ void skip_chunk() { advance(); }
     __device__ __forceinline__ void fetch_whole(float (&r)[8])
     {
         if (KMAJOR) {
@@ -830,51 +833,63 @@ constexpr int kBigWorkgroups = 256;  // one per CU of an MI355X
 // rows of a tile for a result with I rows: 256, 192 or 128 (NX = 4, 3, 2); 0: I is no multiple of any
 inline int big_rows(int I) { return I % 256 == 0 ? 256 : I % 192 == 0 ? 192 : I % 128 == 0 ? 128 : 0; }
 
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VA, bool VB, int NX>
+// KC: chunks per trip.  With NX = 2 a trip of one chunk holds 24 MFMAs per wave, too few for what every trip
+// costs besides (barrier, the latency of the first LDS reads, the loads' address arithmetic); two chunks per
+// trip (KC = 2, 150 KB of LDS) halve that share.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, bool VA, bool VB, int NX, int KC = 1>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_gemm_big(GemmParams q)
 {
     constexpr int RA = 64 * NX, LA = RA + 4, LB = kBigJ + 4;
-    __shared__ uint4 as[2][3][2][LA];
-    __shared__ uint4 bs[2][3][2][LB];
+    constexpr int kUnit = KC * kChunk;  // k per trip
+    __shared__ uint4 as[2][3][2 * KC][LA];
+    __shared__ uint4 bs[2][3][2 * KC][LB];
     const int t = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(t >> 6), lane = t & 63;
     const int wi = (wave >> 2) * (32 * NX), wj = (wave & 3) * 64;
     const int l32 = lane & 31, lk = lane >> 5;
-    // Staging slots: 2 RA (row, k half) pairs of A and 512 of B for 512 threads; with NX < 4 the threads
-    // beyond A's pairs stage a pair a second time (same data to the same place).
+    // Staging slots.  A: 2 KC RA (row, eight k) pairs of a trip, one per thread (with fewer pairs than
+    // threads the rest stage a pair a second time: same data to the same place); a K-major operand has
+    // the lanes along the rows and the pair's k uniform in a wave, an I-major one neighbouring threads
+    // along k.  B: 512 (row, k half) pairs per chunk, every thread one pair of each of the trip's chunks.
+    static_assert(2 * KC * RA <= 512, "one pair of A per thread");
     constexpr bool BK = B_KMAJOR && !VB;
-    const int wa = wave % (RA / 32), ta = t % (2 * RA);
-    const int a_ii = A_KMAJOR ? (wa % NX) * 64 + lane : ta >> 1, a_half = A_KMAJOR ? wa / NX : ta & 1;
+    const int wa = wave % (KC * RA / 32), ta = t % (2 * KC * RA);
+    const int a_ii = A_KMAJOR ? (wa % NX) * 64 + lane : ta / (2 * KC);
+    const int a_q = A_KMAJOR ? wa / NX : ta % (2 * KC);  // which eight k of the trip
     const int b_ii = BK ? (t & 255) : (t >> 1), b_half = BK ? (wave >> 2) : (t & 1);
     typename std::conditional<VA, ViewStager<A_KMAJOR>, SplitStager<A_KMAJOR>>::type sa;
     typename std::conditional<VB, ShiftStager, SplitStager<B_KMAJOR>>::type sb;
 
     const int n_tiles = q.ni * q.nj * q.nz;
-    // the tile whose chunks are being loaded: the stagers point into it, left_f of its chunks are still to load
+    // the tile whose chunks are being loaded: the stagers point into it, left_f of its trips are still to load
     int w_f = blockIdx.x, left_f;
     auto open_tile = [&]() {
         int it, jt, z;
         gemm_tile_of(q, w_f, it, jt, z);
         const int batch = z / q.splits, split = z - batch * q.splits;
         const int k_begin = split * q.k_per_split;
-        left_f = (min(q.K, k_begin + q.k_per_split) - k_begin) / kChunk;
+        left_f = (min(q.K, k_begin + q.k_per_split) - k_begin) / kUnit;
+        const int ka = k_begin + (a_q >> 1) * kChunk;  // A: this thread's chunk of every trip
         if constexpr (VA)
-            sa.init(q, batch, it * RA, k_begin, q.I, a_ii, a_half);
+            sa.init(q, batch, it * RA, ka, q.I, a_ii, a_q & 1);
         else
-            sa.init(q.a + batch * q.a_batch_stride, q.lda, it * RA, k_begin, q.I, a_ii, a_half);
+            sa.init(q.a + batch * q.a_batch_stride, q.lda, it * RA, ka, q.I, a_ii, a_q & 1);
         if constexpr (VB)
             sb.init(q, batch, jt * kBigJ, k_begin, q.J, b_ii, b_half);
         else
             sb.init(q.b + batch * q.b_batch_stride, q.ldb, jt * kBigJ, k_begin, q.J, b_ii, b_half);
     };
-    // the next chunk of the stream into a register set; nothing once the last tile is through
-    auto fetch_next = [&](float (&ra)[8], float (&rb)[8]) {
+    // the next trip's worth of the stream into a register set; nothing once the last tile is through
+    auto fetch_next = [&](float (&ra)[8], float (&rb)[KC][8]) {
         if (left_f == 0) {
             if (w_f + (int)gridDim.x >= n_tiles) return;
             w_f += gridDim.x;
             open_tile();
         }
         sa.fetch_whole(ra);
-        sb.fetch_whole(rb);
+#pragma unroll
+        for (int kc = 1; kc < KC; kc++) sa.skip_chunk();
+#pragma unroll
+        for (int kc = 0; kc < KC; kc++) sb.fetch_whole(rb[kc]);
         --left_f;
     };
     // the tile being multiplied
@@ -885,7 +900,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         gemm_tile_of(q, w_m, it, jt, z);
         const int batch = z / q.splits, split = z - batch * q.splits;
         const int k_begin = split * q.k_per_split;
-        left_m = (min(q.K, k_begin + q.k_per_split) - k_begin) / kChunk;
+        left_m = (min(q.K, k_begin + q.k_per_split) - k_begin) / kUnit;
         i0_m = it * RA;
         j0_m = jt * kBigJ;
         out_m = q.c + batch * q.c_batch_stride + split * q.c_split_stride;
@@ -904,39 +919,50 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     open_tile();
     describe_m();
 
-    // Register set c % 2 holds stream chunk c until it is split and written to LDS buffer c % 2, one trip
-    // before it is multiplied; its loads go out two trips before that.
-    float ra[2][8], rb[2][8];
+    // Register set c % 2 holds trip c of the stream until it is split and written to LDS buffer c % 2, one
+    // trip before it is multiplied; its loads go out two trips before that.
+    constexpr int kPairs = 4 + 4 * KC;  // pairs of elements per thread and trip: A, then B chunk by chunk
+    float ra[2][8], rb[2][KC][8];
+    auto write_split = [&](int buf, const unsigned (&hi)[kPairs], const unsigned (&mid)[kPairs], const unsigned (&lo)[kPairs]) {
+        as[buf][0][a_q][a_ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        as[buf][1][a_q][a_ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
+        as[buf][2][a_q][a_ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+#pragma unroll
+        for (int kc = 0; kc < KC; kc++) {
+            const int o = 4 + 4 * kc;
+            bs[buf][0][2 * kc + b_half][b_ii] = make_uint4(hi[o], hi[o + 1], hi[o + 2], hi[o + 3]);
+            bs[buf][1][2 * kc + b_half][b_ii] = make_uint4(mid[o], mid[o + 1], mid[o + 2], mid[o + 3]);
+            bs[buf][2][2 * kc + b_half][b_ii] = make_uint4(lo[o], lo[o + 1], lo[o + 2], lo[o + 3]);
+        }
+    };
     fetch_next(ra[0], rb[0]);
     fetch_next(ra[1], rb[1]);
     {
-        unsigned hi[8], mid[8], lo[8];
+        unsigned hi[kPairs], mid[kPairs], lo[kPairs];
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             split3(ra[0][2 * c], ra[0][2 * c + 1], hi[c], mid[c], lo[c]);
-            split3(rb[0][2 * c], rb[0][2 * c + 1], hi[4 + c], mid[4 + c], lo[4 + c]);
+#pragma unroll
+            for (int kc = 0; kc < KC; kc++)
+                split3(rb[0][kc][2 * c], rb[0][kc][2 * c + 1], hi[4 + 4 * kc + c], mid[4 + 4 * kc + c], lo[4 + 4 * kc + c]);
         }
-        as[0][0][a_half][a_ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        as[0][1][a_half][a_ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
-        as[0][2][a_half][a_ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        bs[0][0][b_half][b_ii] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-        bs[0][1][b_half][b_ii] = make_uint4(mid[4], mid[5], mid[6], mid[7]);
-        bs[0][2][b_half][b_ii] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        write_split(0, hi, mid, lo);
     }
     fetch_next(ra[0], rb[0]);
     __syncthreads();
 
-    // One trip: stream chunk c out of LDS buffer S, chunk c + 1 (register set S ^ 1) split and written to
-    // the other buffer, the loads of chunk c + 3 into that register set.  Past the end of the stream the
+    // One trip: trip c of the stream out of LDS buffer S, trip c + 1 (register set S ^ 1) split and written
+    // to the other buffer, the loads of trip c + 3 into that register set.  Past the end of the stream the
     // split works on stale registers and its result is never read.
     auto trip = [&](auto set) {
         constexpr int S = decltype(set)::value, R = S ^ 1;
         constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};  // smallest terms first; 0 = hi
-        unsigned hi[8], mid[8], lo[8];
-        float r0[8], r1[8];
+        constexpr int kSteps = 3 * kPairs, kMfmas = 12 * NX * KC;
+        unsigned hi[kPairs], mid[kPairs], lo[kPairs];
+        float r0[kPairs], r1[kPairs];
         auto step = [&](int n) {
             const int pr = n / 3, st = n % 3;
-            const float* src = pr < 4 ? ra[R] : rb[R];
+            const float* src = pr < 4 ? ra[R] : rb[R][(pr - 4) >> 2];
             const int e = 2 * (pr & 3);
             if (st == 0) {
                 hi[pr] = pack_bf16(src[e], src[e + 1]);
@@ -951,34 +977,34 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         };
 #pragma unroll
-        for (int p6 = 0; p6 < 6; p6++) {
-            bf16x8 a[NX], b[2];
+        for (int kc = 0; kc < KC; kc++)
 #pragma unroll
-            for (int x = 0; x < NX; x++) a[x] = __builtin_bit_cast(bf16x8, as[S][pa[p6]][lk][wi + 32 * x + l32]);
+            for (int p6 = 0; p6 < 6; p6++) {
+                bf16x8 a[NX], b[2];
 #pragma unroll
-            for (int y = 0; y < 2; y++) b[y] = __builtin_bit_cast(bf16x8, bs[S][pb[p6]][lk][wj + 32 * y + l32]);
+                for (int x = 0; x < NX; x++)
+                    a[x] = __builtin_bit_cast(bf16x8, as[S][pa[p6]][2 * kc + lk][wi + 32 * x + l32]);
 #pragma unroll
-            for (int m = 0; m < 2 * NX; m++) {
-                acc[m >> 1][m & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m >> 1], b[m & 1], acc[m >> 1][m & 1], 0, 0, 0);
-                // 24 steps over the trip's 12 NX MFMAs
-                const int gm = p6 * 2 * NX + m;
+                for (int y = 0; y < 2; y++)
+                    b[y] = __builtin_bit_cast(bf16x8, bs[S][pb[p6]][2 * kc + lk][wj + 32 * y + l32]);
 #pragma unroll
-                for (int n = 2 * gm / NX; n < 2 * (gm + 1) / NX; n++) step(n);
+                for (int m = 0; m < 2 * NX; m++) {
+                    acc[m >> 1][m & 1] =
+                        __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m >> 1], b[m & 1], acc[m >> 1][m & 1], 0, 0, 0);
+                    // the split's steps spread over the trip's MFMAs
+                    const int gm = (kc * 6 + p6) * 2 * NX + m;
+#pragma unroll
+                    for (int n = kSteps * gm / kMfmas; n < kSteps * (gm + 1) / kMfmas; n++) step(n);
+                }
             }
-        }
-        as[R][0][a_half][a_ii] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        as[R][1][a_half][a_ii] = make_uint4(mid[0], mid[1], mid[2], mid[3]);
-        as[R][2][a_half][a_ii] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        bs[R][0][b_half][b_ii] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-        bs[R][1][b_half][b_ii] = make_uint4(mid[4], mid[5], mid[6], mid[7]);
-        bs[R][2][b_half][b_ii] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        write_split(R, hi, mid, lo);
         fetch_next(ra[R], rb[R]);
         __syncthreads();
     };
-    // after a trip: was that the tile's last chunk?  Then its results go out; true when it was the last tile.
+    // after a trip: was that the tile's last?  Then its results go out; true when it was the last tile.
     auto tile_done = [&]() -> bool {
         if (--left_m > 0) return false;
-        store_tile<EPI, NX, 2, 4, true>(q, acc, out_m, i0_m + wi, j0_m + wj, l32, lk);
+        store_tile<EPI, NX, 2, 2, true>(q, acc, out_m, i0_m + wi, j0_m + wj, l32, lk);
         if (w_m + (int)gridDim.x >= n_tiles) return true;
         w_m += gridDim.x;
         describe_m();
@@ -2199,6 +2225,8 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
         // three quarters of the CUs: the eight-wave kernel (the callers have checked the views' alignment).
         const int nx = big_rows(q.I) / 64;
         const bool b_ok = VB || BK || (q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0);
+        // rows of 128: two chunks per trip where the chunks pair up
+        const bool kc2 = nx == 2 && q.K % (2 * kChunk) == 0 && q.k_per_split % (2 * kChunk) == 0;
         if (nx && q.J % kBigJ == 0 && q.K % kChunk == 0 && q.k_per_split % kChunk == 0 && b_ok &&
             (long long)(q.splits - 1) * q.k_per_split < q.K &&
             (long long)(q.I / (64 * nx)) * (q.J / kBigJ) * q.splits * batch >= 3 * kBigWorkgroups / 4) {
@@ -2224,6 +2252,8 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
                 hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 4>), grid, dim3(512), 0, s, q);
             else if (nx == 3)
                 hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 3>), grid, dim3(512), 0, s, q);
+            else if (kc2)
+                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 2, 2>), grid, dim3(512), 0, s, q);
             else
                 hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 2>), grid, dim3(512), 0, s, q);
             return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
