@@ -17,7 +17,8 @@
 //     dcol[k][m] = sum_j Wd[j][k]  * E[m][j]           Wd = (wp ; -wn)
 // All three run on MFMA kernels (fp32 in, fp32 accumulate, fp32 out) that take each operand either
 // K-major or I-major: k_gemm_split forms every fp32 product from six bf16 MFMA products of a three-way
-// split of the operands (aligned operands), k_gemm_f32 uses v_mfma_f32_32x32x2_f32 (any alignment);
+// split of the operands (aligned operands; k_gemm_big is the same product with eight waves on tiles of
+// up to 256 x 256 for the large results), k_gemm_f32 uses v_mfma_f32_32x32x2_f32 (any alignment);
 // exp and the product with g are fused into the first GEMM's epilogue; the second is split over m
 // and reduced deterministically.
 //
