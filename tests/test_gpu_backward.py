@@ -343,23 +343,33 @@ def test_backward_linear_4096_shape(capi):
     assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
 
 
-def test_backward_through_the_eight_wave_gemm(capi):
-    """256->128 3x3 at 16x16, batch 64: all three products take the eight-wave kernel with tiles of 256 rows
-    (at the headline shape they take 256, 192 and 128 rows), 192 tiles each.  Against float64 autograd on the
-    GPU, and bit for bit against the 128 x 128 kernel, which the two products that read col take when the
-    input is off its 16-byte alignment."""
-    x, w = wl.make_inputs((64, 256, 16, 16), (128, 256, 3, 3), "kaiming", seed=11)
+@pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu", [
+    # all three products with tiles of 256 rows (the headline shape takes 256, 192 and 128 rows), 192 tiles each
+    ((64, 256, 16, 16), (128, 256, 3, 3), 1, "y", 1),
+    # 12 add groups of 96 members: the first product only, 768 tiles of six chunks (short streams per workgroup)
+    ((64, 128, 16, 16), (128, 128, 3, 3), 1, "yz", 32),
+    # a 1 x 1 kernel: one group, 256 tiles for the first and third product, 256 splits of one tile for the second
+    ((256, 256, 16, 16), (128, 256, 1, 1), 0, "y", 1),
+])
+def test_backward_through_the_eight_wave_gemm(capi, shape_x, shape_w, pad, mode, zu):
+    """Shapes whose products take the eight-wave kernel, against float64 autograd on the GPU, and bit for bit
+    against the 128 x 128 kernel, which the products that read col take when the input is off its 16-byte
+    alignment."""
+    x, w = wl.make_inputs(shape_x, shape_w, "kaiming", seed=11)
     w = (w * 4).contiguous()
-    g = torch.randn((64, 128, 16, 16), generator=torch.Generator().manual_seed(8))
-    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (1, 1))
-    rx, rw = _fp64_reference_on_gpu(x, w, g, 1)
+    n, c_out = shape_x[0], shape_w[0]
+    ho = shape_x[2] + 2 * pad - shape_w[2] + 1
+    g = torch.randn((n, c_out, ho, ho), generator=torch.Generator().manual_seed(8))
+    kw = dict(accumulate=mode, z_unit=zu)
+    gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad), **kw)
+    rx, rw = _fp64_reference_on_gpu(x, w, g, pad, mode, zu)
     ex, ew = rel_err(gx, rx), rel_err(gw, rw)
-    print(f"256->128 backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
+    print(f"{shape_x} * {shape_w} {mode} backward: grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
     assert ex <= RTOL and ew <= RTOL, (ex, ew)
     assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
     xo = torch.empty(x.numel() + 1, device="cuda")[1:].view(x.shape)
     xo.copy_(x)
-    gx2, gw2 = capi.conv2d_add_partial_backward(xo, w.cuda(), g.cuda(), 128, (1, 1))
+    gx2, gw2 = capi.conv2d_add_partial_backward(xo, w.cuda(), g.cuda(), 128, (pad, pad), **kw)
     assert torch.equal(gx2, gx) and torch.equal(gw2, gw)
 
 
