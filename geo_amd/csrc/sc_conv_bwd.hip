@@ -2374,9 +2374,9 @@ BwdLayout bwd_layout(const Geometry& g)
         b.fused_splits = (int)(want < 1 ? 1 : want);
     }
     // split the m-reduction of the weight gradient so that all groups' tiles together make about one
-    // round of workgroups (three per CU): more splits only add partial sums to write and reduce (C3: 0.85 ms
-    // with two rounds, 0.82 with one, 0.85 with a third of one)
-    // (one per CU where the eight-wave kernel will take that product: the shapes that read col as a view)
+    // round of workgroups: three per CU for the 128 x 128 kernel (more splits only add partial sums to write
+    // and reduce; C3: 0.85 ms with two rounds, 0.82 with one, 0.85 with a third of one), one per CU where the
+    // eight-wave kernel will take the product (the shapes that read col as a view, with whole tiles)
     const bool quads = g.ho % 4 == 0 && g.h_in % 4 == 0 && (g.wo * g.ho) % kChunk == 0 && g.c_out % 2 == 0;
     const int big_i = !b.fused_k && quads && (2 * g.c_out) % kBigJ == 0 ? big_rows(K) : 0;
     const long long tiles = big_i ? (long long)(K / big_i) * (2 * g.c_out / kBigJ)
