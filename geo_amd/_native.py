@@ -48,6 +48,8 @@ C_API = {
     "geo_sc_layer_tail_backward_workspace_size": (ctypes.c_int, [ctypes.c_int] * 4 + [_SZ]),
     "geo_sc_layer_tail_backward": (ctypes.c_int, [_P, _P] + [ctypes.c_int] * 5 + [_P] * 5 + [ctypes.c_int] + [_P] * 4 +
                                    [ctypes.c_size_t, _P]),
+    "geo_sc_count_stats_workspace_size": (ctypes.c_int, [ctypes.c_int] * 4 + [_SZ]),
+    "geo_sc_count_stats": (ctypes.c_int, [_P] + [ctypes.c_int] * 5 + [_P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_bn_fixed_affine": (ctypes.c_int, [_P] * 4 + [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_longlong] +
                                [_P] * 7),
     "geo_sc_conv2d_add_partial_forward_q7": (ctypes.c_int, [_D, _P, _P, _P, _P, ctypes.c_size_t, _P]),

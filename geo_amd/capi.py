@@ -187,6 +187,24 @@ def layer_tail_backward(counts, grad_out, bit_length, w_n, b_n, mean, invstd, ga
     return grad_y, gg, gb
 
 
+def count_stats(counts, bit_length, stream=None):
+    """geo_sc_count_stats: per-channel mean and biased variance of ``counts / bit_length`` over batch and
+    positions, from exact integer sums.  ``counts``: contiguous int32 GPU tensor (n, c, w, h) or (n, c)."""
+    if not (counts.is_cuda and counts.dtype == torch.int32 and counts.is_contiguous() and counts.dim() in (2, 4)):
+        raise ValueError("counts must be a contiguous int32 GPU tensor (n, c, w, h) or (n, c)")
+    n, c = counts.shape[:2]
+    w, h = (counts.shape[2], counts.shape[3]) if counts.dim() == 4 else (1, 1)
+    need = ctypes.c_size_t()
+    _check(_native.lib().geo_sc_count_stats_workspace_size(n, c, w, h, ctypes.byref(need)),
+           "geo_sc_count_stats_workspace_size")
+    ws = torch.empty(max(need.value, 8), dtype=torch.uint8, device=counts.device)
+    mean = torch.empty(c, dtype=torch.float32, device=counts.device)
+    var = torch.empty(c, dtype=torch.float32, device=counts.device)
+    _check(_native.lib().geo_sc_count_stats(_ptr(counts), n, c, w, h, int(bit_length), _ptr(mean), _ptr(var), _ptr(ws),
+                                            ws.numel(), _stream_ptr(stream)), "geo_sc_count_stats")
+    return mean, var
+
+
 def bn_fixed_affine(mean, var, gamma, beta, eps, elements_per_channel, running_mean=None, running_var=None,
                     eps_grad=1e-5, stream=None):
     """geo_sc_bn_fixed_affine: (w_n, b_n, invstd, scale) of a fixed-point batch norm from channel

@@ -192,18 +192,24 @@ __global__ __launch_bounds__(256) void k_tail_bwd_partial(TailParams q, float* _
     }
 }
 
-__global__ __launch_bounds__(256) void k_tail_bwd_finalize(const float* __restrict__ partial, int c, int splits,
-                                                           float* __restrict__ sums /* [c][2]: dbeta, dgamma */)
+// one wave per channel; the order of the additions is fixed (lane, then the xor tree): deterministic
+__global__ __launch_bounds__(64) void k_tail_bwd_finalize(const float* __restrict__ partial, int c, int splits,
+                                                          float* __restrict__ sums /* [c][2]: dbeta, dgamma */)
 {
-    const int ch = blockIdx.x * 256 + threadIdx.x;
-    if (ch >= c) return;
+    const int ch = blockIdx.x;
     float s1 = 0.0f, s2 = 0.0f;
-    for (int s = 0; s < splits; s++) {
+    for (int s = threadIdx.x; s < splits; s += 64) {
         s1 += partial[((size_t)ch * splits + s) * 2];
         s2 += partial[((size_t)ch * splits + s) * 2 + 1];
     }
-    sums[2 * ch] = s1;
-    sums[2 * ch + 1] = s2;
+    for (int step = 32; step >= 1; step >>= 1) {
+        s1 += __shfl_xor(s1, step);
+        s2 += __shfl_xor(s2, step);
+    }
+    if (threadIdx.x == 0) {
+        sums[2 * ch] = s1;
+        sums[2 * ch + 1] = s2;
+    }
 }
 
 __global__ __launch_bounds__(256) void k_tail_bwd_apply(TailParams q, const float* __restrict__ sums,
@@ -283,6 +289,78 @@ __global__ __launch_bounds__(256) void k_bn_fixed_affine(const float* __restrict
         if (running_mean) running_mean[ch] = __fadd_rn(__fmul_rn(running_mean[ch], 0.9f), __fmul_rn(mu, 0.1f));
         if (running_var)
             running_var[ch] = __fadd_rn(__fmul_rn(running_var[ch], 0.9f), __fmul_rn(__fmul_rn(vr, unbias), 0.1f));
+    }
+}
+
+// Channel statistics of y = counts / bit_length (the mean and the biased variance BatchNorm*_fixed takes of
+// the layer's output, utils_class.py:52-56) from the integer counts: the sums of counts and of their squares
+// are exact in 64-bit integers, so the result does not depend on how the elements are dealt to threads.
+// partial[ch][split][2].  VEC: four counts per load (planes of whole int4 in a 16-byte aligned tensor).
+template <bool VEC>
+__global__ __launch_bounds__(256) void k_count_stats_partial(const int32_t* __restrict__ counts, int n, int c, int plane,
+                                                             int splits, unsigned long long* __restrict__ partial)
+{
+    __shared__ unsigned long long red[2][256];
+    const int ch = blockIdx.y;
+    const long long per_channel = (long long)n * plane;
+    unsigned long long s1 = 0, s2 = 0;
+    if (VEC) {
+        const int quads = plane / 4;
+        const long long total = (long long)n * quads;
+        for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)splits * 256) {
+            const long long item = e / quads;
+            const int r = (int)(e - item * quads);
+            const int4 v = *(const int4*)(counts + (item * c + ch) * plane + 4 * r);
+            s1 += (unsigned long long)((long long)v.x + v.y + v.z + v.w);
+            s2 += (unsigned long long)((long long)v.x * v.x + (long long)v.y * v.y + (long long)v.z * v.z +
+                                       (long long)v.w * v.w);
+        }
+    } else {
+        for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < per_channel; e += (long long)splits * 256) {
+            const long long item = e / plane;
+            const int r = (int)(e - item * plane);
+            const long long v = counts[(item * c + ch) * plane + r];
+            s1 += (unsigned long long)v;
+            s2 += (unsigned long long)(v * v);
+        }
+    }
+    red[0][threadIdx.x] = s1;
+    red[1][threadIdx.x] = s2;
+    __syncthreads();
+    for (int step = 128; step >= 1; step >>= 1) {
+        if ((int)threadIdx.x < step) {
+            red[0][threadIdx.x] += red[0][threadIdx.x + step];
+            red[1][threadIdx.x] += red[1][threadIdx.x + step];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partial[((size_t)ch * splits + blockIdx.x) * 2] = red[0][0];
+        partial[((size_t)ch * splits + blockIdx.x) * 2 + 1] = red[1][0];
+    }
+}
+
+// one wave per channel: mean = S1 / (elements * L), var = S2 / (elements * L^2) - mean^2, formed in double
+// precision from the exact sums and rounded to fp32 once (counts may be negative: the sums are signed)
+__global__ __launch_bounds__(64) void k_count_stats_finalize(const unsigned long long* __restrict__ partial, int splits,
+                                                             double inv_elements_len, double inv_elements_len2,
+                                                             float* __restrict__ mean, float* __restrict__ var)
+{
+    const int ch = blockIdx.x;
+    long long s1 = 0, s2 = 0;
+    for (int s = threadIdx.x; s < splits; s += 64) {
+        s1 += (long long)partial[((size_t)ch * splits + s) * 2];
+        s2 += (long long)partial[((size_t)ch * splits + s) * 2 + 1];
+    }
+    for (int step = 32; step >= 1; step >>= 1) {
+        s1 += __shfl_xor(s1, step);
+        s2 += __shfl_xor(s2, step);
+    }
+    if (threadIdx.x == 0) {
+        const double m = (double)s1 * inv_elements_len;
+        const double v = (double)s2 * inv_elements_len2 - m * m;
+        mean[ch] = (float)m;
+        var[ch] = (float)(v > 0.0 ? v : 0.0);
     }
 }
 
@@ -409,11 +487,48 @@ extern "C" int geo_sc_layer_tail_backward(const int32_t* counts, const float* gr
     float* partial = (float*)workspace;
     float* sums = partial + (size_t)2 * c * q.splits;
     hipLaunchKernelGGL(k_tail_bwd_partial, dim3(q.splits, c), dim3(256), 0, s, q, partial);
-    hipLaunchKernelGGL(k_tail_bwd_finalize, dim3((c + 255) / 256), dim3(256), 0, s, partial, c, q.splits, sums);
+    hipLaunchKernelGGL(k_tail_bwd_finalize, dim3(c), dim3(64), 0, s, partial, c, q.splits, sums);
     const long long total = (long long)n * c * w * h;
     long long blocks = (total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
     hipLaunchKernelGGL(k_tail_bwd_apply, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma, grad_beta);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_count_stats_workspace_size(int n, int c, int w, int h, size_t* bytes)
+{
+    if (!bytes || n < 1 || c < 1 || w < 1 || h < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
+    *bytes = sizeof(unsigned long long) * 2 * (size_t)c * tail_splits(n, c, w, h);
+    return GEO_SC_OK;
+}
+
+extern "C" int geo_sc_count_stats(const int32_t* counts, int n, int c, int w, int h, int bit_length, float* mean,
+                                  float* var, void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    if (!counts || !mean || !var) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (n < 1 || c < 1 || w < 1 || h < 1 || c > 65535) return GEO_SC_ERR_INVALID_ARGUMENT;
+    switch (bit_length) {
+    case 8: case 16: case 32: case 64: case 128: case 256: break;
+    default: return GEO_SC_ERR_BIT_LENGTH;
+    }
+    size_t need = 0;
+    geo_sc_count_stats_workspace_size(n, c, w, h, &need);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 7u)) return GEO_SC_ERR_WORKSPACE;
+    // the four-count loads need 16-byte aligned planes
+    const int plane = w * h;
+    const bool vec_plane = plane % 4 == 0 && ((uintptr_t)counts & 15u) == 0;
+    const int splits = tail_splits(n, c, w, h);
+    hipStream_t s = (hipStream_t)stream;
+    unsigned long long* partial = (unsigned long long*)workspace;
+    if (vec_plane)
+        hipLaunchKernelGGL(k_count_stats_partial<true>, dim3(splits, c), dim3(256), 0, s, counts, n, c, plane, splits,
+                           partial);
+    else
+        hipLaunchKernelGGL(k_count_stats_partial<false>, dim3(splits, c), dim3(256), 0, s, counts, n, c, plane, splits,
+                           partial);
+    const double elements = (double)n * plane;
+    hipLaunchKernelGGL(k_count_stats_finalize, dim3(c), dim3(64), 0, s, partial, splits,
+                       1.0 / (elements * bit_length), 1.0 / (elements * bit_length * (double)bit_length), mean, var);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

@@ -93,18 +93,24 @@ class _SCConvBlock(torch.autograd.Function):
         from . import capi
         x = activation.detach().float().contiguous()
         w = weight.detach().float().contiguous()
+        torch_stats = conv_kw.get("torch_stats", False)
+        conv_kw = {k: v for k, v in conv_kw.items() if k != "torch_stats"}
         L = conv_kw["bit_length"]
         counts = capi.conv2d_add_partial_forward(x, w, **conv_kw)
-        y = counts * (1.0 / L)   # one kernel; exact: L is a power of two
-        dims = (0, 2, 3)
-        mean, var = y.mean(dim=dims), y.var(dim=dims, unbiased=False)
+        if torch_stats:
+            # the two PyTorch reductions BatchNorm*_fixed itself runs (utils_class.py:52-56)
+            y = counts * (1.0 / L)   # exact: L is a power of two
+            mean, var = y.mean(dim=(0, 2, 3)), y.var(dim=(0, 2, 3), unbiased=False)
+        else:
+            # the same statistics from exact integer sums: no y in memory, no dependence on a reduction order
+            mean, var = capi.count_stats(counts, L)
         # One launch for what BatchNorm*_fixed computes per channel (utils_class.py:52-62) and for what
         # its F.batch_norm(x, running_mean, running_var, weight, bias, training=True) call
         # (utils_class.py:49) does to the running statistics: that function's default momentum 0.1
         # and, for the gradient, its default eps 1e-5; the batch counter is not touched.
         w_n, b_n, invstd, bn.scale = capi.bn_fixed_affine(
             mean, var, gamma.detach().float().contiguous() if gamma is not None else None,
-            beta.detach().float().contiguous() if beta is not None else None, bn.eps, y.numel() // y.shape[1],
+            beta.detach().float().contiguous() if beta is not None else None, bn.eps, counts.numel() // counts.shape[1],
             bn.running_mean, bn.running_var)
         act, _ = capi.layer_epilogue(counts, L, w_n, b_n, relu=relu, pool=pool, hardtanh=hardtanh, quant7=quant7)
         ctx.save_for_backward(x, w, counts, w_n, b_n, mean, invstd,
@@ -132,12 +138,15 @@ class _SCConvBlock(torch.autograd.Function):
 
 
 def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_unit=8, load_wait_w=2, load_wait_a=2,
-                  prec=7, relu=False, pool=True, hardtanh=True, quant7=True):
+                  prec=7, relu=False, pool=True, hardtanh=True, quant7=True, torch_stats=False):
     """``hardtanh(pool(relu(bn(conv(input)))))`` of a ``Conv2d_Add_Partial`` and a
     ``BatchNorm2d_fixed`` / ``BatchNorm1d_fixed`` in training mode, fused (LFSR generators, GPU
     tensors).  Same in-place quantisation of ``input.data`` and ``conv.weight.data`` as
     ``Conv2d_Add_Partial.forward`` (utils_class.py:32-33).  The output is already quantised to 7
-    bits (the next layer would do that to its input anyway) unless ``quant7=False``."""
+    bits (the next layer would do that to its input anyway) unless ``quant7=False``.  The batch statistics are
+    the correctly rounded mean and variance of ``counts / L`` (exact integer sums, one HIP kernel);
+    ``torch_stats=True`` takes them from PyTorch's float reductions as the module chain does (the two can differ
+    in the last bit, which the 8-bit rounding of the affine hides except at a rounding boundary)."""
     if forward not in ("1d_bin", "z_bin", "yz_bin") or not input.is_cuda:
         raise NotImplementedError("sc_conv_block: LFSR modes 1d_bin / z_bin / yz_bin on GPU tensors")
     if tuple(conv.stride) != (1, 1):
@@ -148,6 +157,6 @@ def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_un
     kw = dict(bit_length=2 ** err, padding=(int(conv.padding[0]), int(conv.padding[1])),
               total_width=utils_functional.prec_default, load_width=int(load_unit), load_wait_w=int(load_wait_w),
               load_wait_a=int(load_wait_a if mode == "yz" else load_wait_w), accumulate=mode,
-              z_unit=max(1, min(int(z_unit), conv.weight.shape[1])))
+              z_unit=max(1, min(int(z_unit), conv.weight.shape[1])), torch_stats=bool(torch_stats))
     gamma, beta = (bn.weight, bn.bias) if bn.affine else (None, None)
     return _SCConvBlock.apply(input, conv.weight, gamma, beta, bn, kw, relu, pool, hardtanh, quant7)

@@ -268,6 +268,18 @@ GEO_SC_API int geo_sc_layer_tail_backward(const int32_t* counts, const float* gr
                                           size_t workspace_bytes, geo_sc_stream_t stream);
 
 /*
+ * The channel statistics BatchNorm2d_fixed / BatchNorm1d_fixed take of an SC layer's output
+ * (utils_class.py:52-56: mean and biased variance over batch and positions of y = counts / bit_length), from the
+ * integer counts (n, c, w, h): the sums of the counts and of their squares are exact 64-bit integers, the two
+ * results are formed from them in double precision and rounded to fp32 once, so they do not depend on a
+ * reduction order.  mean, var: c floats each on the device.  Workspace: geo_sc_count_stats_workspace_size
+ * bytes, 8-byte aligned.
+ */
+GEO_SC_API int geo_sc_count_stats_workspace_size(int n, int c, int w, int h, size_t* bytes);
+GEO_SC_API int geo_sc_count_stats(const int32_t* counts, int n, int c, int w, int h, int bit_length, float* mean,
+                                  float* var, void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
+
+/*
  * The per-channel fixed-point affine of BatchNorm2d_fixed / BatchNorm1d_fixed from channel statistics
  * (utils_class.py:52-62, quantize_shift utils_functional.py:41-57) in one launch:
  * w = gamma / sqrt(var + eps), b = beta - mean * gamma / sqrt(var + eps), both rounded to 8 bits under

@@ -192,3 +192,47 @@ def test_tail_backward_matches_torch_autograd():
         for got, ref in ((gy, y.grad), (gg, bn.weight.grad), (gb, bn.bias.grad)):
             err = (got - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
             assert err < 2e-5, (shape, err)
+
+
+def test_count_stats_are_the_correctly_rounded_channel_statistics():
+    """geo_sc_count_stats against float64 mean and biased variance of counts / L (utils_class.py:52-56):
+    equal to the float64 result rounded to fp32, for whole-quad planes, ragged planes, an unaligned
+    tensor, single-position layers and negative counts."""
+    from geo_amd import capi
+    for shape, L in [((32, 6, 8, 8), 64), ((5, 3, 7, 5), 32), ((256, 32, 16, 16), 64), ((16, 10, 1, 1), 128),
+                     ((3, 70, 4, 4), 256)]:
+        g = torch.Generator().manual_seed(shape[1])
+        counts = torch.randint(-5 * L, 5 * L + 1, shape, generator=g, dtype=torch.int32).cuda()
+        y = counts.double() / L
+        dims = (0, 2, 3)
+        ref_mean, ref_var = y.mean(dims), y.var(dims, unbiased=False)
+        mean, var = capi.count_stats(counts, L)
+        assert torch.equal(mean, ref_mean.float()), shape
+        # the variance is a difference of two exact terms rounded once: within one fp32 step of the fp64 value
+        assert torch.allclose(var.double(), ref_var, rtol=2e-7, atol=0), shape
+        # a tensor that does not start on a 16-byte boundary takes the one-count loads: same bits
+        off = torch.empty(counts.numel() + 1, dtype=torch.int32, device="cuda")[1:].view(shape)
+        off.copy_(counts)
+        m2, v2 = capi.count_stats(off, L)
+        assert torch.equal(m2, mean) and torch.equal(v2, var), shape
+    const = torch.full((4, 2, 4, 4), 37, dtype=torch.int32, device="cuda")
+    mean, var = capi.count_stats(const, 64)
+    assert torch.equal(mean, torch.full((2,), 37 / 64, device="cuda")) and torch.equal(var, torch.zeros(2, device="cuda"))
+
+
+def test_fused_block_with_either_source_of_batch_statistics():
+    """sc_conv_block with the statistics from the exact integer sums (default) and from PyTorch's float
+    reductions (torch_stats=True): the same block output and running statistics to fp32 rounding."""
+    from geo_amd import utils_class
+    outs = []
+    for torch_stats in (False, True):
+        torch.manual_seed(3)
+        conv = utils_class.Conv2d_Add_Partial(8, 12, 3, padding=1, bias=False).cuda()
+        bn = utils_class.BatchNorm2d_fixed(12).cuda().train()
+        x = torch.rand(16, 8, 8, 8, generator=torch.Generator().manual_seed(4)).cuda()
+        out = utils_class.sc_conv_block(conv, bn, x, err=6, torch_stats=torch_stats)
+        outs.append((out.detach().clone(), bn.running_mean.clone(), bn.running_var.clone()))
+    assert torch.allclose(outs[0][0], outs[1][0], atol=1.0 / 128 + 1e-6)   # at most one step of the 7-bit output
+    assert (outs[0][0] != outs[1][0]).float().mean().item() < 0.01
+    assert torch.allclose(outs[0][1], outs[1][1], rtol=1e-5, atol=1e-7)
+    assert torch.allclose(outs[0][2], outs[1][2], rtol=1e-5, atol=1e-7)
