@@ -80,10 +80,11 @@ struct GemmParams {
     long long a_rows_batch;
     int a_item, a_skip;
     // B as a view of E shifted by whole image rows (kernels with VB; the input-gradient product summed over
-    // the kernel rows u): k = u * sh_j + j, and column i = (n, p, b) of B is row (n, p + sh_pad - u, b) of E
-    // (sh_j floats per row of E, ldb apart) where that output row exists, zero elsewhere (read from sh_zero).
+    // the sh_wk kernel rows u): chunk c of the k dimension holds the columns j = (c / sh_wk) * kChunk ... of kernel
+    // row u = c % sh_wk, and column i = (n, p, b) of B is row (n, p + sh_pad - u, b) of E (sh_j floats per row
+    // of E, ldb apart) where that output row exists, zero elsewhere (read from sh_zero).
     const float* __restrict__ sh_zero;
-    int sh_j, sh_wo, sh_ho, sh_win, sh_pad;
+    int sh_j, sh_wo, sh_ho, sh_win, sh_pad, sh_wk;
     // tile extent per workgroup in i and j: kTile, or kTile / 2 in at most one of them (set by
     // launch_gemm): the four waves then line up along the other dimension
     int tile_i, tile_j;
@@ -551,11 +552,13 @@ struct ViewStager {
 };
 
 // Stager of the B operand of the input-gradient product when it sums over the kernel rows inside the GEMM
-// (GemmParams::sh_*): the k dimension runs over (u, j), and for kernel row u the column (n, p, b) of B is
-// the row (n, p + pad - u, b) of E.  I-major: a thread keeps one column and eight consecutive j; when j passes
-// the end of a row of E the thread moves to the row of the next u.  Columns whose output row does not exist
-// for a u read a block of zeros instead (no select on the loaded data, so nothing waits for the load).
-// sh_j is a multiple of kChunk: no chunk straddles two u, and there are no partial chunks.
+// (GemmParams::sh_*): the k dimension runs over chunks of kChunk columns j of E with the kernel row u as the
+// fast index, and for kernel row u the column (n, p, b) of B is the row (n, p + pad - u, b) of E.  I-major: a
+// thread keeps one column and eight consecutive j; from chunk to chunk it moves one image row up, and after the
+// last kernel row on to the next columns - so the rows of E that the kernel rows share are read in consecutive
+// chunks, while they are still in the CU's cache.  Columns whose output row does not exist for a u read a block
+// of zeros instead (no select on the loaded data, so nothing waits for the load).  sh_j is a multiple of
+// kChunk: there are no partial chunks.
 struct ShiftStager {
     const float* e_rows;   // E of this batch member
     const float* zero;
@@ -563,7 +566,7 @@ struct ShiftStager {
     long long ld;
     int j, u, prow, wo;  // j: this thread's first column of E in the current chunk; prow: p + pad
     long long row0;                 // (n * wo + prow + pad) * ho + b: the row of E for u = 0
-    int half, ii, sh_j, ho;
+    int half, ii, sh_j, ho, n_u;
 
     __device__ __forceinline__ void point()
     {
@@ -574,6 +577,7 @@ struct ShiftStager {
     {
         ii = ii_;
         half = half_;
+        n_u = q.sh_wk;
         e_rows = q.b + batch * q.b_batch_stride;
         zero = q.sh_zero;
         ld = q.ldb;
@@ -586,17 +590,17 @@ struct ShiftStager {
         const int pr = rem / q.sh_ho, b = rem - pr * q.sh_ho;
         prow = pr + q.sh_pad;
         row0 = ((long long)n * wo + prow) * ho + b;
-        const int k = k_begin + 8 * half;
-        u = k / sh_j;
-        j = k - u * sh_j;
+        // chunk c of the k dimension: kernel row c % w_k of the columns (c / w_k) * kChunk ...
+        const int chunk = k_begin / kChunk;
+        u = chunk % n_u;
+        j = (chunk / n_u) * kChunk + 8 * half;
         point();
     }
     __device__ __forceinline__ void advance()
     {
-        j += kChunk;
-        if (j >= sh_j) {
-            j -= sh_j;
-            ++u;
+        if (++u == n_u) {
+            u = 0;
+            j += kChunk;
         }
         point();
     }
@@ -1533,8 +1537,10 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad_tiled(const float* __restr
 __global__ __launch_bounds__(64) void k_zero_block(float* __restrict__ p) { p[threadIdx.x] = 0.0f; }
 
 // The A operand of the input-gradient product summed over the kernel rows inside the GEMM (y
-// accumulation: group = kernel column v, members (ci, u)): wdx[g][(u * 2 c_out + j)][ci] = wd[g][j][(ci, u)],
-// i.e. clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one.
+// accumulation: group = kernel column v, members (ci, u)): wdx[g][k][ci] = wd[g][j][(ci, u)], i.e.
+// clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one, with the
+// kernel row as the fast index over chunks of kChunk columns, k = ((j / kChunk) * w_k + u) * kChunk + j % kChunk:
+// consecutive chunks of the product then read the same columns of E one image row apart (ShiftStager).
 __global__ __launch_bounds__(256) void k_weight_dx_operand(const float* __restrict__ w, float* __restrict__ wdx, int g0,
                                                            int c_out, int c_in, int w_k, int h_k, size_t g_stride)
 {
@@ -1544,7 +1550,7 @@ __global__ __launch_bounds__(256) void k_weight_dx_operand(const float* __restri
     const int v = g0 + blockIdx.y;
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
         const int ci = e % c_in, r = e / c_in;
-        const int j = r % J, u = r / J;
+        const int chunk = r / kChunk, u = chunk % w_k, j = (chunk / w_k) * kChunk + r % kChunk;
         const int co = j >= c_out ? j - c_out : j;
         const float wv = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v];
         dst[e] = j < c_out ? fminf(fmaxf(wv, 0.0f), 100.0f) : fminf(fmaxf(wv, -100.0f), 0.0f);
@@ -2650,6 +2656,7 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
             q3.a_batch_stride = (long long)L.w_v; q3.b_batch_stride = (long long)L.e_v;
             q3.c_batch_stride = (long long)g.c_in * m2;
             q3.sh_zero = zero; q3.sh_j = J; q3.sh_wo = g.wo; q3.sh_ho = g.ho; q3.sh_win = g.w_in; q3.sh_pad = g.pad_w;
+            q3.sh_wk = g.w_k;
             if ((rc = launch_gemm<true, false, EPI_STORE, false, true>(q3, nv, s)) != GEO_SC_OK) return rc;
             const long long quads = (long long)g.n * g.c_in * g.w_in * g.h_in / 4;
             hipLaunchKernelGGL(k_shift_sum_v4, dim3(grid1d(quads)), dim3(256), 0, s, dcol, gx, quads, g.n, g.c_in, g.w_in,
