@@ -192,6 +192,98 @@ __global__ __launch_bounds__(256) void k_tail_bwd_partial(TailParams q, float* _
     }
 }
 
+// The pooled tail with even plane sides, one 2 x 2 pool window per thread: the window's four counts as two
+// 8-byte loads, the pooled value and its hardtanh mask once for the four elements (the element-wise kernels
+// recompute them per element), d[0..3] and xhat[0..3] of the window in row order.
+struct TailWindow {
+    float d[4], xhat[4];
+};
+__device__ __forceinline__ TailWindow tail_window(const TailParams& q, long long nc, int a, int b, float wn, float bn,
+                                                  float mu, float is)
+{
+    const bool relu = q.flags & GEO_SC_EPI_RELU;
+    const int32_t* src = q.counts + (nc * q.w + 2 * a) * q.h + 2 * b;
+    const int2 r0 = *(const int2*)src, r1 = *(const int2*)(src + q.h);
+    const int cnt[4] = {r0.x, r0.y, r1.x, r1.y};
+    float v[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = affine(cnt[k], q.inv_len, wn, bn, relu);
+    const float pooled = __fadd_rn(__fadd_rn(__fadd_rn(v[0], v[1]), v[2]), v[3]) / 4.0f;
+    float g = q.gout[(nc * q.wo + a) * q.ho + b];
+    if ((q.flags & GEO_SC_EPI_HARDTANH01) && !(pooled > 0.0f && pooled < 1.0f)) g = 0.0f;
+    g *= 0.25f;
+    TailWindow t;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        t.d[k] = (relu && !(affine(cnt[k], q.inv_len, wn, bn, false) > 0.0f)) ? 0.0f : g;
+        t.xhat[k] = ((float)cnt[k] * q.inv_len - mu) * is;
+    }
+    return t;
+}
+
+__global__ __launch_bounds__(256) void k_tail_bwd_partial_pool(TailParams q, float* __restrict__ partial)
+{
+    __shared__ float red[2][256];
+    const int ch = blockIdx.y;
+    const float wn = q.w_n[ch], bn = q.b_n[ch], mu = q.mean[ch], is = q.invstd[ch];
+    const int windows = q.wo * q.ho;
+    const long long per_channel = (long long)q.n * windows;
+    float s1 = 0.0f, s2 = 0.0f;
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < per_channel; e += (long long)q.splits * 256) {
+        const int item = (int)(e / windows), r = (int)(e - (long long)item * windows);
+        const int a = r / q.ho, b = r - a * q.ho;
+        const TailWindow t = tail_window(q, (long long)item * q.c + ch, a, b, wn, bn, mu, is);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            s1 += t.d[k];
+            s2 += t.d[k] * t.xhat[k];
+        }
+    }
+    red[0][threadIdx.x] = s1;
+    red[1][threadIdx.x] = s2;
+    __syncthreads();
+    for (int step = 128; step >= 1; step >>= 1) {
+        if ((int)threadIdx.x < step) {
+            red[0][threadIdx.x] += red[0][threadIdx.x + step];
+            red[1][threadIdx.x] += red[1][threadIdx.x + step];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partial[((size_t)ch * q.splits + blockIdx.x) * 2] = red[0][0];
+        partial[((size_t)ch * q.splits + blockIdx.x) * 2 + 1] = red[1][0];
+    }
+}
+
+__global__ __launch_bounds__(256) void k_tail_bwd_apply_pool(TailParams q, const float* __restrict__ sums,
+                                                             float* __restrict__ grad_y, float* __restrict__ grad_gamma,
+                                                             float* __restrict__ grad_beta)
+{
+    const int windows = q.wo * q.ho;
+    const long long total = (long long)q.n * q.c * windows;
+    const float inv_m = 1.0f / (float)((long long)q.n * q.w * q.h);
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)gridDim.x * 256) {
+        const long long nc = e / windows;
+        const int r = (int)(e - nc * windows);
+        const int a = r / q.ho, b = r - a * q.ho;
+        const int ch = (int)(nc % q.c);
+        const float is = q.invstd[ch];
+        const TailWindow t = tail_window(q, nc, a, b, q.w_n[ch], q.b_n[ch], q.mean[ch], is);
+        const float gm = (q.gamma ? q.gamma[ch] : 1.0f) * is, sb = sums[2 * ch] * inv_m, sg = sums[2 * ch + 1] * inv_m;
+        float o[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) o[k] = gm * (t.d[k] - sb - t.xhat[k] * sg);
+        float* dst = grad_y + (nc * q.w + 2 * a) * q.h + 2 * b;
+        *(float2*)dst = make_float2(o[0], o[1]);
+        *(float2*)(dst + q.h) = make_float2(o[2], o[3]);
+    }
+    if (blockIdx.x == 0)
+        for (int ch = threadIdx.x; ch < q.c; ch += 256) {
+            if (grad_beta) grad_beta[ch] = sums[2 * ch];
+            if (grad_gamma) grad_gamma[ch] = sums[2 * ch + 1];
+        }
+}
+
 // one wave per channel; the order of the additions is fixed (lane, then the xor tree): deterministic
 __global__ __launch_bounds__(64) void k_tail_bwd_finalize(const float* __restrict__ partial, int c, int splits,
                                                           float* __restrict__ sums /* [c][2]: dbeta, dgamma */)
@@ -486,12 +578,24 @@ extern "C" int geo_sc_layer_tail_backward(const int32_t* counts, const float* gr
     hipStream_t s = (hipStream_t)stream;
     float* partial = (float*)workspace;
     float* sums = partial + (size_t)2 * c * q.splits;
-    hipLaunchKernelGGL(k_tail_bwd_partial, dim3(q.splits, c), dim3(256), 0, s, q, partial);
+    // one pool window per thread where the plane is made of whole windows and rows of counts, of the incoming
+    // gradient's source and of the result start on 8-byte boundaries
+    const bool windows = (flags & GEO_SC_EPI_POOL2) && w % 2 == 0 && h % 2 == 0 && ((uintptr_t)counts & 7u) == 0 &&
+                         ((uintptr_t)grad_y & 7u) == 0;
+    if (windows)
+        hipLaunchKernelGGL(k_tail_bwd_partial_pool, dim3(q.splits, c), dim3(256), 0, s, q, partial);
+    else
+        hipLaunchKernelGGL(k_tail_bwd_partial, dim3(q.splits, c), dim3(256), 0, s, q, partial);
     hipLaunchKernelGGL(k_tail_bwd_finalize, dim3(c), dim3(64), 0, s, partial, c, q.splits, sums);
-    const long long total = (long long)n * c * w * h;
+    const long long total = (long long)n * c * w * h / (windows ? 4 : 1);
     long long blocks = (total + 255) / 256;
     if (blocks > 256 * 32) blocks = 256 * 32;
-    hipLaunchKernelGGL(k_tail_bwd_apply, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma, grad_beta);
+    if (windows)
+        hipLaunchKernelGGL(k_tail_bwd_apply_pool, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma,
+                           grad_beta);
+    else
+        hipLaunchKernelGGL(k_tail_bwd_apply, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma,
+                           grad_beta);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
