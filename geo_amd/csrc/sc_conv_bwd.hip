@@ -54,7 +54,7 @@ constexpr int kTile = 128;   // block tile in I and J
 constexpr int kChunk = 16;   // K per LDS stage
 constexpr int kLd = 132;     // LDS row stride in floats: rows stay 16-byte aligned for float4 stores
 
-enum Epilogue { EPI_STORE = 0, EPI_EXP_TIMES_G = 1 };
+enum Epilogue { EPI_STORE = 0, EPI_EXP_TIMES_G = 1, EPI_EXP_TIMES_G_PLANES = 2 };
 
 struct GemmParams {
     const float* __restrict__ a;
@@ -70,8 +70,10 @@ struct GemmParams {
     long long c_split_stride;
     long long a_batch_stride, b_batch_stride, c_batch_stride;
     // EPI_EXP_TIMES_G: c[i][j] = g[i * c_out + (j % c_out)] * exp(-acc), g = upstream gradient stored [m][c_out]
+    // EPI_EXP_TIMES_G_PLANES (g_planes set, eight-wave kernel only): the same from the gradient as the caller
+    // has it, [n][c_out][npos] with i = n * npos + position; npos a multiple of 32, g 16-byte aligned
     const float* __restrict__ g;
-    int c_out, npos;
+    int c_out, npos, g_planes;
     // A as a view of the shifted input planes instead of a materialised col (kernels with VA): row r of
     // batch member z starts a_rows[z * a_rows_batch + r] elements into `a`, and position m of that row lies
     // m + (m / a_item) * a_skip elements further (a_item positions per item, a_skip elements between the
@@ -202,6 +204,23 @@ __device__ __forceinline__ void store_tile(const GemmParams& q, const floatx16 (
 #pragma unroll
     for (int b0 = 0; b0 < NB; b0 += BB) {
         float gv[BB][16];
+        if (EPI == EPI_EXP_TIMES_G_PLANES) {
+            // a lane's 16 rows are four runs of four consecutive positions of one item: four 16-byte loads from
+            // the plane of its channel (the 32 rows of a block lie in one item)
+#pragma unroll
+            for (int bb = 0; bb < BB; bb++) {
+                const int x = (b0 + bb) / NYd, y = (b0 + bb) % NYd;
+                const int j = jw + y * 32 + l32, ib = iw + x * 32 + 4 * lk;
+                const int co = j >= q.c_out ? j - q.c_out : j;
+                const int item = ib / q.npos;
+                const float* gp = q.g + ((long long)item * q.c_out + co) * q.npos + (ib - item * q.npos);
+#pragma unroll
+                for (int rg = 0; rg < 4; rg++) {
+                    const float4 v = *(const float4*)(gp + 8 * rg);
+                    gv[bb][4 * rg] = v.x; gv[bb][4 * rg + 1] = v.y; gv[bb][4 * rg + 2] = v.z; gv[bb][4 * rg + 3] = v.w;
+                }
+            }
+        }
         if (EPI == EPI_EXP_TIMES_G) {
 #pragma unroll
             for (int bb = 0; bb < BB; bb++) {
@@ -226,7 +245,7 @@ __device__ __forceinline__ void store_tile(const GemmParams& q, const floatx16 (
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int di = 8 * (r >> 2) + (r & 3);
-                const float v = EPI == EPI_EXP_TIMES_G ? gv[bb][r] * exp_neg(acc[x][y][r]) : acc[x][y][r];
+                const float v = EPI != EPI_STORE ? gv[bb][r] * exp_neg(acc[x][y][r]) : acc[x][y][r];
                 if (WHOLE)
                     op[(long long)di * q.ldc] = v;
                 else if (j_ok && ib + di < q.I)
@@ -2223,20 +2242,28 @@ int grid1d(long long total)
 
 // VA: the A operand is a view of the shifted input planes (GemmParams::a_rows); the caller has checked that
 // its rows and chunks are 16-byte aligned.
+// Whether a product of views takes the eight-wave kernel, and with which NX (0: no): whole tiles of 64 NX x 256,
+// whole chunks in every split, no empty split, an aligned B where B is read along k, and tiles for at least three
+// quarters of the CUs (the callers have checked the views' alignment).
+inline int big_tile_nx(const GemmParams& q, int batch, bool b_along_k)
+{
+    const int nx = big_rows(q.I) / 64;
+    const bool b_ok = !b_along_k || (q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0);
+    const bool ok = nx && q.J % kBigJ == 0 && q.K % kChunk == 0 && q.k_per_split % kChunk == 0 && b_ok &&
+                    (long long)(q.splits - 1) * q.k_per_split < q.K &&
+                    (long long)(q.I / (64 * nx)) * (q.J / kBigJ) * q.splits * batch >= 3 * kBigWorkgroups / 4;
+    return ok ? nx : 0;
+}
+
 template <bool AK, bool BK, int EPI, bool VA = false, bool VB = false>
 int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
 {
     GemmParams q = q0;
     if constexpr (VA || VB) {
-        // Whole tiles of 64 NX x 256, whole chunks in every split, no empty split and tiles for at least
-        // three quarters of the CUs: the eight-wave kernel (the callers have checked the views' alignment).
-        const int nx = big_rows(q.I) / 64;
-        const bool b_ok = VB || BK || (q.ldb % 4 == 0 && ((uintptr_t)q.b & 15) == 0 && q.b_batch_stride % 4 == 0);
+        const int nx = big_tile_nx(q, batch, !VB && !BK);
         // rows of 128: two chunks per trip where the chunks pair up
         const bool kc2 = nx == 2 && q.K % (2 * kChunk) == 0 && q.k_per_split % (2 * kChunk) == 0;
-        if (nx && q.J % kBigJ == 0 && q.K % kChunk == 0 && q.k_per_split % kChunk == 0 && b_ok &&
-            (long long)(q.splits - 1) * q.k_per_split < q.K &&
-            (long long)(q.I / (64 * nx)) * (q.J / kBigJ) * q.splits * batch >= 3 * kBigWorkgroups / 4) {
+        if (nx) {
             q.tile_i = 64 * nx;
             q.tile_j = kBigJ;
             q.ni = q.I / q.tile_i;
@@ -2255,17 +2282,29 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
             const long long n_wg = (long long)q.ni * q.nj * q.nz;
             if (n_wg > 0x7fffffffLL) return GEO_SC_ERR_UNSUPPORTED;
             const dim3 grid((unsigned)std::min<long long>(n_wg, kBigWorkgroups));
-            if (nx == 4)
-                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 4>), grid, dim3(512), 0, s, q);
-            else if (nx == 3)
-                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 3>), grid, dim3(512), 0, s, q);
-            else if (kc2)
-                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 2, 2>), grid, dim3(512), 0, s, q);
-            else
-                hipLaunchKernelGGL((k_gemm_big<AK, BK, EPI, VA, VB, 2>), grid, dim3(512), 0, s, q);
+            auto launch = [&](auto epi) {
+                constexpr int E = decltype(epi)::value;
+                if (nx == 4)
+                    hipLaunchKernelGGL((k_gemm_big<AK, BK, E, VA, VB, 4>), grid, dim3(512), 0, s, q);
+                else if (nx == 3)
+                    hipLaunchKernelGGL((k_gemm_big<AK, BK, E, VA, VB, 3>), grid, dim3(512), 0, s, q);
+                else if (kc2)
+                    hipLaunchKernelGGL((k_gemm_big<AK, BK, E, VA, VB, 2, 2>), grid, dim3(512), 0, s, q);
+                else
+                    hipLaunchKernelGGL((k_gemm_big<AK, BK, E, VA, VB, 2>), grid, dim3(512), 0, s, q);
+            };
+            if constexpr (EPI == EPI_EXP_TIMES_G) {
+                if (q.g_planes)
+                    launch(std::integral_constant<int, EPI_EXP_TIMES_G_PLANES>());
+                else
+                    launch(std::integral_constant<int, EPI>());
+            } else {
+                launch(std::integral_constant<int, EPI>());
+            }
             return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
         }
     }
+    if (EPI == EPI_EXP_TIMES_G && q.g_planes) return GEO_SC_ERR_UNSUPPORTED;  // (the caller decides with big_tile_nx)
     // A dimension of at most 192 whose last (or only) 128-tile would be at most half full takes tiles of
     // 64: the 2 x 2 wave arrangement would leave half of the waves of such a tile without work (one
     // dimension only, j first).
@@ -2492,12 +2531,23 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
     if (fused || !view)
         hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
                            g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
+    // Where the first product takes the eight-wave kernel in every round, its epilogue reads the upstream
+    // gradient as it is (items of whole 32-position blocks, 16-byte aligned): no transposed copy.
+    bool g_planes = !fused && view && (g.wo * g.ho) % 32 == 0 && ((uintptr_t)gy & 15) == 0;
+    if (g_planes) {
+        GemmParams t = {};
+        t.I = M; t.J = J; t.K = K; t.splits = 1; t.k_per_split = K;
+        for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
+            const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
+            if (!big_tile_nx(t, nv, false)) g_planes = false;
+        }
+    }
     {
         const int npos = g.wo * g.ho;
         if (fused) {
             hipLaunchKernelGGL(k_tile_grad, dim3((M + kFusedTile - 1) / kFusedTile, L.gt_blocks), dim3(256), 0, s, gy, gt, M,
                                g.c_out, npos, L.gt_blocks, L.gt_dedupe);
-        } else {
+        } else if (!g_planes) {
             if (g.n > 65535) return GEO_SC_ERR_UNSUPPORTED;  // grid.z of the transpose
             hipLaunchKernelGGL(k_transpose_grad, dim3((npos + 31) / 32, (g.c_out + 31) / 32, g.n), dim3(256), 0, s, gy, gt,
                                g.c_out, npos);
@@ -2616,7 +2666,7 @@ int launch_conv_backward(const Geometry& g, const float* x, const float* w, cons
         q1.splits = 1; q1.k_per_split = K; q1.c_split_stride = 0;
         q1.a_batch_stride = (long long)L.col_v; q1.b_batch_stride = (long long)L.w_v;
         q1.c_batch_stride = (long long)L.e_v;
-        q1.g = gt; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
+        q1.g = g_planes ? gy : gt; q1.g_planes = g_planes; q1.c_out = g.c_out; q1.npos = g.wo * g.ho;
         q1.a_rows = view_rows; q1.a_rows_batch = L.view_k_pad; q1.a_item = g.wo * g.ho; q1.a_skip = (g.w_k - 1) * g.ho;
         rc = view ? launch_gemm<true, true, EPI_EXP_TIMES_G, true>(q1, nv, s)
                   : launch_gemm<true, true, EPI_EXP_TIMES_G>(q1, nv, s);
