@@ -25,11 +25,26 @@ class ConvDesc(ctypes.Structure):
         "total_width", "load_width", "load_wait_w", "load_wait_a", "accumulate", "z_unit", "generator", "seed")]
 
 
+class Options(ctypes.Structure):
+    """geo_sc_options of include/geo_sc.h"""
+    _fields_ = [("struct_bytes", ctypes.c_size_t), ("forward_stream_bytes", ctypes.c_size_t),
+                ("backward_groups_per_round", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
 # every symbol include/geo_sc.h declares: name -> (restype, argtypes)
 _P = ctypes.c_void_p
 _SZ = ctypes.POINTER(ctypes.c_size_t)
 _D = ctypes.POINTER(ConvDesc)
+_O = ctypes.POINTER(Options)
 C_API = {
+    "geo_sc_init": (ctypes.c_int, []),
+    "geo_sc_stream_table_copy": (ctypes.c_int, [ctypes.c_int, _P, ctypes.c_size_t, _SZ]),
+    "geo_sc_static_workspace_bytes": (ctypes.c_size_t, []),
+    "geo_sc_conv2d_add_partial_workspace_size_ex": (ctypes.c_int, [_D, _O, _SZ]),
+    "geo_sc_conv2d_add_partial_forward_chunk": (ctypes.c_int, [_D, _O, ctypes.POINTER(ctypes.c_int)]),
+    "geo_sc_conv2d_add_partial_forward_ex": (ctypes.c_int, [_D, _O, _P, _P, _P, _P, ctypes.c_size_t, _P]),
+    "geo_sc_conv2d_add_partial_backward_workspace_size_ex": (ctypes.c_int, [_D, _O, _SZ]),
+    "geo_sc_conv2d_add_partial_backward_ex": (ctypes.c_int, [_D, _O, _P, _P, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_version": (ctypes.c_int, []),
     "geo_sc_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "geo_sc_conv2d_add_partial_workspace_size": (ctypes.c_int, [_D, _SZ]),

@@ -10,7 +10,7 @@ import ctypes
 import torch
 
 from . import _native
-from ._native import ConvDesc
+from ._native import ConvDesc, Options
 
 NEUTRAL_LOADING = dict(total_width=7, load_width=8, load_wait_w=1, load_wait_a=1)
 
@@ -49,6 +49,17 @@ def make_desc(x_shape, w_shape, bit_length, padding=(0, 0), total_width=7, load_
                     ctypes.c_int32(int(seed) & 0xffffffff).value)
 
 
+def make_options(forward_stream_bytes=0, backward_groups_per_round=0) -> Options:
+    """geo_sc_options: the budget (bytes) of the forward's activation stream buffer - a batch whose streams
+    exceed it runs in chunks of items - and the cap on the add groups per round of backward launches;
+    0 leaves a field at the library's default."""
+    return Options(ctypes.sizeof(Options), int(forward_stream_bytes), int(backward_groups_per_round), 0)
+
+
+def _opt_ptr(options):
+    return ctypes.byref(options) if options is not None else None
+
+
 def _stream_ptr(stream=None):
     s = stream if stream is not None else torch.cuda.current_stream()
     return ctypes.c_void_p(s.cuda_stream)
@@ -62,10 +73,18 @@ def version() -> int:
     return _native.lib().geo_sc_version()
 
 
-def workspace_size(desc: ConvDesc) -> int:
+def workspace_size(desc: ConvDesc, options: Options = None) -> int:
     out = ctypes.c_size_t(0)
-    _check(_native.lib().geo_sc_conv2d_add_partial_workspace_size(ctypes.byref(desc), ctypes.byref(out)),
-           "workspace query")
+    _check(_native.lib().geo_sc_conv2d_add_partial_workspace_size_ex(ctypes.byref(desc), _opt_ptr(options),
+                                                                     ctypes.byref(out)), "workspace query")
+    return out.value
+
+
+def forward_chunk(desc: ConvDesc, options: Options = None) -> int:
+    """Batch items per chunk of the forward (geo_sc_conv2d_add_partial_forward_chunk)."""
+    out = ctypes.c_int(0)
+    _check(_native.lib().geo_sc_conv2d_add_partial_forward_chunk(ctypes.byref(desc), _opt_ptr(options),
+                                                                 ctypes.byref(out)), "chunk query")
     return out.value
 
 
@@ -80,32 +99,43 @@ def _require_gpu_f32(t, name):
 
 def conv2d_add_partial_forward(x, w, bit_length, padding=(0, 0), total_width=7, load_width=8, load_wait_w=1,
                                load_wait_a=1, out=None, workspace=None, stream=None, desc=None, accumulate="y",
-                               z_unit=1, generator="lfsr", seed=0):
-    """int32 (N, Cout, Wo, Ho) GPU tensor via geo_sc_conv2d_add_partial_forward."""
+                               z_unit=1, generator="lfsr", seed=0, options=None):
+    """int32 (N, Cout, Wo, Ho) GPU tensor via geo_sc_conv2d_add_partial_forward_ex."""
     _require_gpu_f32(x, "x")
     _require_gpu_f32(w, "w")
     if desc is None:
         desc = make_desc(x.shape, w.shape, bit_length, padding, total_width, load_width, load_wait_w, load_wait_a,
                          accumulate, z_unit, generator, seed)
-    ws_bytes = workspace_size(desc)
     if workspace is None:
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+        workspace = torch.empty(workspace_size(desc, options), dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty(output_shape(desc), dtype=torch.int32, device=x.device)
-    _check(_native.lib().geo_sc_conv2d_add_partial_forward(ctypes.byref(desc), _ptr(x), _ptr(w), _ptr(out),
-                                                           _ptr(workspace), workspace.numel(), _stream_ptr(stream)),
+    _check(_native.lib().geo_sc_conv2d_add_partial_forward_ex(ctypes.byref(desc), _opt_ptr(options), _ptr(x), _ptr(w),
+                                                              _ptr(out), _ptr(workspace), workspace.numel(),
+                                                              _stream_ptr(stream)),
            "geo_sc_conv2d_add_partial_forward")
     return out
 
 
-STATIC_WORKSPACE_BYTES = 32 << 20   # GEO_SC_STATIC_WORKSPACE_BYTES of include/geo_sc.h
+def static_workspace_bytes() -> int:
+    """Size of the library's static device workspace (geo_sc_static_workspace_bytes)."""
+    return int(_native.lib().geo_sc_static_workspace_bytes())
+
+
+def init():
+    """geo_sc_init: per-device lookups of the library on the current device (call before a stream capture)."""
+    _check(_native.lib().geo_sc_init(), "geo_sc_init")
 
 
 def conv2d_add_partial_forward_static(x, w, out, desc: ConvDesc, stream=None):
     """geo_sc_conv2d_add_partial_forward_static: the forward on the library's static device workspace;
-    allocates nothing (``out`` is the caller's int32 tensor of output_shape(desc))."""
+    allocates nothing (``out`` is the caller's int32 tensor of output_shape(desc)).  The workspace is the
+    current device's: all three tensors must live there."""
     _require_gpu_f32(x, "x")
     _require_gpu_f32(w, "w")
+    cur = torch.cuda.current_device()
+    if not (x.device.index == cur and w.device.index == cur and out.device.index == cur):
+        raise ValueError("x, w and out must be on the current device (the static workspace is per device)")
     if not (out.is_cuda and out.dtype == torch.int32 and out.is_contiguous()
             and tuple(out.shape) == output_shape(desc)):
         raise ValueError("out must be a contiguous int32 GPU tensor of the output's shape")
@@ -238,12 +268,6 @@ def quantize(x, prec, out=None, stream=None):
     return out
 
 
-def _tables(bit_length, device):
-    n = ctypes.c_size_t(0)
-    _check(_native.lib().geo_sc_stream_tables_size(int(bit_length), ctypes.byref(n)), "tables size")
-    return torch.empty(n.value, dtype=torch.uint8, device=device)
-
-
 def act_streams(x, desc: ConvDesc, stream=None):
     """int32-typed tensor of stream words (reinterpret as uint32), shaped as the library stores them:
     (N, P, Cin, Wi, Hi), or (P, Cin, Wi, Hi, N) for the geometries whose streams are batch-item-innermost
@@ -264,9 +288,8 @@ def act_streams(x, desc: ConvDesc, stream=None):
     shape = (packs, desc.c_in, wi, hi, desc.n) if inner.value else (desc.n, packs, desc.c_in, wi, hi)
     out = torch.empty(shape, dtype=torch.int32, device=x.device)
     assert out.numel() == n.value
-    tables = _tables(desc.bit_length, x.device)
     fn = _native.lib().geo_sc_act_streams_q7 if q7 else _native.lib().geo_sc_act_streams
-    _check(fn(ctypes.byref(desc), _ptr(x), _ptr(out), _ptr(tables), _stream_ptr(stream)), "geo_sc_act_streams")
+    _check(fn(ctypes.byref(desc), _ptr(x), _ptr(out), None, _stream_ptr(stream)), "geo_sc_act_streams")
     return out
 
 
@@ -284,9 +307,8 @@ def weight_streams(w, desc: ConvDesc, stream=None):
     buf = torch.empty(n.value, dtype=torch.int32, device=w.device)
     assert n.value >= classic
     out = buf[:classic].view(shape)
-    tables = _tables(desc.bit_length, w.device)
-    _check(_native.lib().geo_sc_weight_streams(ctypes.byref(desc), _ptr(w), _ptr(out), _ptr(tables),
-                                               _stream_ptr(stream)), "geo_sc_weight_streams")
+    _check(_native.lib().geo_sc_weight_streams(ctypes.byref(desc), _ptr(w), _ptr(out), None, _stream_ptr(stream)),
+           "geo_sc_weight_streams")
     return out
 
 
@@ -310,8 +332,11 @@ def weight_streams_ok(wgt, desc: ConvDesc, stream=None) -> bool:
     """geo_sc_weight_streams_check on a buffer view as weight_streams() / weight_streams_from_lines()
     return it: False when a caller-written line has two non-zero rails for one channel.  Waits for the
     stream."""
+    n = ctypes.c_size_t(0)
+    # the descriptor on its own first: after this, GEO_SC_ERR_INVALID_ARGUMENT can only mean a flagged buffer
+    _check(_native.lib().geo_sc_weight_stream_words(ctypes.byref(desc), ctypes.byref(n)), "weight words")
     rc = _native.lib().geo_sc_weight_streams_check(ctypes.byref(desc), _ptr(wgt), _stream_ptr(stream))
-    if rc == 1:   # GEO_SC_ERR_INVALID_ARGUMENT: the flagged buffer (the descriptor was valid when the buffer was made)
+    if rc == 1:
         return False
     _check(rc, "geo_sc_weight_streams_check")
     return True
@@ -341,16 +366,17 @@ def conv2d_add_partial_from_streams(act, wgt, desc: ConvDesc, out=None, stream=N
     return out
 
 
-def backward_workspace_size(desc: ConvDesc) -> int:
+def backward_workspace_size(desc: ConvDesc, options: Options = None) -> int:
     out = ctypes.c_size_t(0)
-    _check(_native.lib().geo_sc_conv2d_add_partial_backward_workspace_size(ctypes.byref(desc), ctypes.byref(out)),
+    _check(_native.lib().geo_sc_conv2d_add_partial_backward_workspace_size_ex(ctypes.byref(desc), _opt_ptr(options),
+                                                                              ctypes.byref(out)),
            "backward workspace query")
     return out.value
 
 
 def conv2d_add_partial_backward(x, w, grad_y, bit_length=128, padding=(0, 0), need_grad_x=True, need_grad_w=True,
-                                workspace=None, stream=None, desc=None, accumulate="y", z_unit=1):
-    """(grad_x, grad_w) of the surrogate via geo_sc_conv2d_add_partial_backward; an output
+                                workspace=None, stream=None, desc=None, accumulate="y", z_unit=1, options=None):
+    """(grad_x, grad_w) of the surrogate via geo_sc_conv2d_add_partial_backward_ex; an output
     that is not needed is returned as None."""
     _require_gpu_f32(x, "x")
     _require_gpu_f32(w, "w")
@@ -360,12 +386,12 @@ def conv2d_add_partial_backward(x, w, grad_y, bit_length=128, padding=(0, 0), ne
     if tuple(grad_y.shape) != output_shape(desc):
         raise ValueError(f"grad_y has shape {tuple(grad_y.shape)}, expected {output_shape(desc)}")
     if workspace is None:
-        workspace = torch.empty(backward_workspace_size(desc), dtype=torch.uint8, device=x.device)
+        workspace = torch.empty(backward_workspace_size(desc, options), dtype=torch.uint8, device=x.device)
     gx = torch.empty_like(x) if need_grad_x else None
     gw = torch.empty_like(w) if need_grad_w else None
-    _check(_native.lib().geo_sc_conv2d_add_partial_backward(ctypes.byref(desc), _ptr(x), _ptr(w), _ptr(grad_y),
-                                                            _ptr(gx), _ptr(gw), _ptr(workspace), workspace.numel(),
-                                                            _stream_ptr(stream)),
+    _check(_native.lib().geo_sc_conv2d_add_partial_backward_ex(ctypes.byref(desc), _opt_ptr(options), _ptr(x), _ptr(w),
+                                                               _ptr(grad_y), _ptr(gx), _ptr(gw), _ptr(workspace),
+                                                               workspace.numel(), _stream_ptr(stream)),
            "geo_sc_conv2d_add_partial_backward")
     return gx, gw
 

@@ -119,10 +119,77 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g)
         g->wgt_flag_off = g->wgt_rail_idx_off + lines * g->n_cotile * (kCoTile / 2);
         g->wgt_words = g->wgt_flag_off + 64;
     }
-    g->off_tables = 0;
-    g->off_wgt = align256(table_bytes(g->L));
-    g->off_act = g->off_wgt + align256(g->wgt_words * sizeof(uint32_t));
-    g->ws_bytes = g->off_act + align256(g->act_words * sizeof(uint32_t));
+    return GEO_SC_OK;
+}
+
+Options make_options(const geo_sc_options* o)
+{
+    Options r;
+    r.forward_stream_bytes = kDefaultForwardStreamBytes;
+    r.backward_groups_per_round = 0;
+    if (o && o->struct_bytes >= sizeof(geo_sc_options)) {
+        if (o->forward_stream_bytes) r.forward_stream_bytes = o->forward_stream_bytes;
+        if (o->backward_groups_per_round > 0) r.backward_groups_per_round = o->backward_groups_per_round;
+    }
+    return r;
+}
+
+// The forward walks the batch in chunks of `nc` items (the last one may be shorter): activation streams
+// are generated for one chunk, consumed by its convolution launch, and the buffer is reused, so the
+// scratch does not grow with the batch (the reference keeps streams for 128 blocks whatever the batch,
+// sc_cuda_kernel.cu:658-662, :1787-1789).  Every item is independent (same seeds for every item,
+// sc.cpp:409-413), so the counts do not depend on the cut.
+struct ForwardPlan {
+    Geometry chunk, last;  // geometry of a full chunk and of the shorter last one (n_last == 0: none)
+    int nc, n_full, n_last;
+    bool rail_only;        // every launch reads the rail-packed weight lines only
+    size_t off_wgt, off_act, ws_bytes;
+};
+
+int plan_forward(const geo_sc_conv_desc* d, const Options& opt, ForwardPlan* p)
+{
+    Geometry g;
+    int rc = make_geometry(d, &g);
+    if (rc != GEO_SC_OK) return rc;
+    const size_t item_bytes = sizeof(uint32_t) * (size_t)g.packs * g.act_plane;
+    geo_sc_conv_desc dc = *d;
+    auto geometry_of = [&](int n, Geometry* out) {
+        dc.n = n;
+        return make_geometry(&dc, out);
+    };
+    int nc = g.n;
+    if ((size_t)g.n * item_bytes > opt.forward_stream_bytes) {
+        // largest chunk inside the budget (at least one item), then the size between that and half of it whose
+        // launches fill the GPU's rounds of waves best
+        long long nc_max = (long long)(opt.forward_stream_bytes / item_bytes);
+        if (nc_max < 1) nc_max = 1;
+        if (nc_max > g.n) nc_max = g.n;
+        double best = 0;
+        for (long long c = nc_max; c >= (nc_max + 1) / 2; c--) {
+            Geometry gc, gl;
+            if ((rc = geometry_of((int)c, &gc)) != GEO_SC_OK) return rc;
+            const int full = g.n / (int)c, rem = g.n - full * (int)c;
+            double cost = full * (conv_forward_cost(gc) + 0.25);
+            if (rem) {
+                if ((rc = geometry_of(rem, &gl)) != GEO_SC_OK) return rc;
+                cost += conv_forward_cost(gl) + 0.25;
+            }
+            if (c == nc_max || cost < best * 0.995) {
+                best = cost;
+                nc = (int)c;
+            }
+        }
+    }
+    p->nc = nc;
+    p->n_full = g.n / nc;
+    p->n_last = g.n - p->n_full * nc;
+    if ((rc = geometry_of(nc, &p->chunk)) != GEO_SC_OK) return rc;
+    p->last = p->chunk;
+    if (p->n_last && (rc = geometry_of(p->n_last, &p->last)) != GEO_SC_OK) return rc;
+    p->rail_only = p->chunk.rail && p->last.rail;
+    p->off_wgt = 0;
+    p->off_act = align256(g.wgt_words * sizeof(uint32_t));
+    p->ws_bytes = p->off_act + align256((size_t)nc * item_bytes);
     return GEO_SC_OK;
 }
 
@@ -136,7 +203,9 @@ static __device__ __align__(256) unsigned char scratch[GEO_SC_STATIC_WORKSPACE_B
 
 namespace {
 // Device address of `scratch` on the current device (every GPU holds its own copy of the array at an
-// address of its own), looked up once per device; nullptr if the runtime refuses.
+// address of its own), looked up once per device - by geo_sc_init, or by the first call that needs it;
+// nullptr if the runtime refuses.  The lookup is not stream-ordered work: it must not happen first
+// inside a stream capture.
 void* static_workspace()
 {
     constexpr int kMaxDevices = 64;
@@ -152,31 +221,37 @@ void* static_workspace()
     }
     return addr[dev];
 }
-}  // namespace
 
-namespace {
 // x is fp32, or with Q7 the uint8 integers k of activations k / 128
 template <bool Q7>
-int forward_impl(const geo_sc_conv_desc* desc, const void* x, const float* w, int32_t* y, void* workspace,
-                 size_t workspace_bytes, geo_sc_stream_t stream)
+int forward_impl(const geo_sc_conv_desc* desc, const Options& opt, const void* x, const float* w, int32_t* y,
+                 void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
 {
-    Geometry g;
-    int rc = make_geometry(desc, &g);
+    ForwardPlan p;
+    int rc = plan_forward(desc, opt, &p);
     if (rc != GEO_SC_OK) return rc;
     if (!x || !w || !y) return GEO_SC_ERR_INVALID_ARGUMENT;
-    if (!workspace || workspace_bytes < g.ws_bytes || ((uintptr_t)workspace & 255u)) return GEO_SC_ERR_WORKSPACE;
+    if (!workspace || workspace_bytes < p.ws_bytes || ((uintptr_t)workspace & 255u)) return GEO_SC_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
-    uint32_t* tables = (uint32_t*)(ws + g.off_tables);
-    uint32_t* wgt = (uint32_t*)(ws + g.off_wgt);
-    uint32_t* act = (uint32_t*)(ws + g.off_act);
-    if ((rc = launch_build_tables(g, tables, s)) != GEO_SC_OK) return rc;
-    if ((rc = launch_weight_streams(g, w, wgt, tables, s, g.rail)) != GEO_SC_OK) return rc;
-    if ((rc = launch_rail_pack(g, wgt, s, true)) != GEO_SC_OK) return rc;
-    rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)x, act, tables, s)
-            : launch_act_streams(g, (const float*)x, act, tables, s);
-    if (rc != GEO_SC_OK) return rc;
-    return launch_conv_forward(g, act, wgt, y, s);
+    uint32_t* wgt = (uint32_t*)(ws + p.off_wgt);
+    uint32_t* act = (uint32_t*)(ws + p.off_act);
+    // the weight stream buffer is the same for every batch size: generated once, read by every chunk
+    if ((rc = launch_weight_streams(p.chunk, w, wgt, s, p.rail_only)) != GEO_SC_OK) return rc;
+    if ((rc = launch_rail_pack(p.chunk, wgt, s, true)) != GEO_SC_OK) return rc;
+    const size_t x_item = (size_t)desc->c_in * desc->w_in * desc->h_in * (Q7 ? 1 : sizeof(float));
+    const size_t y_item = (size_t)desc->c_out * p.chunk.wo * p.chunk.ho;
+    const int chunks = p.n_full + (p.n_last ? 1 : 0);
+    for (int c = 0; c < chunks; c++) {
+        const Geometry& g = c < p.n_full ? p.chunk : p.last;
+        const size_t n0 = (size_t)c * p.nc;
+        const char* xc = (const char*)x + n0 * x_item;
+        rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)xc, act, s)
+                : launch_act_streams(g, (const float*)xc, act, s, n0);
+        if (rc != GEO_SC_OK) return rc;
+        if ((rc = launch_conv_forward(g, act, wgt, y + n0 * y_item, s)) != GEO_SC_OK) return rc;
+    }
+    return GEO_SC_OK;
 }
 }  // namespace
 
@@ -197,13 +272,37 @@ const char* geo_sc_status_string(int status)
     }
 }
 
+int geo_sc_init(void)
+{
+    return static_workspace() ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+size_t geo_sc_static_workspace_bytes(void) { return GEO_SC_STATIC_WORKSPACE_BYTES; }
+
+int geo_sc_conv2d_add_partial_workspace_size_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                                size_t* bytes)
+{
+    ForwardPlan p;
+    if (!bytes) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = plan_forward(desc, make_options(options), &p);
+    if (rc != GEO_SC_OK) return rc;
+    *bytes = p.ws_bytes;
+    return GEO_SC_OK;
+}
+
 int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes)
 {
-    Geometry g;
-    if (!bytes) return GEO_SC_ERR_INVALID_ARGUMENT;
-    const int rc = make_geometry(desc, &g);
+    return geo_sc_conv2d_add_partial_workspace_size_ex(desc, nullptr, bytes);
+}
+
+int geo_sc_conv2d_add_partial_forward_chunk(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                            int* items_per_chunk)
+{
+    ForwardPlan p;
+    if (!items_per_chunk) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int rc = plan_forward(desc, make_options(options), &p);
     if (rc != GEO_SC_OK) return rc;
-    *bytes = g.ws_bytes;
+    *items_per_chunk = p.nc;
     return GEO_SC_OK;
 }
 
@@ -214,7 +313,20 @@ int geo_sc_stream_tables_size(int bit_length, size_t* bytes)
     case 8: case 16: case 32: case 64: case 128: case 256: break;
     default: return GEO_SC_ERR_BIT_LENGTH;
     }
-    *bytes = table_bytes(bit_length);
+    *bytes = 0;  // the tables are constant data of the library
+    return GEO_SC_OK;
+}
+
+int geo_sc_stream_table_copy(int bit_length, uint32_t* host_words, size_t capacity_words, size_t* words)
+{
+    size_t n = 0;
+    const uint32_t* t = stream_tables_host(bit_length, &n);
+    if (!t) return GEO_SC_ERR_BIT_LENGTH;
+    if (words) *words = n;
+    if (host_words) {
+        if (capacity_words < n) return GEO_SC_ERR_INVALID_ARGUMENT;
+        for (size_t i = 0; i < n; i++) host_words[i] = t[i];
+    }
     return GEO_SC_OK;
 }
 
@@ -254,11 +366,9 @@ int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* s
     Geometry g;
     int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
-    if (!x || !streams || !tables) return GEO_SC_ERR_INVALID_ARGUMENT;
-    hipStream_t s = (hipStream_t)stream;
-    rc = launch_build_tables(g, (uint32_t*)tables, s);
-    if (rc != GEO_SC_OK) return rc;
-    return launch_act_streams(g, x, streams, (const uint32_t*)tables, s);
+    (void)tables;
+    if (!x || !streams) return GEO_SC_ERR_INVALID_ARGUMENT;
+    return launch_act_streams(g, x, streams, (hipStream_t)stream);
 }
 
 int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, uint32_t* streams, void* tables,
@@ -267,11 +377,9 @@ int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, uin
     Geometry g;
     int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
-    if (!x_q7 || !streams || !tables) return GEO_SC_ERR_INVALID_ARGUMENT;
-    hipStream_t s = (hipStream_t)stream;
-    rc = launch_build_tables(g, (uint32_t*)tables, s);
-    if (rc != GEO_SC_OK) return rc;
-    return launch_act_streams_q7(g, x_q7, streams, (const uint32_t*)tables, s);
+    (void)tables;
+    if (!x_q7 || !streams) return GEO_SC_ERR_INVALID_ARGUMENT;
+    return launch_act_streams_q7(g, x_q7, streams, (hipStream_t)stream);
 }
 
 int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
@@ -280,11 +388,10 @@ int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t
     Geometry g;
     int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
-    if (!w || !streams || !tables) return GEO_SC_ERR_INVALID_ARGUMENT;
+    (void)tables;
+    if (!w || !streams) return GEO_SC_ERR_INVALID_ARGUMENT;
     hipStream_t s = (hipStream_t)stream;
-    rc = launch_build_tables(g, (uint32_t*)tables, s);
-    if (rc != GEO_SC_OK) return rc;
-    rc = launch_weight_streams(g, w, streams, (const uint32_t*)tables, s);
+    rc = launch_weight_streams(g, w, streams, s);
     if (rc != GEO_SC_OK) return rc;
     return launch_rail_pack(g, streams, s, true);
 }
@@ -326,52 +433,81 @@ int geo_sc_conv2d_add_partial_from_streams(const geo_sc_conv_desc* desc, const u
 int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
                                       void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
 {
-    return forward_impl<false>(desc, x, w, y, workspace, workspace_bytes, stream);
+    return forward_impl<false>(desc, make_options(nullptr), x, w, y, workspace, workspace_bytes, stream);
+}
+
+int geo_sc_conv2d_add_partial_forward_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options, const float* x,
+                                         const float* w, int32_t* y, void* workspace, size_t workspace_bytes,
+                                         geo_sc_stream_t stream)
+{
+    return forward_impl<false>(desc, make_options(options), x, w, y, workspace, workspace_bytes, stream);
 }
 
 int geo_sc_conv2d_add_partial_forward_static(const geo_sc_conv_desc* desc, const float* x, const float* w,
                                              int32_t* y, geo_sc_stream_t stream)
 {
+    // the whole array is the budget: weight streams first, the rest holds the activation streams of as many
+    // items at a time as fit (at least one, or the problem is too large for this entry point)
     Geometry g;
-    const int rc = make_geometry(desc, &g);
+    int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
-    if (g.ws_bytes > GEO_SC_STATIC_WORKSPACE_BYTES) return GEO_SC_ERR_WORKSPACE;
+    const size_t wgt_bytes = align256(g.wgt_words * sizeof(uint32_t));
+    if (wgt_bytes >= GEO_SC_STATIC_WORKSPACE_BYTES) return GEO_SC_ERR_WORKSPACE;
+    Options opt = make_options(nullptr);
+    opt.forward_stream_bytes = GEO_SC_STATIC_WORKSPACE_BYTES - wgt_bytes - 256;
+    ForwardPlan p;
+    if ((rc = plan_forward(desc, opt, &p)) != GEO_SC_OK) return rc;
+    if (p.ws_bytes > GEO_SC_STATIC_WORKSPACE_BYTES) return GEO_SC_ERR_WORKSPACE;
     void* ws = static_workspace();
     if (!ws) return GEO_SC_ERR_LAUNCH;
     // Every word the kernels read from the workspace is written by this call's own kernels first
-    // (tables, all weight lines including the channel padding, the flag area, every activation word),
-    // so nothing left by an earlier call needs clearing.
-    return forward_impl<false>(desc, x, w, y, ws, GEO_SC_STATIC_WORKSPACE_BYTES, stream);
+    // (all weight lines including the channel padding, the flag area, every activation word of a chunk
+    // before its convolution launch), so nothing left by an earlier call needs clearing.
+    return forward_impl<false>(desc, opt, x, w, y, ws, GEO_SC_STATIC_WORKSPACE_BYTES, stream);
 }
 
 int geo_sc_conv2d_add_partial_forward_q7(const geo_sc_conv_desc* desc, const uint8_t* x_q7, const float* w,
                                          int32_t* y, void* workspace, size_t workspace_bytes,
                                          geo_sc_stream_t stream)
 {
-    return forward_impl<true>(desc, x_q7, w, y, workspace, workspace_bytes, stream);
+    return forward_impl<true>(desc, make_options(nullptr), x_q7, w, y, workspace, workspace_bytes, stream);
 }
 
-int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes)
+int geo_sc_conv2d_add_partial_backward_workspace_size_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                                         size_t* bytes)
 {
     Geometry g;
     if (!bytes) return GEO_SC_ERR_INVALID_ARGUMENT;
     const int rc = make_geometry(desc, &g);
     if (rc != GEO_SC_OK) return rc;
-    *bytes = backward_workspace_bytes(g);
+    *bytes = backward_workspace_bytes(g, make_options(options).backward_groups_per_round);
     return GEO_SC_OK;
+}
+
+int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes)
+{
+    return geo_sc_conv2d_add_partial_backward_workspace_size_ex(desc, nullptr, bytes);
+}
+
+int geo_sc_conv2d_add_partial_backward_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options, const float* x,
+                                          const float* w, const float* grad_y, float* grad_x, float* grad_w,
+                                          void* workspace, size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    Geometry g;
+    const int rc = make_geometry(desc, &g);
+    if (rc != GEO_SC_OK) return rc;
+    if (!x || !w || !grad_y || (!grad_x && !grad_w)) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (!workspace || ((uintptr_t)workspace & 255u)) return GEO_SC_ERR_WORKSPACE;
+    return launch_conv_backward(g, make_options(options).backward_groups_per_round, x, w, grad_y, grad_x, grad_w,
+                                workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float* x, const float* w,
                                        const float* grad_y, float* grad_x, float* grad_w, void* workspace,
                                        size_t workspace_bytes, geo_sc_stream_t stream)
 {
-    Geometry g;
-    const int rc = make_geometry(desc, &g);
-    if (rc != GEO_SC_OK) return rc;
-    if (!x || !w || !grad_y || (!grad_x && !grad_w)) return GEO_SC_ERR_INVALID_ARGUMENT;
-    if (!workspace || workspace_bytes < backward_workspace_bytes(g) || ((uintptr_t)workspace & 255u))
-        return GEO_SC_ERR_WORKSPACE;
-    return launch_conv_backward(g, x, w, grad_y, grad_x, grad_w, workspace, (hipStream_t)stream);
+    return geo_sc_conv2d_add_partial_backward_ex(desc, nullptr, x, w, grad_y, grad_x, grad_w, workspace, workspace_bytes,
+                                                 stream);
 }
 
 }  // extern "C"

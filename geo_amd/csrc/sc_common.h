@@ -58,33 +58,43 @@ struct Geometry {
     // that rail is processed.  wgt_rail: the weight stream buffer carries the rail-packed copy (a
     // property of the weights' shape alone); rail: this geometry's launch reads it.
     bool wgt_rail, rail;
-    // workspace carve-up (byte offsets, 256-aligned)
-    size_t off_tables, off_wgt, off_act, ws_bytes;
 };
 
-// Stream tables (device memory, built per call):
+// Stream tables (one per stream length, constant data of the code object):
 //   posp1[r], r < L-1 : 1 + index in the LFSR cycle of state r+1  (cycle[0] = 1)
 //   thr[code][j]      : bit string, MSB-first, of [code > cycle[j mod (L-1)]] for
 //                       j < 32 * words_per_code, long enough to read L bits from any
 //                       offset <= L-1 plus one spare word for the funnel shift.
-inline __host__ __device__ int table_words_per_code(int L) { return (2 * L + 31) / 32 + 2; }
+constexpr __host__ __device__ int table_words_per_code(int L) { return (2 * L + 31) / 32 + 2; }
 inline __host__ __device__ size_t table_bytes(int L)
 {
     return sizeof(uint32_t) * ((size_t)L + (size_t)L * table_words_per_code(L));
 }
 
+const uint32_t* stream_tables_host(int L, size_t* words);
+
 int make_geometry(const geo_sc_conv_desc* d, Geometry* g);
 
+// Caller's choices that are not part of the problem (geo_sc_options with its defaults filled in).
+struct Options {
+    size_t forward_stream_bytes;    // budget of the forward's activation stream buffer
+    int backward_groups_per_round;  // cap on the add groups per round of backward launches; 0: none
+};
+constexpr size_t kDefaultForwardStreamBytes = (size_t)256 << 20;
+
 // launchers (each returns a geo_sc_status)
-int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s);
-int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s);
-int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* streams, const uint32_t* tables,
-                          hipStream_t s);
+// item0: index of x's first item in the whole batch (the random generators number their sequences by it)
+int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, hipStream_t s, size_t item0 = 0);
+int launch_act_streams_q7(const Geometry& g, const uint8_t* x_q7, uint32_t* streams, hipStream_t s);
 // rail_only: the caller's convolution kernel reads the rail-packed copy only; a generator that writes that
 // copy itself may then leave the two-rail lines unwritten
-int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
-                          hipStream_t s, bool rail_only = false);
+int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, hipStream_t s,
+                          bool rail_only = false);
 int launch_conv_forward(const Geometry& g, const uint32_t* act, const uint32_t* wgt, int32_t* y, hipStream_t s);
+// Predicted duration of that launch in units of one wave walking one (pack, add group) pair on a full GPU:
+// what the forward compares when it cuts a batch into chunks (waves run in rounds of four per SIMD, so a
+// chunk whose waves fill whole rounds costs less per item).
+double conv_forward_cost(const Geometry& g);
 // fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.wgt_rail;
 // with from_generator also where launch_weight_streams has written that part itself)
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator);
@@ -93,8 +103,9 @@ inline bool weight_rows_generator(const Geometry& g)
 {
     return g.generator == GEO_SC_GEN_LFSR && (g.mode == GEO_SC_ACC_Y || g.mode == GEO_SC_ACC_FULL) && g.h_k >= 16;
 }
-size_t backward_workspace_bytes(const Geometry& g);
-int launch_conv_backward(const Geometry& g, const float* x, const float* w, const float* gy, float* gx, float* gw,
-                         void* workspace, hipStream_t s);
+size_t backward_workspace_bytes(const Geometry& g, int groups_per_round);
+// GEO_SC_ERR_WORKSPACE when workspace_bytes is below backward_workspace_bytes(g, groups_per_round)
+int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x, const float* w, const float* gy,
+                         float* gx, float* gw, void* workspace, size_t workspace_bytes, hipStream_t s);
 
 }  // namespace geo_sc

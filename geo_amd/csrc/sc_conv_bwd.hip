@@ -2381,7 +2381,7 @@ size_t view_floats(const Geometry& g)
     return (size_t)g.h_k * g.c_in * g.n * (g.w_in + 2 * g.pad_w) * g.ho + (size_t)g.w_k * g.ho;
 }
 
-BwdLayout bwd_layout(const Geometry& g)
+BwdLayout bwd_layout(const Geometry& g, int groups_per_round)
 {
     BwdLayout b;
     b.m_total = (long long)g.n * g.wo * g.ho;
@@ -2447,11 +2447,8 @@ BwdLayout bwd_layout(const Geometry& g)
     size_t rows = ((size_t)3 << 30) / per_row;
     if (rows < 1) rows = 1;
     if (rows > (size_t)b.G.n_groups) rows = b.G.n_groups;
-    // GEO_SC_BACKWARD_GROUPS_PER_ROUND caps the add groups per round further (less scratch, more launches)
-    if (const char* cap = getenv("GEO_SC_BACKWARD_GROUPS_PER_ROUND")) {
-        const long v = atol(cap);
-        if (v >= 1 && (size_t)v < rows) rows = (size_t)v;
-    }
+    // the caller's cap on the add groups per round (less scratch, more launches)
+    if (groups_per_round >= 1 && (size_t)groups_per_round < rows) rows = (size_t)groups_per_round;
     if (rows * b.splits > 65535) rows = 65535 / b.splits;  // grid.z = rows * splits
     if (rows < 1) rows = 1;
     b.rows_per_chunk = (int)rows;
@@ -2495,12 +2492,13 @@ BwdLayout bwd_layout(const Geometry& g)
 
 }  // namespace
 
-size_t backward_workspace_bytes(const Geometry& g) { return bwd_layout(g).bytes; }
+size_t backward_workspace_bytes(const Geometry& g, int groups_per_round) { return bwd_layout(g, groups_per_round).bytes; }
 
-int launch_conv_backward(const Geometry& g, const float* x, const float* w, const float* gy, float* gx, float* gw,
-                         void* workspace, hipStream_t s)
+int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x, const float* w, const float* gy,
+                         float* gx, float* gw, void* workspace, size_t workspace_bytes, hipStream_t s)
 {
-    const BwdLayout L = bwd_layout(g);
+    const BwdLayout L = bwd_layout(g, groups_per_round);  // once per call: sizes the check and the launches alike
+    if (workspace_bytes < L.bytes) return GEO_SC_ERR_WORKSPACE;
     if (L.m_total > 0x7fffffffLL) return GEO_SC_ERR_INVALID_ARGUMENT;
     char* ws = (char*)workspace;
     float* col = (float*)(ws + L.off_col);

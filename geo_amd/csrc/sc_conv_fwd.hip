@@ -1246,44 +1246,65 @@ __global__ __launch_bounds__(256) void k_zero_i32(int32_t* __restrict__ p, size_
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0;
 }
 
-template <int R, int WK, int CU, bool ROWS_IN_N>
-int launch(const Geometry& g, FwdParams q, hipStream_t s)
+// How a position-parallel launch (R accumulator rows per lane, kernel extent WK in dim 2, 0: run-time) is cut:
+// waves of 64 lane slots per c_out tile, and the (pack, add group) pairs shared out over blockIdx.y.
+struct SplitPlan {
+    int row_groups;
+    long long slots, tiles, waves;
+    int pv, splits, pv_per_block;
+    bool lds;  // the kernel that shares activation words through LDS
+};
+SplitPlan plan_splits(const Geometry& g, int R, int WK, bool rows_in_n)
 {
-    q.row_groups = ROWS_IN_N ? (g.n + R - 1) / R : (g.wo + R - 1) / R;
-    q.slots = ROWS_IN_N ? (long long)q.row_groups * g.ho : (long long)g.n * q.row_groups * g.ho;
-    const long long tiles = (q.slots + 63) / 64;
-    const long long blocks = tiles * g.n_cotile;
-    const long long waves = blocks;
-    if (blocks <= 0 || blocks > 0x7fffffffLL) return GEO_SC_ERR_INVALID_ARGUMENT;
-    // per-lane word offsets are 32-bit
-    if ((unsigned long long)R * g.packs * g.act_plane >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
-    if (ROWS_IN_N != g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
+    SplitPlan sp;
+    sp.row_groups = rows_in_n ? (g.n + R - 1) / R : (g.wo + R - 1) / R;
+    sp.slots = rows_in_n ? (long long)sp.row_groups * g.ho : (long long)g.n * sp.row_groups * g.ho;
+    sp.tiles = (sp.slots + 63) / 64;
+    sp.waves = sp.tiles * g.n_cotile;
     // Fewer than four waves per SIMD (small layers, the SC-linear mapping): split the (pack, add
     // group) sum over blockIdx.y until about twelve waves per SIMD exist, so that three resident
     // waves per SIMD stay available through the tail; the partial sums meet in y through integer
     // atomics.  Measured on MI355X: 4096x4096 linear at batch 1024 7.05 -> 6.24 ms.
-    const int pv = g.packs * g.add_outer * g.add_inner;
+    sp.pv = g.packs * g.add_outer * g.add_inner;
     int splits = 1;
     // the LDS-staged kernel: y mode, 3-wide kernels, whole chunks of 8 channels, 4 or 8 c_out tiles
-    const bool lds = R == 2 && WK == 3 && !ROWS_IN_N && g.rail && g.mode == GEO_SC_ACC_Y &&
-                     g.c_in % kStageChannels == 0 && g.n_cotile % 4 == 0;
-    if (waves < 4096) {
-        splits = (int)((12288 + waves - 1) / waves);
-        if (splits > pv) splits = pv;
-    } else if (g.rail && !ROWS_IN_N) {
+    sp.lds = R == 2 && WK == 3 && !rows_in_n && g.rail && g.mode == GEO_SC_ACC_Y &&
+             g.c_in % kStageChannels == 0 && g.n_cotile % 4 == 0;
+    if (sp.waves < 4096) {
+        splits = (int)((12288 + sp.waves - 1) / sp.waves);
+        if (splits > sp.pv) splits = sp.pv;
+    } else if (g.rail && !rows_in_n) {
         // Equal waves run in rounds of 4096 (four per SIMD): 3.06 rounds take the time of 4.  Splitting the
         // passes 2-, 3- or 4-fold makes the rounds shorter and the last one fuller (C5: 12544 waves, 0.77 ->
         // 0.94 of the rounded-up time); taken when it gains more than the atomics cost.
-        auto fill = [&](int sp) { const double r = (double)waves * sp / 4096.0; return r / (double)(long long)(r + 0.999999); };
+        auto fill = [&](int k) { const double r = (double)sp.waves * k / 4096.0; return r / (double)(long long)(r + 0.999999); };
         double best = fill(1) * 1.08;
-        for (int sp = 2; sp <= 4; sp++)
-            if (pv % sp == 0 && fill(sp) > best) {
-                best = fill(sp);
-                splits = sp;
+        for (int k = 2; k <= 4; k++)
+            if (sp.pv % k == 0 && fill(k) > best) {
+                best = fill(k);
+                splits = k;
             }
     }
-    q.pv_per_block = (pv + splits - 1) / splits;
-    splits = (pv + q.pv_per_block - 1) / q.pv_per_block;
+    sp.pv_per_block = (sp.pv + splits - 1) / splits;
+    sp.splits = (sp.pv + sp.pv_per_block - 1) / sp.pv_per_block;
+    return sp;
+}
+
+template <int R, int WK, int CU, bool ROWS_IN_N>
+int launch(const Geometry& g, FwdParams q, hipStream_t s)
+{
+    const SplitPlan sp = plan_splits(g, R, WK, ROWS_IN_N);
+    q.row_groups = sp.row_groups;
+    q.slots = sp.slots;
+    const long long tiles = sp.tiles, blocks = sp.waves, waves = sp.waves;
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return GEO_SC_ERR_INVALID_ARGUMENT;
+    // per-lane word offsets are 32-bit
+    if ((unsigned long long)R * g.packs * g.act_plane >= 0xffffffffull) return GEO_SC_ERR_UNSUPPORTED;
+    if (ROWS_IN_N != g.act_item_inner) return GEO_SC_ERR_INVALID_ARGUMENT;
+    const int pv = sp.pv;
+    int splits = sp.splits;
+    const bool lds = sp.lds;
+    q.pv_per_block = sp.pv_per_block;
     const bool plain = splits == 1 && g.mode == GEO_SC_ACC_Y && !ROWS_IN_N;
     if constexpr (ROWS_IN_N) {
         static_assert(R == 2 && WK > 0, "item-innermost launches take two items per lane");
@@ -1346,6 +1367,20 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
 }
 
 }  // namespace
+
+double conv_forward_cost(const Geometry& g)
+{
+    const double pv = (double)g.packs * g.add_outer * g.add_inner;
+    if (g.thin || g.act_item_inner || g.wo < 2) {
+        // lanes over OR members, or workgroups that share out the pairs themselves: no rounding modelled
+        const double waves = ((double)g.n * g.wo * g.ho / 128.0 + 1.0) * g.n_cotile;
+        return waves * pv / 4096.0;
+    }
+    const int wk = g.w_k == 1 || g.w_k == 3 || g.w_k == 5 ? g.w_k : 0;
+    const SplitPlan sp = plan_splits(g, wk ? 2 : 1, wk, false);
+    const double rounds = (double)((sp.waves * sp.splits + 4095) / 4096);
+    return rounds * sp.pv_per_block;
+}
 
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator)
 {

@@ -3,7 +3,8 @@
 // A stream bit is [code > state], the register being advanced before each comparison
 // (sc.cpp:365-378, :429-432).  All six registers are maximal, so the states an element
 // sees are one fixed cycle of period L-1 entered at an offset that depends on its seed
-// only.  Instead of stepping a register L times per element, a per-call table holds, for
+// only.  Instead of stepping a register L times per element, a table per stream length (evaluated at
+// compile time, part of the code object) holds, for
 // every code, the comparison results along that cycle as a bit string; an element's P
 // stream words are then P funnel shifts out of the string at its seed's offset.  The few
 // leading cycles that progressive loading alters are patched bit by bit from the same
@@ -16,14 +17,9 @@ namespace {
 
 constexpr int kGenThreads = 256;
 
-__device__ __forceinline__ uint32_t lfsr_step(uint32_t s, uint32_t tap_mask, uint32_t state_mask)
-{
-    // Fibonacci LFSR: shift left, feed back the parity of the tapped bits.
-    // taps (bit indices): 3:{2,1} 4:{3,2} 5:{4,2} 6:{5,4} 7:{6,5} 8:{7,5,4,3}  (sc.cpp:262-290)
-    return ((s << 1) & state_mask) | (__popc(s & tap_mask) & 1u);
-}
-
-__host__ __device__ inline uint32_t tap_mask_for(int n_bits)
+// Fibonacci LFSR: shift left, feed back the parity of the tapped bits.
+// taps (bit indices): 3:{2,1} 4:{3,2} 5:{4,2} 6:{5,4} 7:{6,5} 8:{7,5,4,3}  (sc.cpp:262-290)
+constexpr uint32_t tap_mask_for(int n_bits)
 {
     switch (n_bits) {
     case 3: return 0x06u;
@@ -35,33 +31,56 @@ __host__ __device__ inline uint32_t tap_mask_for(int n_bits)
     }
 }
 
-// One block.  tables = posp1[L] (entry L-1 unused) followed by thr[L][wpc].
-__global__ __launch_bounds__(kGenThreads) void k_build_tables(uint32_t* __restrict__ tables, int L, int n_bits)
+constexpr uint32_t lfsr_step(uint32_t s, uint32_t tap_mask, uint32_t state_mask)
 {
-    __shared__ uint16_t cyc[256];
-    const int period = L - 1;
-    if (threadIdx.x == 0) {
+    return ((s << 1) & state_mask) | ((uint32_t)__builtin_popcount(s & tap_mask) & 1u);
+}
+
+// Stream tables of one stream length L = 2^NB, evaluated by the compiler and stored in the code object:
+// posp1[L] (entry L-1 unused) followed by thr[L][wpc] (see sc_common.h).  They depend on L alone, so
+// no launch has to build them.
+template <int NB>
+struct StreamTables {
+    static constexpr int L = 1 << NB, kPeriod = L - 1, kWpc = table_words_per_code(L);
+    uint32_t v[L + L * kWpc];
+    constexpr StreamTables() : v{}
+    {
+        // the register's cycle from state 1
+        uint32_t cyc[L] = {};
         uint32_t s = 1;
-        const uint32_t tm = tap_mask_for(n_bits), sm = (uint32_t)L - 1u;
-        for (int j = 0; j < period; j++) {
-            cyc[j] = (uint16_t)s;
-            s = lfsr_step(s, tm, sm);
+        for (int j = 0; j < kPeriod; j++) {
+            cyc[j] = s;
+            s = lfsr_step(s, tap_mask_for(NB), (uint32_t)(L - 1));
         }
+        for (int j = 0; j < kPeriod; j++) v[cyc[j] - 1] = (uint32_t)(j + 1);
+        for (int code = 0; code < L; code++)
+            for (int wi = 0; wi < kWpc; wi++) {
+                int j = (wi * 32) % kPeriod;
+                uint32_t word = 0;
+                for (int b = 0; b < 32; b++) {
+                    word = (word << 1) | (uint32_t)(code > (int)cyc[j]);
+                    j = (j + 1 == kPeriod) ? 0 : j + 1;
+                }
+                v[L + code * kWpc + wi] = word;
+            }
     }
-    __syncthreads();
-    for (int j = threadIdx.x; j < period; j += kGenThreads) tables[cyc[j] - 1] = (uint32_t)(j + 1);
-    if (threadIdx.x == 0) tables[L - 1] = 0;
-    const int wpc = table_words_per_code(L);
-    uint32_t* thr = tables + L;
-    for (int idx = threadIdx.x; idx < L * wpc; idx += kGenThreads) {
-        const int code = idx / wpc, wi = idx % wpc;
-        int j = (wi * 32) % period;
-        uint32_t word = 0;
-        for (int b = 0; b < 32; b++) {
-            word = (word << 1) | (uint32_t)(code > (int)cyc[j]);
-            j = (j + 1 == period) ? 0 : j + 1;
-        }
-        thr[idx] = word;
+};
+__device__ const StreamTables<3> kTables8{};
+__device__ const StreamTables<4> kTables16{};
+__device__ const StreamTables<5> kTables32{};
+__device__ const StreamTables<6> kTables64{};
+__device__ const StreamTables<7> kTables128{};
+__device__ const StreamTables<8> kTables256{};
+
+__device__ __forceinline__ const uint32_t* stream_tables(int L)
+{
+    switch (L) {
+    case 8: return kTables8.v;
+    case 16: return kTables16.v;
+    case 32: return kTables32.v;
+    case 64: return kTables64.v;
+    case 128: return kTables128.v;
+    default: return kTables256.v;
     }
 }
 
@@ -101,8 +120,9 @@ __device__ __forceinline__ uint32_t stream_word(const uint32_t* thr_lds, int cod
     return word;
 }
 
-__device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, const uint32_t* __restrict__ tables, int L, int wpc)
+__device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, int L, int wpc)
 {
+    const uint32_t* __restrict__ tables = stream_tables(L);
     const int n = L + L * wpc;
     for (int i = threadIdx.x; i < n; i += kGenThreads) lds[i] = tables[i];
     __syncthreads();
@@ -115,13 +135,13 @@ __device__ __forceinline__ void load_tables_to_lds(uint32_t* lds, const uint32_t
 template <bool ITEM_INNER, typename XT, int V = 1>
 __global__ __launch_bounds__(kGenThreads) void k_act_streams(const XT* __restrict__ x,
                                                             uint32_t* __restrict__ streams,
-                                                            const uint32_t* __restrict__ tables, GenParams gp, int n,
+                                                            GenParams gp, int n,
                                                             int c_in, int w_in, int h_in, int pad_w, int pad_h,
                                                             uint32_t seed_wrap)
 {
     static_assert(V == 1 || (V == 4 && !ITEM_INNER), "four elements per thread along the item's flat index only");
     extern __shared__ uint32_t lds[];
-    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    load_tables_to_lds(lds, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
     const int wi = w_in + 2 * pad_w, hi = h_in + 2 * pad_h;
@@ -196,11 +216,11 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const XT* __restric
 // (h, k, padded c_out), c_out fastest so that a wave writes whole tiles.
 __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __restrict__ w,
                                                                uint32_t* __restrict__ streams,
-                                                               const uint32_t* __restrict__ tables, GenParams gp,
-                                                               int c_out, int c_in, int w_k, int h_k, int n_cotile)
+                                                               GenParams gp, int c_out, int c_in, int w_k, int h_k,
+                                                               int n_cotile)
 {
     extern __shared__ uint32_t lds[];
-    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    load_tables_to_lds(lds, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
     const int k_or = c_in * w_k;
@@ -241,14 +261,14 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __r
 // (a caller whose convolution kernel reads the rail-packed copy only).
 __global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float* __restrict__ w,
                                                                     uint32_t* __restrict__ streams,
-                                                                    const uint32_t* __restrict__ tables, GenParams gp,
-                                                                    int c_out, int c_in, int w_k, int h_k, int n_cotile,
+                                                                    GenParams gp, int c_out, int c_in, int w_k,
+                                                                    int h_k, int n_cotile,
                                                                     int v_chunks, uint32_t* __restrict__ rail_words,
                                                                     uint16_t* __restrict__ rail_fields,
                                                                     size_t rail_lines, int two_rail)
 {
     extern __shared__ uint32_t lds[];
-    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    load_tables_to_lds(lds, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
     float* wt = reinterpret_cast<float*>(lds + gp.L + gp.L * gp.wpc);  // [row][member][channel], rows of 17
@@ -306,12 +326,11 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float
 // u*h_k + v (sc_cuda_kernel.cu:322-324).  Otherwise: outer group = block of zu input channels,
 // inner group = kernel row, seed index (channel within the block)*w_k + u (:232).
 __global__ __launch_bounds__(kGenThreads) void k_weight_streams_grouped(
-    const float* __restrict__ w, uint32_t* __restrict__ streams, const uint32_t* __restrict__ tables, GenParams gp,
-    int c_out, int c_in, int w_k, int h_k, int n_cotile, int z_mode, int add_outer, int add_inner, int or_ch_total,
+    const float* __restrict__ w, uint32_t* __restrict__ streams, GenParams gp, int c_out, int c_in, int w_k, int h_k, int n_cotile, int z_mode, int add_outer, int add_inner, int or_ch_total,
     int zu)
 {
     extern __shared__ uint32_t lds[];
-    load_tables_to_lds(lds, tables, gp.L, gp.wpc);
+    load_tables_to_lds(lds, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
     const int co_pad = n_cotile * kCoTile;
@@ -457,11 +476,13 @@ __device__ __forceinline__ void random_stream(const RandParams& rp, int code, ui
     }
 }
 
-// Activation streams [n][P][c_in][Wi][Hi] of the random generators; element index = flat index in
-// the padded tensor (n, c_in, Wi, Hi).  Padding positions give zero words.
+// Activation streams [n][P][c_in][Wi][Hi] of the random generators; element index = index0 + flat index in
+// the padded tensor (n, c_in, Wi, Hi), index0 being the index of the first item when x is a slice of a
+// larger batch.  Padding positions give zero words.
 __global__ __launch_bounds__(kGenThreads) void k_act_streams_random(const float* __restrict__ x,
                                                                    uint32_t* __restrict__ streams, RandParams rp, int n,
-                                                                   int c_in, int w_in, int h_in, int pad_w, int pad_h)
+                                                                   int c_in, int w_in, int h_in, int pad_w, int pad_h,
+                                                                   uint64_t index0)
 {
     const int wi = w_in + 2 * pad_w, hi = h_in + 2 * pad_h;
     const uint32_t plane = (uint32_t)c_in * wi * hi;
@@ -481,7 +502,7 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams_random(const float*
             code = (int)ceilf(fminf(fmaxf(v * Lf, 0.0f), top));
         }
         uint32_t* dst = streams + (size_t)item * rp.packs * plane + i;
-        random_stream(rp, code, 0u, (uint64_t)e, [&](int pk, uint32_t word) { dst[(size_t)pk * plane] = word; });
+        random_stream(rp, code, 0u, index0 + e, [&](int pk, uint32_t word) { dst[(size_t)pk * plane] = word; });
     }
 }
 
@@ -560,21 +581,15 @@ int grid_for(size_t total)
 
 }  // namespace
 
-int launch_build_tables(const Geometry& g, uint32_t* tables, hipStream_t s)
-{
-    hipLaunchKernelGGL(k_build_tables, dim3(1), dim3(kGenThreads), 0, s, tables, g.L, g.n_bits);
-    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
-}
-
 template <typename XT>
-static int launch_act_streams_t(const Geometry& g, const XT* x, uint32_t* streams, const uint32_t* tables,
-                                hipStream_t s)
+static int launch_act_streams_t(const Geometry& g, const XT* x, uint32_t* streams, hipStream_t s, size_t item0)
 {
     if (g.generator != GEO_SC_GEN_LFSR) {
         if (sizeof(XT) != sizeof(float)) return GEO_SC_ERR_UNSUPPORTED;  // fp32 activations only
         const size_t n_el = (size_t)g.n * g.act_plane;
         hipLaunchKernelGGL(k_act_streams_random, dim3(grid_for(n_el)), dim3(kGenThreads), 0, s, (const float*)x,
-                           streams, rand_params(g), g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h);
+                           streams, rand_params(g), g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h,
+                           (uint64_t)item0 * g.act_plane);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     const GenParams gp = gen_params(g, g.load_wait_a);
@@ -582,29 +597,48 @@ static int launch_act_streams_t(const Geometry& g, const XT* x, uint32_t* stream
     const uint32_t wrap = (uint32_t)g.seed_wrap;
     if (g.act_item_inner)
         hipLaunchKernelGGL((k_act_streams<true, XT>), dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, x,
-                           streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
+                           streams, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     else if (g.act_plane % 4 == 0 && ((uintptr_t)streams & 15) == 0)
         hipLaunchKernelGGL((k_act_streams<false, XT, 4>), dim3(grid_for(total / 4)), dim3(kGenThreads), table_bytes(g.L),
-                           s, x, streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
+                           s, x, streams, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     else
         hipLaunchKernelGGL((k_act_streams<false, XT>), dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s,
-                           x, streams, tables, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
+                           x, streams, gp, g.n, g.c_in, g.w_in, g.h_in, g.pad_w, g.pad_h, wrap);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
-int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, const uint32_t* tables, hipStream_t s)
+// the table the generators read for stream length L, from the host's evaluation of the same constructor
+const uint32_t* stream_tables_host(int L, size_t* words)
 {
-    return launch_act_streams_t(g, x, streams, tables, s);
+    static constexpr StreamTables<3> t8{};
+    static constexpr StreamTables<4> t16{};
+    static constexpr StreamTables<5> t32{};
+    static constexpr StreamTables<6> t64{};
+    static constexpr StreamTables<7> t128{};
+    static constexpr StreamTables<8> t256{};
+    *words = (size_t)L + (size_t)L * table_words_per_code(L);
+    switch (L) {
+    case 8: return t8.v;
+    case 16: return t16.v;
+    case 32: return t32.v;
+    case 64: return t64.v;
+    case 128: return t128.v;
+    case 256: return t256.v;
+    default: *words = 0; return nullptr;
+    }
 }
 
-int launch_act_streams_q7(const Geometry& g, const uint8_t* x, uint32_t* streams, const uint32_t* tables,
-                          hipStream_t s)
+int launch_act_streams(const Geometry& g, const float* x, uint32_t* streams, hipStream_t s, size_t item0)
 {
-    return launch_act_streams_t(g, x, streams, tables, s);
+    return launch_act_streams_t(g, x, streams, s, item0);
 }
 
-int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, const uint32_t* tables,
-                          hipStream_t s, bool rail_only)
+int launch_act_streams_q7(const Geometry& g, const uint8_t* x, uint32_t* streams, hipStream_t s)
+{
+    return launch_act_streams_t(g, x, streams, s, 0);
+}
+
+int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, hipStream_t s, bool rail_only)
 {
     if (g.generator != GEO_SC_GEN_LFSR) {
         const size_t n_el = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
@@ -617,7 +651,7 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
         const size_t padded =
             (size_t)g.add_outer * g.add_inner * g.or_ch_per_group * g.w_k * g.n_cotile * kCoTile;
         hipLaunchKernelGGL(k_weight_streams_grouped, dim3(grid_for(padded)), dim3(kGenThreads), table_bytes(g.L), s,
-                           w, streams, tables, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile,
+                           w, streams, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile,
                            g.mode == GEO_SC_ACC_Z ? 1 : 0, g.add_outer, g.add_inner, g.or_ch_total, g.or_ch_per_group);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
@@ -626,7 +660,7 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
         const size_t n_blocks = (size_t)v_chunks * k_chunks * g.n_cotile;
         const bool two_rail = !(rail_only && g.wgt_rail);
         hipLaunchKernelGGL(k_weight_streams_rows, dim3((unsigned)(n_blocks > 256 * 16 ? 256 * 16 : n_blocks)),
-                           dim3(kGenThreads), table_bytes(g.L) + 16 * 16 * 17 * sizeof(float), s, w, streams, tables, gp,
+                           dim3(kGenThreads), table_bytes(g.L) + 16 * 16 * 17 * sizeof(float), s, w, streams, gp,
                            g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile, v_chunks,
                            g.wgt_rail ? streams + g.wgt_rail_off : nullptr,
                            g.wgt_rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
@@ -635,7 +669,7 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
     }
     const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
     hipLaunchKernelGGL(k_weight_streams, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, w, streams,
-                       tables, gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile);
+                       gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

@@ -49,6 +49,10 @@ class CONV_tiny_add_partial(nn.Module):
         # training mode on the GPU with the LFSR kernels: run every conv + batch norm + pool +
         # hardtanh block as one fused autograd node (same values; gradients to fp32 rounding)
         self.fused_blocks = False
+        # batch statistics of the fused blocks: False = from exact integer sums of the counts (one HIP kernel,
+        # independent of any reduction order), True = PyTorch's two float reductions, as BatchNorm*_fixed runs
+        # them (utils_class.py:52-56): bit-identical to the module chain
+        self.fused_torch_stats = False
         if uniform:
             self.conv1.weight_org *= 2
             self.conv2.weight_org *= 2
@@ -68,7 +72,8 @@ class CONV_tiny_add_partial(nn.Module):
     def _fused(self, conv, bn, x, i, j, **tail):
         return utils_class.sc_conv_block(conv, bn, x, err=self.err[i], forward=self.compute,
                                          z_unit=2 ** self.z_unit[i], load_unit=self.load_unit[i],
-                                         load_wait_w=self.load_wait[j], load_wait_a=self.load_wait[i], **tail)
+                                         load_wait_w=self.load_wait[j], load_wait_a=self.load_wait[i],
+                                         torch_stats=self.fused_torch_stats, **tail)
 
     def _block(self, conv, bn, x, i):
         if self._fusable(x):

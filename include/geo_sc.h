@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define GEO_SC_VERSION 1
+#define GEO_SC_VERSION 2
 #define GEO_SC_API __attribute__((visibility("default")))
 
 /* A hipStream_t, passed as an opaque pointer so that C consumers need no HIP headers.
@@ -107,19 +107,56 @@ typedef struct geo_sc_conv_desc {
     int32_t seed;         /* key of the random generators (its 32 bits); unused with GEO_SC_GEN_LFSR */
 } geo_sc_conv_desc;
 
+/*
+ * Choices of the caller that are not part of the problem.  No counterpart in the reference, whose GPU op
+ * sizes and allocates its scratch itself on every call (sc_cuda_kernel.cu:1747-1796).  A NULL pointer, or a
+ * zero field, means the default.  struct_bytes = sizeof(geo_sc_options) of the caller's build.
+ *   forward_stream_bytes       budget of the forward's activation stream buffer.  A batch whose streams
+ *                              exceed it is processed in chunks of items, each chunk's streams generated
+ *                              into the same buffer and consumed by its own convolution launch (weight
+ *                              streams once); the counts do not depend on the cut.  At least one item's
+ *                              streams are always held.  Default 256 MiB.  The reference likewise keeps
+ *                              activation streams for 128 thread blocks whatever the batch
+ *                              (sc_cuda_kernel.cu:658-662, :1787-1789).
+ *   backward_groups_per_round  the backward processes its add groups (kernel rows in mode Y) in rounds of
+ *                              launches of as many groups as fit about 3 GB of scratch; this lowers that
+ *                              number and the workspace size with it.  Default: no further cap.
+ * The same options must be given to a size query and to the call that uses the workspace.
+ */
+typedef struct geo_sc_options {
+    size_t struct_bytes;
+    size_t forward_stream_bytes;
+    int32_t backward_groups_per_round;
+    int32_t reserved;
+} geo_sc_options;
+
 /* Library version (GEO_SC_VERSION of the build). */
 GEO_SC_API int geo_sc_version(void);
+
+/*
+ * Optional.  Looks up, for the current device, what the library keeps per device (the address of the static
+ * workspace of geo_sc_conv2d_add_partial_forward_static).  Entry points do this themselves at their first
+ * call on a device; a caller that records HIP graphs calls it once per device beforehand, because the
+ * lookup is not stream-ordered work and must not happen inside a stream capture.  No counterpart in the
+ * reference.
+ */
+GEO_SC_API int geo_sc_init(void);
 
 /* Static, human-readable text of a status code. */
 GEO_SC_API const char* geo_sc_status_string(int status);
 
 /*
- * Bytes of device scratch the forward needs for `desc` (tables + bit-packed weight streams
- * + bit-packed activation streams).  The reference allocates the same buffers itself with
+ * Bytes of device scratch the forward needs for `desc` (bit-packed weight streams + the bit-packed
+ * activation streams of one chunk of the batch).  The reference allocates the same buffers itself with
  * cudaMallocManaged on every call (sc_cuda_kernel.cu:1747-1796); here the caller brings
  * them so that a framework allocator can be used.
  */
 GEO_SC_API int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
+GEO_SC_API int geo_sc_conv2d_add_partial_workspace_size_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                                           size_t* bytes);
+/* Batch items per chunk of the forward under `options` (desc->n when the batch is not cut). */
+GEO_SC_API int geo_sc_conv2d_add_partial_forward_chunk(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                                       int* items_per_chunk);
 
 /*
  * SC convolution forward with y-dimension (H) partial binary accumulation and LFSR stream
@@ -134,10 +171,15 @@ GEO_SC_API int geo_sc_conv2d_add_partial_workspace_size(const geo_sc_conv_desc* 
  *
  * x: (n, c_in, w_in, h_in) fp32;  w: (c_out, c_in, w_k, h_k) fp32;
  * y: (n, c_out, Wo, Ho) int32, fully overwritten.
- * workspace: at least the size reported above, 256-byte aligned.
+ * workspace: at least the size reported above, 256-byte aligned.  The workspace holds the weight streams
+ * and the activation streams of one chunk of the batch (geo_sc_options.forward_stream_bytes); the _ex form
+ * takes the options, the plain form runs with the defaults.
  */
 GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, const float* x, const float* w, int32_t* y,
                                       void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
+GEO_SC_API int geo_sc_conv2d_add_partial_forward_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                                    const float* x, const float* w, int32_t* y, void* workspace,
+                                                    size_t workspace_bytes, geo_sc_stream_t stream);
 
 /*
  * The two stream generators on their own (the forward runs exactly these kernels).
@@ -163,9 +205,22 @@ GEO_SC_API int geo_sc_conv2d_add_partial_forward(const geo_sc_conv_desc* desc, c
  * words pos | neg, then per line 8 words holding 16 bits per channel: which rail);
  * geo_sc_weight_stream_words is the size of the whole buffer, geo_sc_weight_streams fills all of it.
  *
- * `tables` is scratch of geo_sc_stream_tables_size(L) bytes.
+ * `tables` is not used and may be NULL: the comparison tables of the six stream lengths are constant
+ * data of the library (until version 1 they were built per call into this scratch);
+ * geo_sc_stream_tables_size reports 0 bytes.  The arguments remain so that callers need not change.
+ * These stage entry points work on the whole batch at once (no chunks): above 4 GiB of activation streams
+ * geo_sc_conv2d_add_partial_from_streams runs the kernels that process both rails (about half the speed),
+ * and the item-innermost layout is not used.
  */
 GEO_SC_API int geo_sc_stream_tables_size(int bit_length, size_t* bytes);
+/*
+ * The comparison table of one stream length as the generators read it, copied to HOST memory (for
+ * inspection and tests; no GPU needed): posp1[L], then thr[L][wpc] with wpc = (2 L + 31) / 32 + 2.
+ * posp1[s - 1] = 1 + index of LFSR state s in the register's cycle from state 1 (sc.cpp:262-290;
+ * entry L - 1 unused); thr[code] = the bits [code > cycle[j mod (L - 1)]], j = 0, 1, ..., MSB-first.
+ * *words receives the table's size; host_words may be NULL to query it.
+ */
+GEO_SC_API int geo_sc_stream_table_copy(int bit_length, uint32_t* host_words, size_t capacity_words, size_t* words);
 GEO_SC_API int geo_sc_act_streams(const geo_sc_conv_desc* desc, const float* x, uint32_t* streams, void* tables,
                        geo_sc_stream_t stream);
 GEO_SC_API int geo_sc_weight_streams(const geo_sc_conv_desc* desc, const float* w, uint32_t* streams, void* tables,
@@ -212,14 +267,19 @@ GEO_SC_API int geo_sc_weight_stream_words(const geo_sc_conv_desc* desc, size_t* 
  * be NULL to skip it.  bit_length and the loading fields of `desc` are validated but do not
  * enter the result.
  * The add groups (kernel rows in mode Y) are processed in rounds of launches of as many groups as
- * fit about 3 GB of scratch; the environment variable GEO_SC_BACKWARD_GROUPS_PER_ROUND (an integer
- * >= 1, read at every call) lowers that number and the workspace size with it.  It must not change
- * between the size query and the call that uses the workspace.
+ * fit about 3 GB of scratch; geo_sc_options.backward_groups_per_round (the _ex forms) lowers that number
+ * and the workspace size with it.  The result does not depend on it beyond fp32 summation order of grad_x.
  */
 GEO_SC_API int geo_sc_conv2d_add_partial_backward_workspace_size(const geo_sc_conv_desc* desc, size_t* bytes);
 GEO_SC_API int geo_sc_conv2d_add_partial_backward(const geo_sc_conv_desc* desc, const float* x, const float* w,
                                                   const float* grad_y, float* grad_x, float* grad_w,
                                                   void* workspace, size_t workspace_bytes, geo_sc_stream_t stream);
+GEO_SC_API int geo_sc_conv2d_add_partial_backward_workspace_size_ex(const geo_sc_conv_desc* desc,
+                                                                    const geo_sc_options* options, size_t* bytes);
+GEO_SC_API int geo_sc_conv2d_add_partial_backward_ex(const geo_sc_conv_desc* desc, const geo_sc_options* options,
+                                                     const float* x, const float* w, const float* grad_y,
+                                                     float* grad_x, float* grad_w, void* workspace,
+                                                     size_t workspace_bytes, geo_sc_stream_t stream);
 
 /*
  * Layer epilogue fused into one pass over the convolution's int32 counts.  Replaces the chain of
@@ -320,16 +380,20 @@ GEO_SC_API int geo_sc_act_streams_q7(const geo_sc_conv_desc* desc, const uint8_t
 /*
  * geo_sc_conv2d_add_partial_forward for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
- * reference.  Same arguments and result, without the workspace: tables and both stream buffers live
+ * reference.  Same arguments and result, without the workspace: both stream buffers live
  * in a static device array of GEO_SC_STATIC_WORKSPACE_BYTES inside the library, which every GPU the
  * library runs on holds until the process ends.  The call allocates and frees nothing and clears
- * nothing with memset nodes.  A problem whose geo_sc_conv2d_add_partial_workspace_size exceeds the
- * limit returns GEO_SC_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls that overlap
- * on one GPU (different streams, different threads) race; calls on one stream do not.
+ * nothing with memset nodes.  The array is the activation stream budget: the weight streams come first,
+ * the batch is cut into chunks whose streams fit behind them.  A problem whose weight streams plus one
+ * item's activation streams exceed the array returns GEO_SC_ERR_WORKSPACE.  All calls on one GPU share
+ * that GPU's array: calls that overlap on one GPU (different streams, different threads) race; calls on one
+ * stream do not.  Under stream capture: call geo_sc_init (or this entry point once) on the device before
+ * the capture begins.  geo_sc_static_workspace_bytes returns the limit of the loaded library.
  */
 #define GEO_SC_STATIC_WORKSPACE_BYTES ((size_t)32 << 20)
 GEO_SC_API int geo_sc_conv2d_add_partial_forward_static(const geo_sc_conv_desc* desc, const float* x, const float* w,
                                                         int32_t* y, geo_sc_stream_t stream);
+GEO_SC_API size_t geo_sc_static_workspace_bytes(void);
 
 #ifdef __cplusplus
 }

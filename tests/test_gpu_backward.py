@@ -1,6 +1,12 @@
 """GPU parity of the HIP surrogate backward, through the C ABI and through the autograd
 binding.  Tolerance (stated by the task for fp32 gradients): 1e-5 relative, measured as
-max|got - ref| <= 1e-5 * max|ref| against the float64 gradient oracle."""
+max|got - ref| <= 1e-5 * max|ref| against the float64 gradient oracle.
+
+TIGHT = 2e-6 is held in addition by every case whose products run on the matrix cores.  The kernels form
+an fp32 product from six bf16 term products of a three-way operand split, which is as accurate as an fp32
+GEMM: the errors observed on the full-size shapes are 2e-7 .. 8e-7 of max|ref|.  The mistake that
+arithmetic invites - dropping the low-order terms, three products instead of six - gives about 4e-6 and
+would still pass the 1e-5 bound; TIGHT sits between the two, so that variant fails here."""
 import numpy as np
 import pytest
 import torch
@@ -10,6 +16,7 @@ from geo_amd import workloads as wl
 pytestmark = pytest.mark.gpu
 
 RTOL = 1e-5
+TIGHT = 2e-6
 
 
 @pytest.fixture(scope="module")
@@ -22,6 +29,14 @@ def capi():
 def rel_err(got, ref):
     ref = ref.double().cpu()
     return ((got.double().cpu() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+
+
+def check(what, got, ref, bound=TIGHT):
+    """Asserts max|got - ref| <= bound * max|ref| and prints the observed level (pytest -s / on failure)."""
+    e = rel_err(got, ref)
+    print(f"{what}: error {e:.2e} of max|ref| (bound {bound:.0e})")
+    assert e <= bound, (what, e, bound)
+    return e
 
 
 CASES = [
@@ -49,14 +64,15 @@ def test_backward_matches_float64_oracle(capi, shape_x, shape_w, pad, mode, scal
     torch.cuda.synchronize()
     rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad)
     assert gx.shape == x.shape and gw.shape == w.shape
-    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
-    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    check("grad_x", gx, rx)
+    check("grad_w", gw, rw)
     # skipping one output leaves the other unchanged (a weight gradient asked for alone may take the
     # fused kernel for small OR groups: same value up to the summation order)
     gx2, none = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_w=False)
     none2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad, need_grad_x=False)
     assert none is None and none2 is None
-    assert torch.equal(gx2, gx) and rel_err(gw2, gw) <= 1e-6 and rel_err(gw2, rw) <= RTOL
+    assert torch.equal(gx2, gx) and rel_err(gw2, gw) <= 1e-6
+    check("grad_w alone", gw2, rw)
 
 
 GEMM_CASES = [
@@ -94,8 +110,8 @@ def test_backward_through_the_gemm_kernels(capi, shape_x, shape_w, pad, scale):
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, pad)
     torch.cuda.synchronize()
     rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad)
-    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
-    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    check("grad_x", gx, rx)
+    check("grad_w", gw, rw)
 
 
 def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
@@ -112,8 +128,8 @@ def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
     xp = torch.nn.functional.pad(xr, (pad, pad, pad, pad))
     p, n = surrogate.surrogate_rails(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)))
     (p - n).backward(g.double())
-    assert rel_err(gx, xr.grad) <= RTOL, rel_err(gx, xr.grad)
-    assert rel_err(gw, wr.grad) <= RTOL, rel_err(gw, wr.grad)
+    check("C3 grad_x", gx, xr.grad)
+    check("C3 grad_w", gw, wr.grad)
     # linear in the upstream gradient
     gx2, gw2 = capi.conv2d_add_partial_backward(xd, wd, 2 * g, 128, (pad, pad))
     assert rel_err(gx2, 2 * gx) <= 1e-6 and rel_err(gw2, 2 * gw) <= 1e-6
@@ -138,14 +154,16 @@ def test_autograd_binding_matches_reference_composition(capi):
     g = torch.randn(y.shape, generator=torch.Generator().manual_seed(3))
     y.backward(g.cuda())
     rx, rw, _ = surrogate.surrogate_autograd(x, w, g, (1, 1), sc_value=y.detach().cpu().double())
-    assert rel_err(xg.grad, rx) <= RTOL and rel_err(wg.grad, rw) <= RTOL
+    check("grad_x", xg.grad, rx)
+    check("grad_w", wg.grad, rw)
     # host tensors go through the same kernels and come back on the host
     xc = x.clone().requires_grad_(True)
     wc = w.clone().requires_grad_(True)
     yc = uf.conv2d_generic(xc, wc, (1, 1), (1, 1), bit_length=64, forward="1d_bin", generator="lfsr")
     assert not yc.is_cuda and torch.equal(yc.detach(), y.detach().cpu())
     yc.backward(g)
-    assert rel_err(xc.grad, rx) <= RTOL and rel_err(wc.grad, rw) <= RTOL
+    check("grad_x (host tensors)", xc.grad, rx)
+    check("grad_w (host tensors)", wc.grad, rw)
     with pytest.raises(NotImplementedError):
         uf.conv2d_generic(xg, wg, (1, 1), (1, 1), bit_length=64, forward="2d_bin", generator="lfsr")
     with pytest.raises(NotImplementedError):
@@ -191,9 +209,9 @@ def test_weight_gradient_of_small_or_groups(capi, shape_x, shape_w, pad, mode, z
                                                 accumulate=mode, z_unit=zu)
     assert none is None
     _, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
-    assert rel_err(gw, rw) <= RTOL, rel_err(gw, rw)
+    check("grad_w", gw, rw)
     _, gw_general = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, accumulate=mode, z_unit=zu)
-    assert rel_err(gw, gw_general) <= RTOL
+    check("grad_w against the general path", gw, gw_general)
     _, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False,
                                               accumulate=mode, z_unit=zu)
     assert torch.equal(gw, gw2)   # deterministic
@@ -222,8 +240,8 @@ def test_backward_through_the_gemms_in_every_mode(capi, shape_x, shape_w, pad, m
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
     torch.cuda.synchronize()
     rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
-    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
-    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    check("grad_x", gx, rx)
+    check("grad_w", gw, rw)
     # an input that does not start on a 16-byte boundary takes the materialised col: same bits
     xo = torch.empty(x.numel() + 1, device="cuda")[1:].view(x.shape)
     xo.copy_(x)
@@ -257,12 +275,13 @@ def test_whole_backward_of_small_or_groups(capi, shape_x, shape_w, pad, mode, zu
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
     torch.cuda.synchronize()
     rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
-    assert rel_err(gx, rx) <= RTOL, ("grad_x", rel_err(gx, rx))
-    assert rel_err(gw, rw) <= RTOL, ("grad_w", rel_err(gw, rw))
+    check("grad_x", gx, rx)
+    check("grad_w", gw, rw)
     gx2, none = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_w=False, **kw)
     none2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False, **kw)
     assert none is None and none2 is None
-    assert torch.equal(gx2, gx) and rel_err(gw2, rw) <= RTOL
+    assert torch.equal(gx2, gx)
+    check("grad_w alone", gw2, rw)
     gx3, gw3 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
     assert torch.equal(gx3, gx) and torch.equal(gw3, gw)   # deterministic
 
@@ -276,8 +295,8 @@ def test_whole_backward_of_small_or_groups(capi, shape_x, shape_w, pad, mode, zu
     ((2, 44, 6, 6), (5, 44, 3, 3), (1, 1), "yz", 20, 2),   # yz through the GEMMs (K = 60), ragged last block, rounds of 2
     ((4, 3, 9, 9), (16, 3, 5, 5), (2, 2), "y", 1, 2),      # weight gradient alone of a first layer (K = 15)
 ])
-def test_backward_in_several_rounds_of_add_groups(capi, monkeypatch, shape_x, shape_w, pad, mode, zu, cap):
-    """GEO_SC_BACKWARD_GROUPS_PER_ROUND forces what a 3 GB scratch budget only does for very large
+def test_backward_in_several_rounds_of_add_groups(capi, shape_x, shape_w, pad, mode, zu, cap):
+    """geo_sc_options.backward_groups_per_round forces what a 3 GB scratch budget only does for very large
     layers: the add groups go through the kernels in several rounds, later rounds accumulating into
     grad_x.  Same gradients as in one round and as the float64 oracle."""
     from oracle import surrogate
@@ -289,14 +308,21 @@ def test_backward_in_several_rounds_of_add_groups(capi, monkeypatch, shape_x, sh
     kw = dict(accumulate=mode, z_unit=zu)
     one_x, one_w = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
     bytes_one = capi.backward_workspace_size(d)
-    monkeypatch.setenv("GEO_SC_BACKWARD_GROUPS_PER_ROUND", str(cap))
-    assert capi.backward_workspace_size(d) < bytes_one
+    opt = capi.make_options(backward_groups_per_round=cap)
+    assert capi.backward_workspace_size(d, opt) < bytes_one
+    kw["options"] = opt
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, **kw)
     _, gw_alone = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, need_grad_x=False, **kw)
     torch.cuda.synchronize()
-    monkeypatch.delenv("GEO_SC_BACKWARD_GROUPS_PER_ROUND")
+    # a workspace sized for the capped rounds is too small for the uncapped call: refused, not overrun
+    small = torch.empty(capi.backward_workspace_size(d, opt), dtype=torch.uint8, device="cuda")
+    with pytest.raises(capi.GeoScError):
+        capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 64, pad, workspace=small, accumulate=mode,
+                                         z_unit=zu)
     rx, rw, _ = surrogate.surrogate_autograd(x, w, g, pad, mode=mode, z_unit=zu)
-    assert rel_err(gx, rx) <= RTOL and rel_err(gw, rw) <= RTOL and rel_err(gw_alone, rw) <= RTOL
+    check("grad_x", gx, rx)
+    check("grad_w", gw, rw)
+    check("grad_w alone", gw_alone, rw)
     assert rel_err(gx, one_x) <= 1e-6 and rel_err(gw, one_w) <= 1e-6
 
 
@@ -320,9 +346,8 @@ def test_backward_resnet_shape_full_size(capi):
     g = torch.randn((128, 64, 56, 56), generator=torch.Generator().manual_seed(3))
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 256, (pad, pad))
     rx, rw = _fp64_reference_on_gpu(x, w, g, pad)
-    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
-    print(f"C5 backward: grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
-    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    check("C5 grad_x", gx, rx)
+    check("C5 grad_w", gw, rw)
     gx2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 256, (pad, pad))
     assert torch.equal(gx2, gx) and torch.equal(gw2, gw)   # deterministic
 
@@ -337,10 +362,40 @@ def test_backward_linear_4096_shape(capi):
     g = torch.randn((64, 4096, 1, 1), generator=torch.Generator().manual_seed(5))
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad))
     rx, rw = _fp64_reference_on_gpu(x, w, g, pad)
-    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
-    print(f"C4 backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
-    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    check("C4 (batch 64) grad_x", gx, rx)
+    check("C4 (batch 64) grad_w", gw, rw)
     assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
+
+
+def test_backward_linear_4096_full_batch(capi):
+    """The same layer at its full batch of 1024 (8192 workgroups of the fused kernel, 32 dcol slices of the whole
+    batch): a float64 reference of that size is out of reach, so the batch-64 result, which the test above holds
+    against float64, is carried over by what the mathematics fixes.  Items are independent in grad_x (an item's
+    input gradient depends on its own activations and upstream gradient only), so the first 64 items of the
+    full-batch grad_x equal the batch-64 call's; grad_w is linear in the upstream gradient, so with the
+    gradient of all other items zeroed it equals the batch-64 call's, and with the full gradient it is the sum
+    over the sixteen slices of 64 items."""
+    x, w, pad, _ = wl.named("C4", "q7")
+    w = (w * 16).contiguous()
+    xd, wd = x.cuda(), w.cuda()
+    g = torch.randn((1024, 4096, 1, 1), generator=torch.Generator().manual_seed(5)).cuda()
+    gx, gw = capi.conv2d_add_partial_backward(xd, wd, g, 128, (pad, pad))
+    gx64, gw64 = capi.conv2d_add_partial_backward(xd[:64].contiguous(), wd, g[:64].contiguous(), 128, (pad, pad))
+    check("C4 full batch, grad_x of the first 64 items against the batch-64 call", gx[:64], gx64)
+    g_first = g.clone()
+    g_first[64:] = 0
+    gx_f, gw_f = capi.conv2d_add_partial_backward(xd, wd, g_first, 128, (pad, pad))
+    check("C4 full batch, grad_w with the other items' gradient zeroed against the batch-64 call", gw_f, gw64)
+    assert float(gx_f[64:].abs().max()) == 0.0
+    total = torch.zeros_like(gw64, dtype=torch.float64)
+    for i in range(0, 1024, 64):
+        total += capi.conv2d_add_partial_backward(xd[i:i + 64].contiguous(), wd, g[i:i + 64].contiguous(), 128,
+                                                  (pad, pad), need_grad_x=False)[1].double()
+    check("C4 full batch, grad_w against the sum over sixteen slices", gw, total)
+    check("C4 full batch, grad_x of the last 64 items against their own call", gx[960:],
+          capi.conv2d_add_partial_backward(xd[960:].contiguous(), wd, g[960:].contiguous(), 128, (pad, pad))[0])
+    gx2, gw2 = capi.conv2d_add_partial_backward(xd, wd, g, 128, (pad, pad))
+    assert torch.equal(gx2, gx) and torch.equal(gw2, gw)   # deterministic
 
 
 @pytest.mark.parametrize("shape_x,shape_w,pad,mode,zu", [
@@ -363,9 +418,8 @@ def test_backward_through_the_eight_wave_gemm(capi, shape_x, shape_w, pad, mode,
     kw = dict(accumulate=mode, z_unit=zu)
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad), **kw)
     rx, rw = _fp64_reference_on_gpu(x, w, g, pad, mode, zu)
-    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
-    print(f"{shape_x} * {shape_w} {mode} backward: grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
-    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    check(f"{shape_x} * {shape_w} {mode} grad_x", gx, rx)
+    check(f"{shape_x} * {shape_w} {mode} grad_w", gw, rw)
     assert float(rx.abs().max()) > 0 and float(rw.abs().max()) > 0
     xo = torch.empty(x.numel() + 1, device="cuda")[1:].view(x.shape)
     xo.copy_(x)
@@ -384,8 +438,7 @@ def test_backward_small_groups_at_the_headline_shape(capi, mode, zu):
     g = torch.randn((64, 128, 16, 16), generator=torch.Generator().manual_seed(7))
     gx, gw = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad), accumulate=mode, z_unit=zu)
     rx, rw = _fp64_reference_on_gpu(x, w, g, pad, mode, zu)
-    ex, ew = rel_err(gx, rx), rel_err(gw, rw)
-    print(f"{mode} z_unit {zu} backward (batch 64): grad_x error {ex:.2e}, grad_w error {ew:.2e} of max|ref| (bound {RTOL:.0e})")
-    assert ex <= RTOL and ew <= RTOL, (ex, ew)
+    check(f"{mode} z_unit {zu} (batch 64) grad_x", gx, rx)
+    check(f"{mode} z_unit {zu} (batch 64) grad_w", gw, rw)
     gx2, gw2 = capi.conv2d_add_partial_backward(x.cuda(), w.cuda(), g.cuda(), 128, (pad, pad), accumulate=mode, z_unit=zu)
     assert torch.equal(gx2, gx) and torch.equal(gw2, gw)   # deterministic

@@ -451,3 +451,72 @@ def test_large_y_mode_launches_skip_the_zero_rail(capi, so, shape_x, shape_w, pa
     with pytest.raises(ValueError):
         short = torch.zeros(P * H * Cin * W * ((Cout + 15) // 16) * 32, dtype=torch.int32, device="cuda")
         capi.conv2d_add_partial_from_streams(capi.act_streams(x.cuda(), d), short, d)
+
+
+# ------------------------------------------------------------------ batches cut into chunks
+@pytest.mark.parametrize("shape_x,shape_w,pad,L,kw", [
+    ((11, 6, 9, 8), (20, 6, 3, 3), (1, 1), 64, {}),                                   # position-major, 3-wide
+    ((11, 6, 9, 8), (20, 6, 3, 3), (1, 1), 128, dict(total_width=7, load_width=2, load_wait_w=2, load_wait_a=2)),
+    ((13, 16, 1, 24), (40, 16, 1, 24), (0, 0), 32, {}),                               # SC-linear mapping: item-innermost chunks,
+                                                                                      # a last chunk of one item is position-major
+    ((10, 64, 4, 4), (10, 64, 4, 4), (0, 0), 64, {}),                                 # classifier layer (lanes over OR members)
+    ((9, 5, 8, 8), (7, 5, 3, 3), (1, 1), 32, dict(accumulate="z")),
+    ((9, 8, 8, 8), (7, 8, 3, 3), (1, 1), 32, dict(accumulate="yz", z_unit=3)),
+    ((9, 4, 8, 8), (18, 4, 3, 3), (1, 1), 64, dict(generator="acc", seed=5)),         # random sequences are numbered by the
+    ((9, 4, 8, 8), (18, 4, 3, 3), (1, 1), 64, dict(generator="rand", seed=6, accumulate="full")),  # item's index in the batch
+])
+def test_forward_in_chunks_of_the_batch(capi, so, shape_x, shape_w, pad, L, kw):
+    """geo_sc_options.forward_stream_bytes below the batch's activation streams: the forward generates and
+    consumes the streams of a few items at a time (3 - 4 chunks here, the last one shorter).  Same counts as the
+    oracle and as the uncut call, bit for bit, whatever the cut."""
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_x[0] + L)
+    w = (w * 3).clamp(-1, 1).contiguous()
+    xd, wd = x.cuda(), w.cuda()
+    d = capi.make_desc(x.shape, w.shape, L, pad, **kw)
+    whole = capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d)
+    assert capi.forward_chunk(d) == shape_x[0]
+    if kw.get("generator", "lfsr") == "lfsr":
+        mode = kw.get("accumulate", "y")
+        loading = {k: v for k, v in kw.items() if k.startswith(("total", "load"))}
+        exp = so.conv2d_modes(x.numpy(), w.numpy(), L, pad, mode, kw.get("z_unit", 1), **loading)
+    else:
+        exp = so.conv2d_general(x.numpy(), w.numpy(), L, pad, kw.get("accumulate", "y"), 1, kw["generator"], kw["seed"])
+    assert np.array_equal(whole.cpu().numpy(), exp)
+    item = 4 * ((L + 31) // 32) * shape_x[1] * (shape_x[2] + 2 * pad[1]) * (shape_x[3] + 2 * pad[0])
+    seen = set()
+    for items in (1, 3, 4, 6):
+        opt = capi.make_options(forward_stream_bytes=items * item + 5)
+        nc = capi.forward_chunk(d, opt)
+        assert (items + 1) // 2 <= nc <= items
+        seen.add(nc)
+        assert capi.workspace_size(d, opt) < capi.workspace_size(d)
+        out = torch.full(capi.output_shape(d), -3, dtype=torch.int32, device="cuda")
+        capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d, out=out, options=opt)
+        assert torch.equal(out, whole), (items, nc)
+    assert len(seen) >= 3
+    # a workspace sized for chunks is refused by the call that would hold the whole batch
+    small = torch.empty(capi.workspace_size(d, capi.make_options(forward_stream_bytes=item)), dtype=torch.uint8,
+                        device="cuda")
+    with pytest.raises(capi.GeoScError) as e:
+        capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d, workspace=small)
+    assert e.value.status == 3
+
+
+def test_forward_uncut_at_the_resnet_shape(capi, checksums):
+    """The default budget cuts the batch of the 64->64 3x3 layer at 56x56 (0.88 GB of streams) into chunks -
+    test_forward_full_size_checksums runs that way; here the whole batch in one launch, same checksum, and the
+    7-bit integer entry point through its chunks."""
+    c = checksums["C5_kaiming_L256"]
+    x, w, pad, _ = wl.named(c["shape_name"], c["mode"])
+    xd, wd = x.cuda(), w.cuda()
+    d = capi.make_desc(xd.shape, wd.shape, c["L"], (pad, pad))
+    assert capi.forward_chunk(d) < 128 and capi.workspace_size(d) <= 300 << 20
+    whole = capi.make_options(forward_stream_bytes=1 << 40)
+    assert capi.forward_chunk(d, whole) == 128
+    y = capi.conv2d_add_partial_forward(xd, wd, c["L"], (pad, pad), desc=d, options=whole).cpu().numpy()
+    assert hashlib.sha256(np.ascontiguousarray(y).tobytes()).hexdigest() == c["sha256"]
+    xq7, wq7, _, _ = wl.named("C5", "q7")
+    k = (xq7 * 128).round().to(torch.uint8).cuda()
+    a = capi.conv2d_add_partial_forward_q7(k, wq7.cuda(), 256, (pad, pad))
+    b = capi.conv2d_add_partial_forward(xq7.cuda(), wq7.cuda(), 256, (pad, pad), options=whole)
+    assert torch.equal(a, b) and int(a.abs().max()) > 0
