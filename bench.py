@@ -49,6 +49,9 @@ def parse():
     ap.add_argument("--generator", default="lfsr", choices=["lfsr", "acc", "rand"])
     ap.add_argument("--pass", dest="passes", default="fwdbwd", choices=["fwd", "fwdbwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--fused-only", action="store_true",
+                    help="workload C2: time the fused, graph-replayed training step only (no module-chain and eager "
+                         "legs): the run that kernel traces of the step are taken from")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the other benchmark configurations that the default run times after the headline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
@@ -146,28 +149,44 @@ def network_step_result(args, torch):
     t = torch.randint(10, (256,), generator=g).cuda()
     crit = torch.nn.CrossEntropyLoss()
 
-    def timed_steps(fused_blocks):
-        """ms per training step; fused_blocks: every conv + batch norm + pool + hardtanh block as one
-        autograd node on the fused HIP tail kernels (same values as the module chain)."""
+    def timed_steps(fused_blocks, graph=False, torch_stats=False):
+        """ms per training step.  fused_blocks: every conv + batch norm + pool + hardtanh block as one autograd
+        node on the fused HIP tail kernels (same values as the module chain); graph: the step recorded once into
+        a HIP graph and replayed (network.GraphedTrainStep); torch_stats: batch statistics from PyTorch's float
+        reductions instead of the exact integer sums."""
         torch.manual_seed(0)
         model = network.CONV_tiny_add_partial().cuda().train()
         model.err = [L.bit_length() - 1] * 4
         model.load_unit = [2] * 4
         model.load_wait = [2] * 4
         model.fused_blocks = fused_blocks
+        model.fused_torch_stats = torch_stats
         copies = network.make_param_copies(model)
-        opt = torch.optim.Adam(copies, lr=2e-3)
+        # the optimiser of the training script (main_conv.py:213); its multi-tensor form in one kernel, step
+        # count on the device so that the step can be recorded
+        opt = torch.optim.Adam(copies, lr=2e-3, capturable=True, fused=True) if graph \
+            else torch.optim.Adam(copies, lr=2e-3)
+        if graph:
+            replay = network.GraphedTrainStep(model, crit, opt, copies, x, t)
+            step = lambda: replay(x, t)
+        else:
+            step = lambda: network.train_step(model, x.clone(), t, crit, opt, copies)
         for _ in range(args.warmup):
-            network.train_step(model, x.clone(), t, crit, opt, copies)
+            step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
-            network.train_step(model, x.clone(), t, crit, opt, copies)
+            step()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    ms_module_chain = timed_steps(False)
-    ms_per_step = timed_steps(True)
+    ms_per_step = timed_steps(True, graph=True)
+    if args.fused_only:
+        ms_module_chain = ms_eager = ms_torch_stats = None
+    else:
+        ms_module_chain = timed_steps(False)
+        ms_eager = timed_steps(True)
+        ms_torch_stats = timed_steps(True, graph=True, torch_stats=True)
 
     layers = {}
     B_total = 0
@@ -204,8 +223,13 @@ def network_step_result(args, torch):
         "data": "synthetic (torch.manual_seed(0); images U[0,1), uniform random labels)",
         "config": {"workload": "C2: 4-layer SC CNN (3->32 k5 @32, 32->32 k5 @16, 32->64 k5 @8, 64->10 k4 @4), batch "
                                f"256, stream length {L}, load_unit 2 / load_wait 2, fwd+bwd+Adam step, fused "
-                               "conv + batch-norm + pool + hardtanh blocks",
+                               "conv + batch-norm + pool + hardtanh blocks, batch statistics from exact integer sums "
+                               "of the counts, step replayed from a HIP graph",
                    "pass": "train step", "bit_macs_per_step": B_total},
+        # the same step launched kernel by kernel from Python; with PyTorch's float reductions for the batch
+        # statistics (bit-identical to the module chain); module by module with PyTorch ops between the SC kernels
+        "eager_ms_per_step": ms_eager,
+        "torch_statistics_ms_per_step": ms_torch_stats,
         "module_chain_ms_per_step": ms_module_chain,
         "layers": layers,
         "roofline": {"bound": "valu", "kernel": "the four layers' convolution launches together",
@@ -391,7 +415,9 @@ def other_configs(args, torch):
     net_args.steps, net_args.warmup, net_args.length = steps, warmup, 64
     r = network_step_result(net_args, torch)
     out["C2_L64_train_step"] = {
-        "ms_per_step": r["ms_per_step"], "module_chain_ms_per_step": r["module_chain_ms_per_step"],
+        "ms_per_step": r["ms_per_step"], "eager_ms_per_step": r["eager_ms_per_step"],
+        "torch_statistics_ms_per_step": r["torch_statistics_ms_per_step"],
+        "module_chain_ms_per_step": r["module_chain_ms_per_step"], "workload": r["config"]["workload"],
         "bit_macs_per_s": r["value"], "kernel_ms": r["roofline"]["kernel_ms_sum"],
         "executed_frac": r["roofline"]["frac"],
         "fwd_ms": sum(l["fwd_ms"] for l in r["layers"].values()),

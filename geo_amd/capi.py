@@ -255,6 +255,34 @@ def bn_fixed_affine(mean, var, gamma, beta, eps, elements_per_channel, running_m
     return w_n, b_n, invstd, scale
 
 
+def bn_fixed_from_counts(counts, bit_length, gamma, beta, eps, running_mean=None, running_var=None, eps_grad=1e-5,
+                         stream=None):
+    """geo_sc_bn_fixed_from_counts: (mean, var, w_n, b_n, invstd, scale) of a fixed-point batch norm on the batch
+    statistics of ``counts / bit_length`` (exact integer sums), updating running_mean / running_var in place
+    when given: count_stats + bn_fixed_affine in two launches."""
+    if not (counts.is_cuda and counts.dtype == torch.int32 and counts.is_contiguous() and counts.dim() in (2, 4)):
+        raise ValueError("counts must be a contiguous int32 GPU tensor (n, c, w, h) or (n, c)")
+    n, c = counts.shape[:2]
+    w, h = (counts.shape[2], counts.shape[3]) if counts.dim() == 4 else (1, 1)
+    dev = counts.device
+    for t in (gamma, beta, running_mean, running_var):
+        if t is not None and not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == c):
+            raise ValueError("parameters and running statistics must be contiguous float32 GPU tensors of c entries")
+    need = ctypes.c_size_t()
+    _check(_native.lib().geo_sc_count_stats_workspace_size(n, c, w, h, ctypes.byref(need)),
+           "geo_sc_count_stats_workspace_size")
+    ws = torch.empty(max(need.value, 8), dtype=torch.uint8, device=dev)
+    out = torch.empty((5, c), dtype=torch.float32, device=dev)   # mean, var, w_n, b_n, invstd
+    scale = torch.empty((), dtype=torch.float32, device=dev)
+    mean, var, w_n, b_n, invstd = out[0], out[1], out[2], out[3], out[4]
+    _check(_native.lib().geo_sc_bn_fixed_from_counts(_ptr(counts), n, c, w, h, int(bit_length), _ptr(gamma), _ptr(beta),
+                                                     float(eps), float(eps_grad), _ptr(running_mean),
+                                                     _ptr(running_var), _ptr(mean), _ptr(var), _ptr(w_n), _ptr(b_n),
+                                                     _ptr(invstd), _ptr(scale), _ptr(ws), ws.numel(),
+                                                     _stream_ptr(stream)), "geo_sc_bn_fixed_from_counts")
+    return mean, var, w_n, b_n, invstd, scale
+
+
 def quantize(x, prec, out=None, stream=None):
     """geo_sc_quantize: round(x * 2^prec) clamped to +-(2^prec - 1), over 2^prec, in one launch.
     ``x`` is a contiguous fp32 GPU tensor; ``out`` may be ``x`` itself."""

@@ -98,11 +98,13 @@ double conv_forward_cost(const Geometry& g);
 // fills the rail-packed part of a weight stream buffer from its two-rail lines (no-op unless g.wgt_rail;
 // with from_generator also where launch_weight_streams has written that part itself)
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator);
-// kernels long in dim 3 take the row-chunked LFSR weight generator, which also writes the rail-packed copy
-inline bool weight_rows_generator(const Geometry& g)
+// the LFSR weight generators of the y-mode line order write the rail-packed copy (and clear the flag area)
+// themselves; kernels long in dim 3 take the row-chunked one
+inline bool generator_packs_rails(const Geometry& g)
 {
-    return g.generator == GEO_SC_GEN_LFSR && (g.mode == GEO_SC_ACC_Y || g.mode == GEO_SC_ACC_FULL) && g.h_k >= 16;
+    return g.generator == GEO_SC_GEN_LFSR && (g.mode == GEO_SC_ACC_Y || g.mode == GEO_SC_ACC_FULL);
 }
+inline bool weight_rows_generator(const Geometry& g) { return generator_packs_rails(g) && g.h_k >= 16; }
 size_t backward_workspace_bytes(const Geometry& g, int groups_per_round);
 // GEO_SC_ERR_WORKSPACE when workspace_bytes is below backward_workspace_bytes(g, groups_per_round)
 int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x, const float* w, const float* gy,

@@ -1288,17 +1288,6 @@ __global__ __launch_bounds__(256) void k_shift_planes(const float* __restrict__ 
     }
 }
 
-// rows[g - g0][k]: where row k of group g's col starts in the planes of k_shift_planes (elements).
-__global__ __launch_bounds__(256) void k_view_rows(long long* __restrict__ rows, int g0, int ng, Groups G, long long plane,
-                                                   int ho, int k_pad)
-{
-    for (int e = blockIdx.x * 256 + threadIdx.x; e < ng * k_pad; e += gridDim.x * 256) {
-        const int gi = e / k_pad, k = e - gi * k_pad;
-        const Member mb = member_of(G, g0 + gi, k < G.n_members ? k : G.n_members - 1);
-        rows[e] = ((long long)mb.v * G.c_in + mb.ci) * plane + (long long)mb.u * ho;
-    }
-}
-
 // Weight operands of groups g0 + blockIdx.y:
 //   wcat[g][k][j]: j < c_out -> clamp(w,0,100), j >= c_out -> -clamp(w,-100,0)   (utils_functional.py:611-612)
 //   wd[g][j][k]  : the same with the negative rail negated (it enters dL/dx with a minus sign)
@@ -1552,27 +1541,66 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad_tiled(const float* __restr
     }
 }
 
-// 64 zeros (a fill kernel rather than a memset, so that a caller may capture the launch sequence in a graph)
-__global__ __launch_bounds__(64) void k_zero_block(float* __restrict__ p) { p[threadIdx.x] = 0.0f; }
-
-// The A operand of the input-gradient product summed over the kernel rows inside the GEMM (y
-// accumulation: group = kernel column v, members (ci, u)): wdx[g][k][ci] = wd[g][j][(ci, u)], i.e.
-// clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one, with the
-// kernel row as the fast index over chunks of kChunk columns, k = ((j / kChunk) * w_k + u) * kChunk + j % kChunk:
-// consecutive chunks of the product then read the same columns of E one image row apart (ShiftStager).
-__global__ __launch_bounds__(256) void k_weight_dx_operand(const float* __restrict__ w, float* __restrict__ wdx, int g0,
-                                                           int c_out, int c_in, int w_k, int h_k, size_t g_stride)
+// What a round of GEMM launches needs beforehand, in one launch (grid: blocks x groups of the round):
+//  * the weight operands wcat / wd of k_weight_operands, for group g0 + blockIdx.y;
+//  * with dx_rows, in wd's place, the A operand of the input-gradient product that sums the kernel rows inside
+//    the GEMM (y accumulation: group = kernel column v, members (ci, u)): wdx[g][k][ci] = wd[g][j][(ci, u)], i.e.
+//    clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one, with the
+//    kernel row as the fast index over chunks of kChunk columns, k = ((j / kChunk) * w_k + u) * kChunk + j % kChunk:
+//    consecutive chunks of the product then read the same columns of E one image row apart (ShiftStager);
+//  * from the blocks of the round's first group: view_rows[g][k], where row k of group g's col starts in the
+//    planes of k_shift_planes (elements), for every group; and 64 zeros for the shifted view of E (a store
+//    rather than a memset, so that a caller may capture the launch sequence in a graph).
+struct PrepParams {
+    const float* __restrict__ w;
+    float* __restrict__ wcat;
+    float* __restrict__ wd;
+    int g0, c_out;
+    Groups G;
+    size_t g_stride;
+    int dx_rows;            // wd holds the wdx operand (y accumulation: c_in, w_k, h_k from G)
+    long long* view_rows;   // null: no view
+    int view_groups, view_k_pad, ho;
+    long long plane;
+    float* zero;            // null: no block of zeros wanted
+};
+__global__ __launch_bounds__(256) void k_bwd_prep(PrepParams q)
 {
-    const int J = 2 * c_out;
-    const int total = w_k * J * c_in;
-    float* dst = wdx + (size_t)blockIdx.y * g_stride;
-    const int v = g0 + blockIdx.y;
-    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
-        const int ci = e % c_in, r = e / c_in;
-        const int chunk = r / kChunk, u = chunk % w_k, j = (chunk / w_k) * kChunk + r % kChunk;
-        const int co = j >= c_out ? j - c_out : j;
-        const float wv = w[(((size_t)co * c_in + ci) * w_k + u) * h_k + v];
-        dst[e] = j < c_out ? fminf(fmaxf(wv, 0.0f), 100.0f) : fminf(fmaxf(wv, -100.0f), 0.0f);
+    const int K = q.G.n_members, c_out = q.c_out;
+    const int g = q.g0 + blockIdx.y;
+    float* wcatg = q.wcat + (size_t)blockIdx.y * q.g_stride;
+    float* wdg = q.wd + (size_t)blockIdx.y * q.g_stride;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < K * c_out; e += gridDim.x * 256) {
+        const int co = e % c_out, k = e / c_out;
+        const Member mb = member_of(q.G, g, k);
+        const float wv = mb.ok ? q.w[(((long long)co * q.G.c_in + mb.ci) * q.G.w_k + mb.u) * q.G.h_k + mb.v] : 0.0f;
+        const float wp = fminf(fmaxf(wv, 0.0f), 100.0f);
+        const float wn = -fminf(fmaxf(wv, -100.0f), 0.0f);
+        wcatg[(long long)k * 2 * c_out + co] = wp;
+        wcatg[(long long)k * 2 * c_out + c_out + co] = wn;
+        if (!q.dx_rows) {
+            wdg[(long long)co * K + k] = wp;
+            wdg[(long long)(c_out + co) * K + k] = -wn;
+        }
+    }
+    if (q.dx_rows) {
+        const int J = 2 * c_out, c_in = q.G.c_in, w_k = q.G.w_k, h_k = q.G.h_k;
+        for (int e = blockIdx.x * 256 + threadIdx.x; e < w_k * J * c_in; e += gridDim.x * 256) {
+            const int ci = e % c_in, r = e / c_in;
+            const int chunk = r / kChunk, u = chunk % w_k, j = (chunk / w_k) * kChunk + r % kChunk;
+            const int co = j >= c_out ? j - c_out : j;
+            const float wv = q.w[(((size_t)co * c_in + ci) * w_k + u) * h_k + g];
+            wdg[e] = j < c_out ? fminf(fmaxf(wv, 0.0f), 100.0f) : fminf(fmaxf(wv, -100.0f), 0.0f);
+        }
+    }
+    if (blockIdx.y == 0) {
+        if (q.view_rows)
+            for (int e = blockIdx.x * 256 + threadIdx.x; e < q.view_groups * q.view_k_pad; e += gridDim.x * 256) {
+                const int gi = e / q.view_k_pad, k = e - gi * q.view_k_pad;
+                const Member mb = member_of(q.G, gi, k < K ? k : K - 1);
+                q.view_rows[e] = ((long long)mb.v * q.G.c_in + mb.ci) * q.plane + (long long)mb.u * q.ho;
+            }
+        if (q.zero && blockIdx.x == 0 && threadIdx.x < 64) q.zero[threadIdx.x] = 0.0f;
     }
 }
 
@@ -2634,8 +2662,6 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
         const long long quads = (long long)g.h_k * g.c_in * plane / 4;
         hipLaunchKernelGGL(k_shift_planes, dim3(grid1d(quads)), dim3(256), 0, s, x, col, quads, g.n, g.c_in, g.w_in, g.h_in,
                            g.pad_w, g.pad_h, g.ho);
-        hipLaunchKernelGGL(k_view_rows, dim3(grid1d((long long)G.n_groups * L.view_k_pad)), dim3(256), 0, s, view_rows, 0,
-                           G.n_groups, G, plane, g.ho, L.view_k_pad);
     }
     for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
         const int nv = G.n_groups - v0 < L.rows_per_chunk ? G.n_groups - v0 : L.rows_per_chunk;
@@ -2651,10 +2677,22 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
                                dim3(m_blocks > 1024 ? 1024 : m_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
                                dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, G, g.w_in, g.h_in, L.col_v);
         }
+        const bool dx_rows = gx && L.dx_rows && ((uintptr_t)gx & 15) == 0;
         {
-            int wb = grid1d((long long)K * g.c_out);
-            hipLaunchKernelGGL(k_weight_operands, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wcat, wd, v0,
-                               g.c_out, G, L.w_v);
+            // weight operands of the round's groups; with the first round the view's row table and the block of zeros
+            PrepParams pp = {};
+            pp.w = w; pp.wcat = wcat; pp.wd = wd; pp.g0 = v0; pp.c_out = g.c_out; pp.G = G; pp.g_stride = L.w_v;
+            pp.dx_rows = dx_rows ? 1 : 0;
+            if (v0 == 0 && view) {
+                pp.view_rows = view_rows; pp.view_groups = G.n_groups; pp.view_k_pad = L.view_k_pad; pp.ho = g.ho;
+                pp.plane = (long long)g.n * (g.w_in + 2 * g.pad_w) * g.ho;
+            }
+            if (dx_rows) pp.zero = (float*)(ws + L.off_zero);
+            long long work = (long long)K * g.c_out;
+            if (dx_rows && (long long)g.w_k * J * g.c_in > work) work = (long long)g.w_k * J * g.c_in;
+            if (pp.view_rows && (long long)G.n_groups * L.view_k_pad > work) work = (long long)G.n_groups * L.view_k_pad;
+            const int wb = grid1d(work);
+            hipLaunchKernelGGL(k_bwd_prep, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, pp);
         }
         // E[v][m][j] = g * exp(-(col_v^T . wcat_v)), col stored [K][M]
         GemmParams q1 = {};
@@ -2685,16 +2723,13 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
                                L.splits, g.c_out, G, L.part_v);
         }
         if (!gx) continue;
-        if (L.dx_rows && ((uintptr_t)gx & 15) == 0) {
+        if (dx_rows) {
             // d[v][ci][(n, p, b)] = sum_(u, j) wd_v[j][(ci, u)] * E_v[(n, p + pad - u, b)][j]: the kernel rows
             // summed inside the GEMM (three times the k of the product per (ci, u), a third of its rows and of
-            // its output), then the kernel columns by k_shift_sum_v4
+            // its output), then the kernel columns by k_shift_sum_v4; the operand wdx and the block of zeros
+            // come from k_bwd_prep
             float* zero = (float*)(ws + L.off_zero);
-            hipLaunchKernelGGL(k_zero_block, dim3(1), dim3(64), 0, s, zero);
             const int k3 = g.w_k * J;
-            int wb = grid1d((long long)k3 * g.c_in);
-            hipLaunchKernelGGL(k_weight_dx_operand, dim3(wb > 256 ? 256 : wb, nv), dim3(256), 0, s, w, wd, v0, g.c_out,
-                               g.c_in, g.w_k, g.h_k, L.w_v);
             const long long m2 = (long long)g.n * g.w_in * g.ho;
             GemmParams q3 = {};
             q3.a = wd; q3.b = e; q3.c = dcol;

@@ -1385,8 +1385,8 @@ double conv_forward_cost(const Geometry& g)
 int launch_rail_pack(const Geometry& g, uint32_t* wgt, hipStream_t s, bool from_generator)
 {
     if (!g.wgt_rail) return GEO_SC_OK;
+    if (from_generator && generator_packs_rails(g)) return GEO_SC_OK;  // written, flag area included, by the generator
     hipLaunchKernelGGL(k_zero_i32, dim3(1), dim3(256), 0, s, reinterpret_cast<int32_t*>(wgt + g.wgt_flag_off), (size_t)64);
-    if (from_generator && weight_rows_generator(g)) return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     const size_t lines = g.wgt_rail_lines;
     size_t blocks = (lines * g.n_cotile + 255) / 256;
     hipLaunchKernelGGL(k_rail_pack, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, wgt,

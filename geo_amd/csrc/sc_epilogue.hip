@@ -116,8 +116,8 @@ __global__ __launch_bounds__(256) void k_layer_epilogue_pool_vec(EpiParams q, un
 //     d[n,c,i,j]  = grad_out[n,c,i/2,j/2] * [0 < pooled value < 1] / 4 * [value before relu > 0]
 //     dbeta[c]    = sum d,   dgamma[c] = sum d * xhat,   xhat = (y - mean[c]) * invstd[c]
 //     dy          = gamma[c] * invstd[c] * (d - dbeta[c] / M - xhat * dgamma[c] / M),  M = n*w*h
-// Three kernels: per-channel partial sums (fixed-order tree per block), their sum in split order
-// (deterministic), and the element-wise application.
+// Two kernels: per-channel partial sums (fixed-order tree per block), then the element-wise application, whose
+// blocks first add the few partial sums of every channel in split order (deterministic).
 struct TailParams {
     const int32_t* __restrict__ counts;
     const float* __restrict__ gout;
@@ -255,10 +255,29 @@ __global__ __launch_bounds__(256) void k_tail_bwd_partial_pool(TailParams q, flo
     }
 }
 
-__global__ __launch_bounds__(256) void k_tail_bwd_apply_pool(TailParams q, const float* __restrict__ sums,
+// sums[c][2] (dbeta, dgamma) in LDS from partial[c][splits][2]: every block adds the splits of every channel in
+// split order, so all blocks hold the same bits whatever the scheduling
+__device__ __forceinline__ void tail_sums_to_lds(float* __restrict__ sums, const float* __restrict__ partial, int c,
+                                                 int splits)
+{
+    for (int ch = threadIdx.x; ch < c; ch += 256) {
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int s = 0; s < splits; s++) {
+            s1 += partial[((size_t)ch * splits + s) * 2];
+            s2 += partial[((size_t)ch * splits + s) * 2 + 1];
+        }
+        sums[2 * ch] = s1;
+        sums[2 * ch + 1] = s2;
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void k_tail_bwd_apply_pool(TailParams q, const float* __restrict__ partial,
                                                              float* __restrict__ grad_y, float* __restrict__ grad_gamma,
                                                              float* __restrict__ grad_beta)
 {
+    extern __shared__ float sums[];
+    tail_sums_to_lds(sums, partial, q.c, q.splits);
     const int windows = q.wo * q.ho;
     const long long total = (long long)q.n * q.c * windows;
     const float inv_m = 1.0f / (float)((long long)q.n * q.w * q.h);
@@ -284,30 +303,12 @@ __global__ __launch_bounds__(256) void k_tail_bwd_apply_pool(TailParams q, const
         }
 }
 
-// one wave per channel; the order of the additions is fixed (lane, then the xor tree): deterministic
-__global__ __launch_bounds__(64) void k_tail_bwd_finalize(const float* __restrict__ partial, int c, int splits,
-                                                          float* __restrict__ sums /* [c][2]: dbeta, dgamma */)
-{
-    const int ch = blockIdx.x;
-    float s1 = 0.0f, s2 = 0.0f;
-    for (int s = threadIdx.x; s < splits; s += 64) {
-        s1 += partial[((size_t)ch * splits + s) * 2];
-        s2 += partial[((size_t)ch * splits + s) * 2 + 1];
-    }
-    for (int step = 32; step >= 1; step >>= 1) {
-        s1 += __shfl_xor(s1, step);
-        s2 += __shfl_xor(s2, step);
-    }
-    if (threadIdx.x == 0) {
-        sums[2 * ch] = s1;
-        sums[2 * ch + 1] = s2;
-    }
-}
-
-__global__ __launch_bounds__(256) void k_tail_bwd_apply(TailParams q, const float* __restrict__ sums,
+__global__ __launch_bounds__(256) void k_tail_bwd_apply(TailParams q, const float* __restrict__ partial,
                                                         float* __restrict__ grad_y, float* __restrict__ grad_gamma,
                                                         float* __restrict__ grad_beta)
 {
+    extern __shared__ float sums[];
+    tail_sums_to_lds(sums, partial, q.c, q.splits);
     const int plane = q.w * q.h;
     const long long total = (long long)q.n * q.c * plane;
     const float inv_m = 1.0f / (float)((long long)q.n * plane);
@@ -338,16 +339,38 @@ __global__ __launch_bounds__(256) void k_tail_bwd_apply(TailParams q, const floa
 // in PyTorch's operation order, one rounding per operation.  Also the running statistics of
 // F.batch_norm(training=True) (momentum 0.1, unbiased variance) and 1 / sqrt(var + eps_grad) for the
 // backward.  The channel mean is accumulated in double precision.
-__global__ __launch_bounds__(256) void k_bn_fixed_affine(const float* __restrict__ mean, const float* __restrict__ var,
+__global__ __launch_bounds__(256) void k_bn_fixed_affine(const float* mean, const float* var,
                                                          const float* __restrict__ gamma, const float* __restrict__ beta,
                                                          int c, float eps, float eps_grad, float unbias,
                                                          float* __restrict__ running_mean,
                                                          float* __restrict__ running_var, float* __restrict__ w_n,
                                                          float* __restrict__ b_n, float* __restrict__ invstd,
-                                                         float* __restrict__ scale_out)
+                                                         float* __restrict__ scale_out,
+                                                         const unsigned long long* __restrict__ partial, int splits,
+                                                         double inv_elements_len, double inv_elements_len2,
+                                                         float* __restrict__ mean_out, float* __restrict__ var_out)
 {
     __shared__ double red[256];
     __shared__ float scale_s;
+    if (partial) {
+        // the statistics themselves, from the exact integer sums of k_count_stats_partial (as
+        // k_count_stats_finalize forms them); mean / var then point at mean_out / var_out
+        for (int ch = threadIdx.x; ch < c; ch += 256) {
+            long long s1 = 0, s2 = 0;
+            for (int s = 0; s < splits; s++) {
+                s1 += (long long)partial[((size_t)ch * splits + s) * 2];
+                s2 += (long long)partial[((size_t)ch * splits + s) * 2 + 1];
+            }
+            const double m = (double)s1 * inv_elements_len;
+            const double v = (double)s2 * inv_elements_len2 - m * m;
+            mean_out[ch] = (float)m;
+            var_out[ch] = (float)(v > 0.0 ? v : 0.0);
+        }
+        __threadfence_block();
+        __syncthreads();
+        mean = mean_out;
+        var = var_out;
+    }
     double part = 0.0;
     for (int ch = threadIdx.x; ch < c; ch += 256) {
         const float inv = __fsqrt_rn(__fadd_rn(var[ch], eps));
@@ -470,15 +493,19 @@ __global__ __launch_bounds__(256) void k_quantize(const float* __restrict__ src,
     }
 }
 
+constexpr int kTailMaxChannels = 4096;
+
 int tail_splits(int n, int c, int w, int h)
 {
     // enough blocks to fill the GPU, not more than the channel has 256-element chunks
     const long long per_channel = (long long)n * w * h;
+    // few enough that the kernel after the partial sums adds them itself (no launch in between)
     long long s = (4096 + c - 1) / c;
     const long long chunks = (per_channel + 255) / 256;
     if (s > chunks) s = chunks;
     if (s < 1) s = 1;
-    if (s > 1024) s = 1024;
+    if (s > 16 && (long long)c * 16 >= 512) s = 16;
+    if (s > 32) s = 32;
     return (int)s;
 }
 
@@ -536,7 +563,7 @@ extern "C" int geo_sc_layer_epilogue(const int32_t* counts, int n, int c, int w,
 extern "C" int geo_sc_layer_tail_backward_workspace_size(int n, int c, int w, int h, size_t* bytes)
 {
     if (!bytes || n < 1 || c < 1 || w < 1 || h < 1) return GEO_SC_ERR_INVALID_ARGUMENT;
-    *bytes = sizeof(float) * 2 * ((size_t)c * tail_splits(n, c, w, h) + (size_t)c);
+    *bytes = sizeof(float) * 2 * (size_t)c * tail_splits(n, c, w, h);
     return GEO_SC_OK;
 }
 
@@ -547,7 +574,8 @@ extern "C" int geo_sc_layer_tail_backward(const int32_t* counts, const float* gr
                                           size_t workspace_bytes, geo_sc_stream_t stream)
 {
     if (!counts || !grad_out || !w_n || !b_n || !mean || !invstd || !grad_y) return GEO_SC_ERR_INVALID_ARGUMENT;
-    if (n < 1 || c < 1 || w < 1 || h < 1 || c > 65535) return GEO_SC_ERR_INVALID_ARGUMENT;
+    // the application kernel keeps two sums per channel in LDS
+    if (n < 1 || c < 1 || w < 1 || h < 1 || c > kTailMaxChannels) return GEO_SC_ERR_INVALID_ARGUMENT;
     if (flags & ~(GEO_SC_EPI_RELU | GEO_SC_EPI_POOL2 | GEO_SC_EPI_HARDTANH01 | GEO_SC_EPI_QUANT7))
         return GEO_SC_ERR_INVALID_ARGUMENT;
     switch (bit_length) {
@@ -577,7 +605,6 @@ extern "C" int geo_sc_layer_tail_backward(const int32_t* counts, const float* gr
     q.splits = tail_splits(n, c, w, h);
     hipStream_t s = (hipStream_t)stream;
     float* partial = (float*)workspace;
-    float* sums = partial + (size_t)2 * c * q.splits;
     // one pool window per thread where the plane is made of whole windows and rows of counts, of the incoming
     // gradient's source and of the result start on 8-byte boundaries
     const bool windows = (flags & GEO_SC_EPI_POOL2) && w % 2 == 0 && h % 2 == 0 && ((uintptr_t)counts & 7u) == 0 &&
@@ -586,15 +613,15 @@ extern "C" int geo_sc_layer_tail_backward(const int32_t* counts, const float* gr
         hipLaunchKernelGGL(k_tail_bwd_partial_pool, dim3(q.splits, c), dim3(256), 0, s, q, partial);
     else
         hipLaunchKernelGGL(k_tail_bwd_partial, dim3(q.splits, c), dim3(256), 0, s, q, partial);
-    hipLaunchKernelGGL(k_tail_bwd_finalize, dim3(c), dim3(64), 0, s, partial, c, q.splits, sums);
     const long long total = (long long)n * c * w * h / (windows ? 4 : 1);
     long long blocks = (total + 255) / 256;
-    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (blocks > 256 * 8) blocks = 256 * 8;   // every block first adds the partial sums of all channels
+    const size_t lds = sizeof(float) * 2 * (size_t)c;
     if (windows)
-        hipLaunchKernelGGL(k_tail_bwd_apply_pool, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma,
-                           grad_beta);
+        hipLaunchKernelGGL(k_tail_bwd_apply_pool, dim3((unsigned)blocks), dim3(256), lds, s, q, partial, grad_y,
+                           grad_gamma, grad_beta);
     else
-        hipLaunchKernelGGL(k_tail_bwd_apply, dim3((unsigned)blocks), dim3(256), 0, s, q, sums, grad_y, grad_gamma,
+        hipLaunchKernelGGL(k_tail_bwd_apply, dim3((unsigned)blocks), dim3(256), lds, s, q, partial, grad_y, grad_gamma,
                            grad_beta);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
@@ -646,7 +673,42 @@ extern "C" int geo_sc_bn_fixed_affine(const float* mean, const float* var, const
                              ? (float)((double)elements_per_channel / (double)(elements_per_channel - 1))
                              : 1.0f;
     hipLaunchKernelGGL(k_bn_fixed_affine, dim3(1), dim3(256), 0, (hipStream_t)stream, mean, var, gamma, beta, c, eps,
-                       eps_grad, unbias, running_mean, running_var, w_n, b_n, invstd, scale);
+                       eps_grad, unbias, running_mean, running_var, w_n, b_n, invstd, scale,
+                       (const unsigned long long*)nullptr, 0, 0.0, 0.0, (float*)nullptr, (float*)nullptr);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_bn_fixed_from_counts(const int32_t* counts, int n, int c, int w, int h, int bit_length,
+                                           const float* gamma, const float* beta, float eps, float eps_grad,
+                                           float* running_mean, float* running_var, float* mean, float* var,
+                                           float* w_n, float* b_n, float* invstd, float* scale, void* workspace,
+                                           size_t workspace_bytes, geo_sc_stream_t stream)
+{
+    if (!counts || !mean || !var || !w_n || !b_n) return GEO_SC_ERR_INVALID_ARGUMENT;
+    if (n < 1 || c < 1 || w < 1 || h < 1 || c > 65535) return GEO_SC_ERR_INVALID_ARGUMENT;
+    switch (bit_length) {
+    case 8: case 16: case 32: case 64: case 128: case 256: break;
+    default: return GEO_SC_ERR_BIT_LENGTH;
+    }
+    size_t need = 0;
+    geo_sc_count_stats_workspace_size(n, c, w, h, &need);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 7u)) return GEO_SC_ERR_WORKSPACE;
+    const int plane = w * h;
+    const bool vec_plane = plane % 4 == 0 && ((uintptr_t)counts & 15u) == 0;
+    const int splits = tail_splits(n, c, w, h);
+    hipStream_t s = (hipStream_t)stream;
+    unsigned long long* partial = (unsigned long long*)workspace;
+    if (vec_plane)
+        hipLaunchKernelGGL(k_count_stats_partial<true>, dim3(splits, c), dim3(256), 0, s, counts, n, c, plane, splits,
+                           partial);
+    else
+        hipLaunchKernelGGL(k_count_stats_partial<false>, dim3(splits, c), dim3(256), 0, s, counts, n, c, plane, splits,
+                           partial);
+    const double elements = (double)n * plane;
+    const float unbias = elements > 1 ? (float)(elements / (elements - 1)) : 1.0f;
+    hipLaunchKernelGGL(k_bn_fixed_affine, dim3(1), dim3(256), 0, s, (const float*)nullptr, (const float*)nullptr, gamma,
+                       beta, c, eps, eps_grad, unbias, running_mean, running_var, w_n, b_n, invstd, scale, partial, splits,
+                       1.0 / (elements * bit_length), 1.0 / (elements * bit_length * (double)bit_length), mean, var);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

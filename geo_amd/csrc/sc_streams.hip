@@ -214,15 +214,22 @@ __global__ __launch_bounds__(kGenThreads) void k_act_streams(const XT* __restric
 
 // Weight streams, tiled layout [P][h_k][k][cotile][rail][16]; one thread per
 // (h, k, padded c_out), c_out fastest so that a wave writes whole tiles.
+// rail_words / rail_fields: the rail-packed copy in the same pass, [c_out tile][line][channel] with
+// line = (pack, kernel row, member): the non-zero rail's word and the 16-bit M0 field of the channel's rail
+// (see k_rail_pack); the first block also clears the buffer's flag area.  two_rail = 0 leaves the two-rail
+// lines unwritten (a caller whose convolution kernel reads the rail-packed copy only).
 __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __restrict__ w,
                                                                uint32_t* __restrict__ streams,
                                                                GenParams gp, int c_out, int c_in, int w_k, int h_k,
-                                                               int n_cotile)
+                                                               int n_cotile, uint32_t* __restrict__ rail_words,
+                                                               uint16_t* __restrict__ rail_fields, size_t rail_lines,
+                                                               uint32_t* __restrict__ flags, int two_rail)
 {
     extern __shared__ uint32_t lds[];
     load_tables_to_lds(lds, gp.L, gp.wpc);
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
+    if (flags && blockIdx.x == 0 && threadIdx.x < 64) flags[threadIdx.x] = 0u;
     const int k_or = c_in * w_k;
     const int co_pad = n_cotile * kCoTile;
     const size_t total = (size_t)h_k * k_or * co_pad;
@@ -243,10 +250,20 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams(const float* __r
         }
         const int op = (int)posp1[(67 + k) % (gp.L - 1)];  // sc.cpp:345
         const int on = (int)posp1[(37 + k) % (gp.L - 1)];  // sc.cpp:346
-        const size_t base = (((size_t)v * k_or + k) * n_cotile + co / kCoTile) * (2 * kCoTile) + (co % kCoTile);
+        const int cot = co / kCoTile, co_l = co % kCoTile;
+        const size_t base = (((size_t)v * k_or + k) * n_cotile + cot) * (2 * kCoTile) + co_l;
         for (int pk = 0; pk < gp.packs; pk++) {
-            streams[pk * pack_stride + base] = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
-            streams[pk * pack_stride + base + kCoTile] = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+            const uint32_t wp = cp ? stream_word(thr, cp, op, pk, gp) : 0u;
+            const uint32_t wn = cn ? stream_word(thr, cn, on, pk, gp) : 0u;
+            if (two_rail) {
+                streams[pk * pack_stride + base] = wp;
+                streams[pk * pack_stride + base + kCoTile] = wn;
+            }
+            if (rail_words) {
+                const size_t dst = ((size_t)cot * rail_lines + ((size_t)pk * h_k + v) * k_or + k) * kCoTile + co_l;
+                rail_words[dst] = wp | wn;
+                rail_fields[dst] = (uint16_t)(0xC000u | ((cn ? 2u * kCoTile : 0u) + 2u * co_l));
+            }
         }
     }
 }
@@ -265,10 +282,12 @@ __global__ __launch_bounds__(kGenThreads) void k_weight_streams_rows(const float
                                                                     int h_k, int n_cotile,
                                                                     int v_chunks, uint32_t* __restrict__ rail_words,
                                                                     uint16_t* __restrict__ rail_fields,
-                                                                    size_t rail_lines, int two_rail)
+                                                                    size_t rail_lines, uint32_t* __restrict__ flags,
+                                                                    int two_rail)
 {
     extern __shared__ uint32_t lds[];
     load_tables_to_lds(lds, gp.L, gp.wpc);
+    if (flags && blockIdx.x == 0 && threadIdx.x < 64) flags[threadIdx.x] = 0u;
     const uint32_t* posp1 = lds;
     const uint32_t* thr = lds + gp.L;
     float* wt = reinterpret_cast<float*>(lds + gp.L + gp.L * gp.wpc);  // [row][member][channel], rows of 17
@@ -664,12 +683,15 @@ int launch_weight_streams(const Geometry& g, const float* w, uint32_t* streams, 
                            g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile, v_chunks,
                            g.wgt_rail ? streams + g.wgt_rail_off : nullptr,
                            g.wgt_rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
-                           g.wgt_rail_lines, two_rail ? 1 : 0);
+                           g.wgt_rail_lines, g.wgt_rail ? streams + g.wgt_flag_off : nullptr, two_rail ? 1 : 0);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
     const size_t total = (size_t)g.h_k * g.k_or * g.n_cotile * kCoTile;
+    const bool two_rail = !(rail_only && g.wgt_rail);
     hipLaunchKernelGGL(k_weight_streams, dim3(grid_for(total)), dim3(kGenThreads), table_bytes(g.L), s, w, streams,
-                       gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile);
+                       gp, g.c_out, g.c_in, g.w_k, g.h_k, g.n_cotile, g.wgt_rail ? streams + g.wgt_rail_off : nullptr,
+                       g.wgt_rail ? reinterpret_cast<uint16_t*>(streams + g.wgt_rail_idx_off) : nullptr,
+                       g.wgt_rail_lines, g.wgt_rail ? streams + g.wgt_flag_off : nullptr, two_rail ? 1 : 0);
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 

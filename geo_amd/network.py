@@ -267,9 +267,8 @@ def apply_update(model, optimizer, param_copy):
     """The part of the reference's step that follows ``loss.backward()`` (utils_own.py:98-114): restore
     the full-precision weights, hand the gradients to the master copies and un-scale them, optimiser
     step on the copies, copy back, refresh ``weight_org`` clamped to [-1, 0.999]."""
-    for m in model.modules():
-        if hasattr(m, "weight_org"):
-            m.weight.data.copy_(m.weight_org)
+    # (the reference first copies weight_org back into weight.data; the copy-back from the master copies below
+    # overwrites every parameter before anything reads it, so that copy changes nothing and is not launched)
     params = list(model.parameters())
     # the per-parameter loops of the reference as multi-tensor calls: one kernel for all gradients,
     # one for all copies
@@ -284,7 +283,7 @@ def apply_update(model, optimizer, param_copy):
     torch._foreach_copy_([p.data for p in params], [master.data for master in param_copy])
     for m in model.modules():
         if hasattr(m, "weight_org"):
-            m.weight_org.copy_(m.weight.data.clamp(-1, 0.999))
+            torch.clamp(m.weight.data, -1, 0.999, out=m.weight_org)
     optimizer.zero_grad()
 
 
@@ -298,3 +297,62 @@ def train_step(model, inputs, target, criterion, optimizer, param_copy):
     loss.backward()
     apply_update(model, optimizer, param_copy)
     return loss.detach() / SCALE_FACTOR
+
+
+class GraphedTrainStep:
+    """``train_step`` for a fixed batch shape, recorded once into a HIP graph and replayed: the step's ~130
+    short launches then cost the host one submission instead of one each (at batch 256 the eager step of the
+    4-layer CNN is bound by the host's launch rate, not by the GPU).  Same kernels, same arithmetic, same state:
+    weights, master copies, optimiser moments and running statistics live where they did and are updated in
+    place by the replayed kernels.
+
+    The optimiser must keep its step count on the device (``torch.optim.Adam(..., capturable=True)``).  Recording
+    needs the allocator and the kernels warmed up by real steps; the state they change is put back afterwards
+    (model buffers and parameters, master copies, optimiser state), so constructing this object leaves the
+    training state as it found it.  The model must be in training mode and stay as it is (same settings, same
+    ``fused_blocks``) for as long as the graph is replayed."""
+
+    def __init__(self, model, criterion, optimizer, param_copy, inputs, target, warmup=3):
+        import copy
+        self.model, self.optimizer, self.param_copy = model, optimizer, param_copy
+        self.inputs, self.target = inputs.detach().clone(), target.detach().clone()
+        model_state = {k: v.detach().clone() for k, v in model.state_dict().items()}
+        masters = [m.detach().clone() for m in param_copy]
+        had_state = {id(p) for p in optimizer.state}
+        opt_state = copy.deepcopy({id(p): {k: v for k, v in st.items()} for p, st in optimizer.state.items()})
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(max(1, int(warmup))):
+                train_step(model, self.inputs.clone(), self.target, criterion, optimizer, param_copy)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            # a second handle on the static batch: the layer re-points its input's .data at the quantised values,
+            # which must not re-point self.inputs away from the memory the recorded kernels read
+            self.loss = train_step(model, self.inputs.detach(), self.target, criterion, optimizer, param_copy)
+        # put the training state back, in place: the graph holds the addresses
+        with torch.no_grad():
+            now = model.state_dict()
+            for k, v in model_state.items():
+                now[k].copy_(v)
+            for m, saved in zip(param_copy, masters):
+                m.copy_(saved)
+            for p, st in optimizer.state.items():
+                for k, v in st.items():
+                    if not torch.is_tensor(v):
+                        continue
+                    if id(p) in had_state:
+                        v.copy_(opt_state[id(p)][k])
+                    else:
+                        v.zero_()   # a fresh state is all zeros (step count, moments)
+        torch.cuda.synchronize()
+
+    def __call__(self, inputs, target):
+        """One step on a batch of the recorded shape; returns the (unscaled) loss tensor of that step, which the
+        next call overwrites."""
+        self.inputs.copy_(inputs)
+        self.target.copy_(target)
+        self.graph.replay()
+        return self.loss

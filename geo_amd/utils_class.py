@@ -97,21 +97,23 @@ class _SCConvBlock(torch.autograd.Function):
         conv_kw = {k: v for k, v in conv_kw.items() if k != "torch_stats"}
         L = conv_kw["bit_length"]
         counts = capi.conv2d_add_partial_forward(x, w, **conv_kw)
-        if torch_stats:
-            # the two PyTorch reductions BatchNorm*_fixed itself runs (utils_class.py:52-56)
-            y = counts * (1.0 / L)   # exact: L is a power of two
-            mean, var = y.mean(dim=(0, 2, 3)), y.var(dim=(0, 2, 3), unbiased=False)
-        else:
-            # the same statistics from exact integer sums: no y in memory, no dependence on a reduction order
-            mean, var = capi.count_stats(counts, L)
+        gm = gamma.detach().float().contiguous() if gamma is not None else None
+        bt = beta.detach().float().contiguous() if beta is not None else None
         # One launch for what BatchNorm*_fixed computes per channel (utils_class.py:52-62) and for what
         # its F.batch_norm(x, running_mean, running_var, weight, bias, training=True) call
         # (utils_class.py:49) does to the running statistics: that function's default momentum 0.1
         # and, for the gradient, its default eps 1e-5; the batch counter is not touched.
-        w_n, b_n, invstd, bn.scale = capi.bn_fixed_affine(
-            mean, var, gamma.detach().float().contiguous() if gamma is not None else None,
-            beta.detach().float().contiguous() if beta is not None else None, bn.eps, counts.numel() // counts.shape[1],
-            bn.running_mean, bn.running_var)
+        if torch_stats:
+            # the two PyTorch reductions BatchNorm*_fixed itself runs (utils_class.py:52-56)
+            y = counts * (1.0 / L)   # exact: L is a power of two
+            mean, var = y.mean(dim=(0, 2, 3)), y.var(dim=(0, 2, 3), unbiased=False)
+            w_n, b_n, invstd, bn.scale = capi.bn_fixed_affine(mean, var, gm, bt, bn.eps,
+                                                              counts.numel() // counts.shape[1], bn.running_mean,
+                                                              bn.running_var)
+        else:
+            # the same statistics from exact integer sums: no y in memory, no dependence on a reduction order
+            mean, var, w_n, b_n, invstd, bn.scale = capi.bn_fixed_from_counts(counts, L, gm, bt, bn.eps,
+                                                                              bn.running_mean, bn.running_var)
         act, _ = capi.layer_epilogue(counts, L, w_n, b_n, relu=relu, pool=pool, hardtanh=hardtanh, quant7=quant7)
         ctx.save_for_backward(x, w, counts, w_n, b_n, mean, invstd,
                               gamma.detach() if gamma is not None else torch.empty(0, device=x.device))
@@ -151,7 +153,9 @@ def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_un
         raise NotImplementedError("sc_conv_block: LFSR modes 1d_bin / z_bin / yz_bin on GPU tensors")
     if tuple(conv.stride) != (1, 1):
         raise NotImplementedError("the SC kernels compute stride 1 only")
-    input.data = utils_functional.quantize(input.data, prec=prec)
+    # an input that is the untouched 7-bit output of a fused block already holds quantize(input, 7)
+    if not (prec == 7 and getattr(input, "_geo_q7_version", None) == input._version):
+        input.data = utils_functional.quantize(input.data, prec=prec)
     conv.weight.data = utils_functional.quantize(conv.weight_org, prec=prec)
     mode = {"1d_bin": "y", "z_bin": "z", "yz_bin": "yz"}[forward]
     kw = dict(bit_length=2 ** err, padding=(int(conv.padding[0]), int(conv.padding[1])),
@@ -159,4 +163,7 @@ def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_un
               load_wait_a=int(load_wait_a if mode == "yz" else load_wait_w), accumulate=mode,
               z_unit=max(1, min(int(z_unit), conv.weight.shape[1])), torch_stats=bool(torch_stats))
     gamma, beta = (bn.weight, bn.bias) if bn.affine else (None, None)
-    return _SCConvBlock.apply(input, conv.weight, gamma, beta, bn, kw, relu, pool, hardtanh, quant7)
+    out = _SCConvBlock.apply(input, conv.weight, gamma, beta, bn, kw, relu, pool, hardtanh, quant7)
+    if quant7 and hardtanh:
+        out._geo_q7_version = out._version   # values k / 128, 0 <= k <= 127, until somebody writes to the tensor
+    return out

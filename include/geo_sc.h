@@ -318,7 +318,8 @@ GEO_SC_API int geo_sc_layer_epilogue(const int32_t* counts, int n, int c, int w,
  *   gamma                     the batch norm's weight, or NULL for 1
  *   grad_y                    fp32 (n, c, w, h): gradient with respect to y = count / L
  *   grad_gamma, grad_beta     per channel, may be NULL
- * Deterministic (fixed summation order).  Workspace: geo_sc_layer_tail_backward_workspace_size.
+ * Deterministic (fixed summation order).  Workspace: geo_sc_layer_tail_backward_workspace_size.  At most 4096
+ * channels.
  */
 GEO_SC_API int geo_sc_layer_tail_backward_workspace_size(int n, int c, int w, int h, size_t* bytes);
 GEO_SC_API int geo_sc_layer_tail_backward(const int32_t* counts, const float* grad_out, int n, int c, int w, int h,
@@ -353,6 +354,19 @@ GEO_SC_API int geo_sc_bn_fixed_affine(const float* mean, const float* var, const
                                       int c, float eps, float eps_grad, long long elements_per_channel,
                                       float* running_mean, float* running_var, float* w_n, float* b_n, float* invstd,
                                       float* scale, geo_sc_stream_t stream);
+
+/*
+ * geo_sc_count_stats and geo_sc_bn_fixed_affine in two launches instead of three: the channel statistics of
+ * y = counts / bit_length from exact integer sums (written to mean, var: c floats each), then the fixed-point
+ * affine, 1 / sqrt(var + eps_grad) and the running statistics from them (utils_class.py:49-62), the number of
+ * elements per channel being n * w * h.  Same values as the two calls.  Workspace:
+ * geo_sc_count_stats_workspace_size bytes, 8-byte aligned.
+ */
+GEO_SC_API int geo_sc_bn_fixed_from_counts(const int32_t* counts, int n, int c, int w, int h, int bit_length,
+                                           const float* gamma, const float* beta, float eps, float eps_grad,
+                                           float* running_mean, float* running_var, float* mean, float* var,
+                                           float* w_n, float* b_n, float* invstd, float* scale, void* workspace,
+                                           size_t workspace_bytes, geo_sc_stream_t stream);
 
 /*
  * quantize (utils_functional.py:33-39) in one pass: dst = clamp(round(src * 2^prec), -(2^prec - 1), 2^prec - 1)

@@ -47,7 +47,7 @@ def test_static_workspace_forward_allocates_nothing_and_cuts_large_batches(capi)
     """Free device memory is the same before and after (the caller's tensors exist beforehand), also for a
     batch whose streams are several times the array: those run in chunks behind the weight streams."""
     assert capi.static_workspace_bytes() == 32 << 20
-    x, w = wl.make_inputs((96, 32, 16, 16), (32, 32, 3, 3), "sparse", seed=5)
+    x, w = wl.make_inputs((512, 32, 16, 16), (32, 32, 3, 3), "sparse", seed=5)
     xd, wd = x.cuda(), w.cuda()
     L, pad = 128, (1, 1)
     d = capi.make_desc(xd.shape, wd.shape, L, pad)
