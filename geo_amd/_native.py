@@ -28,7 +28,7 @@ class ConvDesc(ctypes.Structure):
 class Options(ctypes.Structure):
     """geo_sc_options of include/geo_sc.h"""
     _fields_ = [("struct_bytes", ctypes.c_size_t), ("forward_stream_bytes", ctypes.c_size_t),
-                ("backward_groups_per_round", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("backward_groups_per_round", ctypes.c_int32), ("forward_single_stream", ctypes.c_int32)]
 
 
 # every symbol include/geo_sc.h declares: name -> (restype, argtypes)

@@ -49,11 +49,13 @@ def make_desc(x_shape, w_shape, bit_length, padding=(0, 0), total_width=7, load_
                     ctypes.c_int32(int(seed) & 0xffffffff).value)
 
 
-def make_options(forward_stream_bytes=0, backward_groups_per_round=0) -> Options:
+def make_options(forward_stream_bytes=0, backward_groups_per_round=0, forward_single_stream=False) -> Options:
     """geo_sc_options: the budget (bytes) of the forward's activation stream buffer - a batch whose streams
     exceed it runs in chunks of items - and the cap on the add groups per round of backward launches;
-    0 leaves a field at the library's default."""
-    return Options(ctypes.sizeof(Options), int(forward_stream_bytes), int(backward_groups_per_round), 0)
+    0 leaves a field at the library's default.  forward_single_stream keeps a cut batch on the caller's stream
+    (by default its odd chunks run on a second stream of the library)."""
+    return Options(ctypes.sizeof(Options), int(forward_stream_bytes), int(backward_groups_per_round),
+                   1 if forward_single_stream else 0)
 
 
 def _opt_ptr(options):

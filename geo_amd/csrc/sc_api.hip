@@ -127,9 +127,11 @@ Options make_options(const geo_sc_options* o)
     Options r;
     r.forward_stream_bytes = kDefaultForwardStreamBytes;
     r.backward_groups_per_round = 0;
+    r.forward_single_stream = false;
     if (o && o->struct_bytes >= sizeof(geo_sc_options)) {
         if (o->forward_stream_bytes) r.forward_stream_bytes = o->forward_stream_bytes;
         if (o->backward_groups_per_round > 0) r.backward_groups_per_round = o->backward_groups_per_round;
+        r.forward_single_stream = o->forward_single_stream != 0;
     }
     return r;
 }
@@ -139,11 +141,15 @@ Options make_options(const geo_sc_options* o)
 // scratch does not grow with the batch (the reference keeps streams for 128 blocks whatever the batch,
 // sc_cuda_kernel.cu:658-662, :1787-1789).  Every item is independent (same seeds for every item,
 // sc.cpp:409-413), so the counts do not depend on the cut.
+// A cut batch uses the budget as two buffers, chunks alternating between them: a chunk's generator then runs
+// while the chunk before it is still being convolved (on a second stream where the library may use one), and
+// the draining tail of one convolution launch overlaps the head of the next.
 struct ForwardPlan {
     Geometry chunk, last;  // geometry of a full chunk and of the shorter last one (n_last == 0: none)
     int nc, n_full, n_last;
+    int buffers;           // 1: the whole batch at once; 2: chunks
     bool rail_only;        // every launch reads the rail-packed weight lines only
-    size_t off_wgt, off_act, ws_bytes;
+    size_t off_wgt, off_act[2], ws_bytes;
 };
 
 int plan_forward(const geo_sc_conv_desc* d, const Options& opt, ForwardPlan* p)
@@ -158,10 +164,12 @@ int plan_forward(const geo_sc_conv_desc* d, const Options& opt, ForwardPlan* p)
         return make_geometry(&dc, out);
     };
     int nc = g.n;
+    p->buffers = 1;
     if ((size_t)g.n * item_bytes > opt.forward_stream_bytes) {
-        // largest chunk inside the budget (at least one item), then the size between that and half of it whose
-        // launches fill the GPU's rounds of waves best
-        long long nc_max = (long long)(opt.forward_stream_bytes / item_bytes);
+        // two buffers of half the budget; largest chunk inside one (at least one item), then the size between
+        // that and half of it whose launches fill the GPU's rounds of waves best
+        p->buffers = 2;
+        long long nc_max = (long long)(opt.forward_stream_bytes / 2 / item_bytes);
         if (nc_max < 1) nc_max = 1;
         if (nc_max > g.n) nc_max = g.n;
         double best = 0;
@@ -188,8 +196,9 @@ int plan_forward(const geo_sc_conv_desc* d, const Options& opt, ForwardPlan* p)
     if (p->n_last && (rc = geometry_of(p->n_last, &p->last)) != GEO_SC_OK) return rc;
     p->rail_only = p->chunk.rail && p->last.rail;
     p->off_wgt = 0;
-    p->off_act = align256(g.wgt_words * sizeof(uint32_t));
-    p->ws_bytes = p->off_act + align256((size_t)nc * item_bytes);
+    p->off_act[0] = align256(g.wgt_words * sizeof(uint32_t));
+    p->off_act[1] = p->off_act[0] + (p->buffers == 2 ? align256((size_t)nc * item_bytes) : 0);
+    p->ws_bytes = p->off_act[p->buffers - 1] + align256((size_t)nc * item_bytes);
     return GEO_SC_OK;
 }
 
@@ -222,6 +231,39 @@ void* static_workspace()
     return addr[dev];
 }
 
+// The library's second stream on the current device, for the chunked forward: created once per device
+// (geo_sc_init, or the first call that wants it), never inside a stream capture.  mu serialises the calls that
+// enqueue on it (its two events are shared).
+struct SideStream {
+    std::mutex mu;
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    bool tried = false, ok = false;
+};
+SideStream* side_stream(hipStream_t caller)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex table_mu;
+    static SideStream table[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(table_mu);
+    SideStream& ss = table[dev];
+    if (!ss.tried) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(caller, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return nullptr;  // not now: creating a stream is not capturable work
+        }
+        ss.tried = true;
+        ss.ok = hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking) == hipSuccess &&
+                hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) == hipSuccess &&
+                hipEventCreateWithFlags(&ss.join, hipEventDisableTiming) == hipSuccess;
+        if (!ss.ok) (void)hipGetLastError();
+    }
+    return ss.ok ? &ss : nullptr;
+}
+
 // x is fp32, or with Q7 the uint8 integers k of activations k / 128
 template <bool Q7>
 int forward_impl(const geo_sc_conv_desc* desc, const Options& opt, const void* x, const float* w, int32_t* y,
@@ -235,23 +277,38 @@ int forward_impl(const geo_sc_conv_desc* desc, const Options& opt, const void* x
     hipStream_t s = (hipStream_t)stream;
     char* ws = (char*)workspace;
     uint32_t* wgt = (uint32_t*)(ws + p.off_wgt);
-    uint32_t* act = (uint32_t*)(ws + p.off_act);
     // the weight stream buffer is the same for every batch size: generated once, read by every chunk
     if ((rc = launch_weight_streams(p.chunk, w, wgt, s, p.rail_only)) != GEO_SC_OK) return rc;
     if ((rc = launch_rail_pack(p.chunk, wgt, s, true)) != GEO_SC_OK) return rc;
     const size_t x_item = (size_t)desc->c_in * desc->w_in * desc->h_in * (Q7 ? 1 : sizeof(float));
     const size_t y_item = (size_t)desc->c_out * p.chunk.wo * p.chunk.ho;
     const int chunks = p.n_full + (p.n_last ? 1 : 0);
+    // odd chunks on the library's second stream (forked behind the weight streams, joined at the end); a
+    // chunk follows the chunk two before it on its own stream, which is the one that used its buffer
+    SideStream* side = (chunks > 1 && !opt.forward_single_stream) ? side_stream(s) : nullptr;
+    std::unique_lock<std::mutex> side_lock;
+    if (side) {
+        side_lock = std::unique_lock<std::mutex>(side->mu);
+        if (hipEventRecord(side->fork, s) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+            return GEO_SC_ERR_LAUNCH;
+    }
     for (int c = 0; c < chunks; c++) {
         const Geometry& g = c < p.n_full ? p.chunk : p.last;
         const size_t n0 = (size_t)c * p.nc;
         const char* xc = (const char*)x + n0 * x_item;
-        rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)xc, act, s)
-                : launch_act_streams(g, (const float*)xc, act, s, n0);
-        if (rc != GEO_SC_OK) return rc;
-        if ((rc = launch_conv_forward(g, act, wgt, y + n0 * y_item, s)) != GEO_SC_OK) return rc;
+        uint32_t* act = (uint32_t*)(ws + p.off_act[c & (p.buffers - 1)]);
+        hipStream_t sc = (side && (c & 1)) ? side->stream : s;
+        rc = Q7 ? launch_act_streams_q7(g, (const uint8_t*)xc, act, sc)
+                : launch_act_streams(g, (const float*)xc, act, sc, n0);
+        if (rc == GEO_SC_OK) rc = launch_conv_forward(g, act, wgt, y + n0 * y_item, sc);
+        if (rc != GEO_SC_OK) break;
     }
-    return GEO_SC_OK;
+    if (side) {
+        // joined also after a failed launch: the caller's stream must not run ahead of what was enqueued
+        if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(s, side->join, 0) != hipSuccess)
+            return GEO_SC_ERR_LAUNCH;
+    }
+    return rc;
 }
 }  // namespace
 
@@ -274,6 +331,7 @@ const char* geo_sc_status_string(int status)
 
 int geo_sc_init(void)
 {
+    side_stream(nullptr);  // optional: without it a cut batch runs on the caller's stream alone
     return static_workspace() ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }
 
@@ -454,7 +512,8 @@ int geo_sc_conv2d_add_partial_forward_static(const geo_sc_conv_desc* desc, const
     const size_t wgt_bytes = align256(g.wgt_words * sizeof(uint32_t));
     if (wgt_bytes >= GEO_SC_STATIC_WORKSPACE_BYTES) return GEO_SC_ERR_WORKSPACE;
     Options opt = make_options(nullptr);
-    opt.forward_stream_bytes = GEO_SC_STATIC_WORKSPACE_BYTES - wgt_bytes - 256;
+    opt.forward_single_stream = true;   // nothing of the library's beyond the array
+    opt.forward_stream_bytes = GEO_SC_STATIC_WORKSPACE_BYTES - wgt_bytes - 512;
     ForwardPlan p;
     if ((rc = plan_forward(desc, opt, &p)) != GEO_SC_OK) return rc;
     if (p.ws_bytes > GEO_SC_STATIC_WORKSPACE_BYTES) return GEO_SC_ERR_WORKSPACE;

@@ -79,6 +79,7 @@ int make_geometry(const geo_sc_conv_desc* d, Geometry* g);
 struct Options {
     size_t forward_stream_bytes;    // budget of the forward's activation stream buffer
     int backward_groups_per_round;  // cap on the add groups per round of backward launches; 0: none
+    bool forward_single_stream;     // a cut batch runs on the caller's stream alone
 };
 constexpr size_t kDefaultForwardStreamBytes = (size_t)256 << 20;
 

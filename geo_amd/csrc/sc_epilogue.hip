@@ -255,19 +255,29 @@ __global__ __launch_bounds__(256) void k_tail_bwd_partial_pool(TailParams q, flo
     }
 }
 
-// sums[c][2] (dbeta, dgamma) in LDS from partial[c][splits][2]: every block adds the splits of every channel in
-// split order, so all blocks hold the same bits whatever the scheduling
+// sums[c][2] (dbeta, dgamma) in LDS from partial[c][splits][2], splits <= 32: half a wave per channel, one
+// partial sum per lane, then a xor tree over the 32 lanes - the same order of additions in every block, so
+// all blocks hold the same bits whatever the scheduling
 __device__ __forceinline__ void tail_sums_to_lds(float* __restrict__ sums, const float* __restrict__ partial, int c,
                                                  int splits)
 {
-    for (int ch = threadIdx.x; ch < c; ch += 256) {
+    const int sub = threadIdx.x & 31;
+    for (int ch0 = 0; ch0 < c; ch0 += 8) {
+        const int ch = ch0 + (threadIdx.x >> 5);
         float s1 = 0.0f, s2 = 0.0f;
-        for (int s = 0; s < splits; s++) {
-            s1 += partial[((size_t)ch * splits + s) * 2];
-            s2 += partial[((size_t)ch * splits + s) * 2 + 1];
+        if (ch < c && sub < splits) {
+            const float2 p = *(const float2*)(partial + ((size_t)ch * splits + sub) * 2);
+            s1 = p.x;
+            s2 = p.y;
         }
-        sums[2 * ch] = s1;
-        sums[2 * ch + 1] = s2;
+        for (int step = 16; step >= 1; step >>= 1) {
+            s1 += __shfl_xor(s1, step);
+            s2 += __shfl_xor(s2, step);
+        }
+        if (ch < c && sub == 0) {
+            sums[2 * ch] = s1;
+            sums[2 * ch + 1] = s2;
+        }
     }
     __syncthreads();
 }

@@ -117,7 +117,15 @@ typedef struct geo_sc_conv_desc {
  *                              streams once); the counts do not depend on the cut.  At least one item's
  *                              streams are always held.  Default 256 MiB.  The reference likewise keeps
  *                              activation streams for 128 thread blocks whatever the batch
- *                              (sc_cuda_kernel.cu:658-662, :1787-1789).
+ *                              (sc_cuda_kernel.cu:658-662, :1787-1789).  A cut batch uses the budget as two
+ *                              buffers, chunks alternating, so that one chunk's streams are generated while
+ *                              the chunk before it is convolved.
+ *   forward_single_stream      0 (default): the odd chunks of a cut batch are enqueued on a second stream
+ *                              that the library creates once per device, forked from `stream` behind the
+ *                              weight streams and joined into it before the call returns (nothing of it is
+ *                              visible to the caller; the fork and join are events, so the call stays
+ *                              asynchronous and may be recorded into a HIP graph once geo_sc_init has run
+ *                              on the device).  Non-zero: every launch on `stream` itself.
  *   backward_groups_per_round  the backward processes its add groups (kernel rows in mode Y) in rounds of
  *                              launches of as many groups as fit about 3 GB of scratch; this lowers that
  *                              number and the workspace size with it.  Default: no further cap.
@@ -127,15 +135,15 @@ typedef struct geo_sc_options {
     size_t struct_bytes;
     size_t forward_stream_bytes;
     int32_t backward_groups_per_round;
-    int32_t reserved;
+    int32_t forward_single_stream;
 } geo_sc_options;
 
 /* Library version (GEO_SC_VERSION of the build). */
 GEO_SC_API int geo_sc_version(void);
 
 /*
- * Optional.  Looks up, for the current device, what the library keeps per device (the address of the static
- * workspace of geo_sc_conv2d_add_partial_forward_static).  Entry points do this themselves at their first
+ * Optional.  Looks up or creates, for the current device, what the library keeps per device (the address of
+ * the static workspace of geo_sc_conv2d_add_partial_forward_static; the second stream of the chunked forward).  Entry points do this themselves at their first
  * call on a device; a caller that records HIP graphs calls it once per device beforehand, because the
  * lookup is not stream-ordered work and must not happen inside a stream capture.  No counterpart in the
  * reference.

@@ -467,7 +467,7 @@ def test_large_y_mode_launches_skip_the_zero_rail(capi, so, shape_x, shape_w, pa
 ])
 def test_forward_in_chunks_of_the_batch(capi, so, shape_x, shape_w, pad, L, kw):
     """geo_sc_options.forward_stream_bytes below the batch's activation streams: the forward generates and
-    consumes the streams of a few items at a time (3 - 4 chunks here, the last one shorter).  Same counts as the
+    consumes the streams of a few items at a time (2 - 13 chunks here, the last one often shorter).  Same counts as the
     oracle and as the uncut call, bit for bit, whatever the cut."""
     x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_x[0] + L)
     w = (w * 3).clamp(-1, 1).contiguous()
@@ -484,15 +484,21 @@ def test_forward_in_chunks_of_the_batch(capi, so, shape_x, shape_w, pad, L, kw):
     assert np.array_equal(whole.cpu().numpy(), exp)
     item = 4 * ((L + 31) // 32) * shape_x[1] * (shape_x[2] + 2 * pad[1]) * (shape_x[3] + 2 * pad[0])
     seen = set()
-    for items in (1, 3, 4, 6):
-        opt = capi.make_options(forward_stream_bytes=items * item + 5)
+    # (a cut batch uses the budget as two buffers, chunks alternating between them and, unless asked otherwise,
+    # between the caller's stream and a second stream of the library)
+    for items, single in ((2, False), (4, False), (4, True), (8, False), (12, True), (12, False)):
+        opt = capi.make_options(forward_stream_bytes=items * item + 5, forward_single_stream=single)
         nc = capi.forward_chunk(d, opt)
-        assert (items + 1) // 2 <= nc <= items
+        if items >= shape_x[0]:
+            assert nc == shape_x[0]      # inside the budget: not cut
+        else:
+            assert (items // 2 + 1) // 2 <= nc <= items // 2
         seen.add(nc)
-        assert capi.workspace_size(d, opt) < capi.workspace_size(d)
+        if items < shape_x[0]:
+            assert capi.workspace_size(d, opt) < capi.workspace_size(d)
         out = torch.full(capi.output_shape(d), -3, dtype=torch.int32, device="cuda")
         capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d, out=out, options=opt)
-        assert torch.equal(out, whole), (items, nc)
+        assert torch.equal(out, whole), (items, nc, single)
     assert len(seen) >= 3
     # a workspace sized for chunks is refused by the call that would hold the whole batch
     small = torch.empty(capi.workspace_size(d, capi.make_options(forward_stream_bytes=item)), dtype=torch.uint8,
