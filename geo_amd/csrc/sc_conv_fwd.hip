@@ -1338,7 +1338,7 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
             // two channels per trip for 1-wide kernels: with three, the six address pairs push the 32
             // sums out of the 128 registers
             constexpr int CR = WK == 1 ? 2 : 1;
-            if (lds && (plain || waves >= 4096)) {
+            if (lds) {
                 // c_out tiles of one position tile share their activation words through LDS
                 // Four c_out tiles per workgroup.  With eight tiles or more, four position tiles share the
                 // workgroup and its barrier (16 waves, the whole CU in step): the four waves of a c_out tile
