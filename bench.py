@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--fused-only", action="store_true",
                     help="workload C2: time the fused, graph-replayed training step only (no module-chain and eager "
                          "legs): the run that kernel traces of the step are taken from")
+    ap.add_argument("--probe-mfma-forward", action="store_true",
+                    help="instead of a workload: the matrix-core probe (one stream cycle and kernel row of the headline "
+                         "layer's forward as an fp4 GEMM tile per CU) and what it projects for the whole layer")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the other benchmark configurations that the default run times after the headline")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
@@ -425,6 +428,37 @@ def other_configs(args, torch):
     return out
 
 
+def probe_mfma_forward(torch):
+    """The headline layer's forward priced on the matrix cores by measurement: 512 position tiles x 384 (stream
+    cycle, kernel row) slices = 768 slices per CU of a 128 x 256 x 384 fp4 GEMM tile with threshold and count,
+    operands already expanded to one fp4 value per bit.  Times are for that slice count on 256 workgroups."""
+    from geo_amd import capi
+    wgs, slices = 256, 768
+    a, b, _, _ = capi.probe_mfma_operands(2048, 384)   # 54 MB of A tiles (beyond L2), 20 MB of B tiles (inside)
+    out = torch.empty((wgs, capi.PROBE_MFMA_ROWS, capi.PROBE_MFMA_COLS), dtype=torch.int32, device="cuda")
+
+    def ms(mode, sixteenths=16):
+        capi.probe_mfma_slices(mode, a, b, wgs, 8, sixteenths, out)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        capi.probe_mfma_slices(mode, a, b, wgs, slices, sixteenths, out)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1)
+
+    macs = wgs * slices * capi.PROBE_MFMA_ROWS * capi.PROBE_MFMA_COLS * capi.PROBE_MFMA_K
+    t = {"mfma_only_ms": ms(0), "with_lds_fragment_reads_ms": ms(1), "with_threshold_and_count_ms": ms(2)}
+    for f in (16, 12, 8, 4):
+        t[f"with_{72 * f // 16}_kb_of_operands_loaded_per_slice_ms"] = ms(3, f)
+    return {"probe": "SC forward of C3 (128->128 3x3 at 16x16, batch 256, L 128) as fp4 GEMM slices on the matrix cores",
+            "slices_per_cu": slices, "tile": "128 positions x 256 rail-columns x 384 members", "times": t,
+            "fp4_tflops_mfma_only": 2 * macs / (t["mfma_only_ms"] * 1e-3) / 1e12,
+            "fp4_tflops_with_threshold": 2 * macs / (t["with_threshold_and_count_ms"] * 1e-3) / 1e12,
+            "note": "operands arrive expanded to one fp4 value per stream bit; the vector-ALU kernel takes 1.30 ms for "
+                    "the same layer from bit-packed streams"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -437,6 +471,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
+    if args.probe_mfma_forward:
+        print(json.dumps(probe_mfma_forward(torch)))
+        return
     if args.workload == "C2":
         if args.passes == "fwd":
             bench_network_inference(args, torch)

@@ -111,6 +111,8 @@ def probe_lib() -> ctypes.CDLL:
         L = ctypes.CDLL(path)
         L.geo_sc_probe_and_or_rate.restype = ctypes.c_int
         L.geo_sc_probe_and_or_rate.argtypes = [ctypes.c_int, _P, ctypes.c_size_t, ctypes.POINTER(ctypes.c_double), _P]
+        L.geo_sc_probe_mfma_slices.restype = ctypes.c_int
+        L.geo_sc_probe_mfma_slices.argtypes = [ctypes.c_int] * 4 + [_P, ctypes.c_size_t, _P, ctypes.c_size_t, _P, _P]
         _probe = L
     return _probe
 

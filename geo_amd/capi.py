@@ -443,3 +443,35 @@ def probe_and_or_rate(iters=20000, stream=None):
     e1.record()
     torch.cuda.synchronize()
     return ops.value / (e0.elapsed_time(e1) * 1e-3)
+
+
+# tile of the matrix-core probe (csrc/sc_probe.hip): 128 positions x 256 rail-columns, 384 members, operand rows of
+# 384 fp4 values padded to 208 bytes
+PROBE_MFMA_ROWS, PROBE_MFMA_COLS, PROBE_MFMA_K, PROBE_MFMA_ROW_BYTES = 128, 256, 384, 208
+
+
+def probe_mfma_operands(n_a, n_b, seed=0, p_a=1 / 8, p_b=1 / 16):
+    """Random 0 / 1 operand tiles of the probe as fp4 (1.0 = 0x2), uint8 GPU tensors (n, rows, 208)."""
+    g = torch.Generator().manual_seed(seed)
+
+    def tiles(n, rows, p):
+        bits = (torch.rand((n, rows, PROBE_MFMA_K), generator=g) < p).to(torch.uint8)
+        packed = bits[..., 0::2] * 0x2 + bits[..., 1::2] * 0x20
+        out = torch.zeros((n, rows, PROBE_MFMA_ROW_BYTES), dtype=torch.uint8)
+        out[..., :PROBE_MFMA_K // 2] = packed
+        return out.cuda(), bits
+
+    a, a_bits = tiles(n_a, PROBE_MFMA_ROWS, p_a)
+    b, b_bits = tiles(n_b, PROBE_MFMA_COLS, p_b)
+    return a, b, a_bits, b_bits
+
+
+def probe_mfma_slices(mode, a, b, workgroups, slices, reload_sixteenths=16, out=None, stream=None):
+    """geo_sc_probe_mfma_slices: `slices` (cycle, kernel row) slices of the forward as fp4 GEMM tiles per workgroup;
+    returns the int32 counts (workgroups, 128, 256)."""
+    if out is None:
+        out = torch.empty((workgroups, PROBE_MFMA_ROWS, PROBE_MFMA_COLS), dtype=torch.int32, device="cuda")
+    _check(_native.probe_lib().geo_sc_probe_mfma_slices(int(mode), int(reload_sixteenths), int(workgroups), int(slices),
+                                                        _ptr(a), a.shape[0], _ptr(b), b.shape[0], _ptr(out),
+                                                        _stream_ptr(stream)), "geo_sc_probe_mfma_slices")
+    return out
