@@ -450,7 +450,9 @@ def probe_mfma_forward(torch):
     macs = wgs * slices * capi.PROBE_MFMA_ROWS * capi.PROBE_MFMA_COLS * capi.PROBE_MFMA_K
     t = {"mfma_only_ms": ms(0), "with_lds_fragment_reads_ms": ms(1), "with_threshold_and_count_ms": ms(2)}
     for f in (16, 12, 8, 4):
-        t[f"with_{72 * f // 16}_kb_of_operands_loaded_per_slice_ms"] = ms(3, f)
+        t[f"with_{78 * f // 16}_kb_of_operands_loaded_per_slice_ms"] = ms(3, f)
+    for f in (16, 12, 8, 4):
+        t[f"with_{78 * f // 16}_kb_per_slice_loaded_straight_into_lds_ms"] = ms(4, f)
     return {"probe": "SC forward of C3 (128->128 3x3 at 16x16, batch 256, L 128) as fp4 GEMM slices on the matrix cores",
             "slices_per_cu": slices, "tile": "128 positions x 256 rail-columns x 384 members", "times": t,
             "fp4_tflops_mfma_only": 2 * macs / (t["mfma_only_ms"] * 1e-3) / 1e12,

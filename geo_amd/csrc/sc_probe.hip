@@ -53,7 +53,8 @@ __global__ __launch_bounds__(64) void k_probe_and_or(const uint32_t* __restrict_
 //   mode 1: + the operand fragments read from LDS for every slice
 //   mode 2: + threshold (> 0) and count into int32
 //   mode 3: + the next slice's operand tiles (a share of their 72 KB) loaded from memory into the other LDS
-//           buffer while this slice is multiplied, one barrier per slice
+//           buffer while this slice is multiplied (through registers), one barrier per slice
+//   mode 4: the same with loads that write LDS directly (global_load_lds_dwordx4)
 // What it measures is an upper bound on a matrix-core forward: the operands arrive already expanded from one
 // bit to one fp4 value per cycle, which a real kernel would have to do as well.
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -101,7 +102,21 @@ __global__ __launch_bounds__(512) void k_tile(const uint8_t* __restrict__ a_glob
     constexpr int A_LOAD = A_BYTES / 16 * FR / 16, B_LOAD = B_BYTES / 16 * FR / 16;
     constexpr int A_PER = A_LOAD / 512 + 1, B_PER = B_LOAD / 512 + 1;
     for (int it = 0; it < iters; it++) {
-        const int buf = MODE == 3 ? (it & 1) : 0;
+        const int buf = MODE >= 3 ? (it & 1) : 0;
+        if (MODE == 4) {
+            // the next slice's tiles straight into the other LDS buffer: every wave instruction moves 64 x 16
+            // bytes from per-lane addresses to one contiguous kilobyte of LDS, no registers in between
+            const size_t ta = ((size_t)blockIdx.x * 131 + it + 1) % a_tiles, tb = (size_t)(it + 1) % b_tiles;
+            const uint8_t* sa = a_glob + ta * A_BYTES;
+            const uint8_t* sb = b_glob + tb * B_BYTES;
+            constexpr int A_KB = A_BYTES / 1024 * FR / 16, B_KB = B_BYTES / 1024 * FR / 16;
+            for (int kb = wave; kb < A_KB; kb += 8)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sa + kb * 1024 + lane * 16),
+                                                 (__attribute__((address_space(3))) void*)(a_buf(buf ^ 1) + kb * 1024), 16, 0, 0);
+            for (int kb = wave; kb < B_KB; kb += 8)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sb + kb * 1024 + lane * 16),
+                                                 (__attribute__((address_space(3))) void*)(b_buf(buf ^ 1) + kb * 1024), 16, 0, 0);
+        }
         uint4 na[A_PER], nb[B_PER];
         if (MODE == 3) {
             const size_t ta = ((size_t)blockIdx.x * 131 + it + 1) % a_tiles, tb = (size_t)(it + 1) % b_tiles;
@@ -169,6 +184,10 @@ __global__ __launch_bounds__(512) void k_tile(const uint8_t* __restrict__ a_glob
             }
             __syncthreads();
         }
+        if (MODE == 4) {
+            __builtin_amdgcn_s_waitcnt(0);   // everything this wave asked for has arrived
+            __syncthreads();
+        }
     }
     // result layout of the 32x32 MFMA: lane l holds column l % 32, rows 8 * (i / 4) + 4 * (l / 32)... + i % 4
 #pragma unroll
@@ -216,6 +235,10 @@ extern "C" GEO_SC_API int geo_sc_probe_mfma_slices(int mode, int reload_sixteent
     else if (mode == 3 && reload_sixteenths == 12) GEO_SC_PROBE_LAUNCH(3, 12);
     else if (mode == 3 && reload_sixteenths == 8) GEO_SC_PROBE_LAUNCH(3, 8);
     else if (mode == 3 && reload_sixteenths == 4) GEO_SC_PROBE_LAUNCH(3, 4);
+    else if (mode == 4 && reload_sixteenths == 16) GEO_SC_PROBE_LAUNCH(4, 16);
+    else if (mode == 4 && reload_sixteenths == 12) GEO_SC_PROBE_LAUNCH(4, 12);
+    else if (mode == 4 && reload_sixteenths == 8) GEO_SC_PROBE_LAUNCH(4, 8);
+    else if (mode == 4 && reload_sixteenths == 4) GEO_SC_PROBE_LAUNCH(4, 4);
     else return GEO_SC_ERR_INVALID_ARGUMENT;
 #undef GEO_SC_PROBE_LAUNCH
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
