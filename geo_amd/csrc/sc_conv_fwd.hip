@@ -442,69 +442,73 @@ __global__ __launch_bounds__(64) void k_conv_fwd_thin(FwdParams q)
 // instructions in between must not be indexed.
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 
-#define GEO_SC_RAIL_PAIR(W, SET)                                                                                       \
-    SET "v_and_or_b32 v64, %[" W "], %[a0], v64\n"                                                                     \
-        "v_and_or_b32 v65, %[" W "], %[a1], v65\n"
 // M0 of a channel from its 16-bit field: index in bits 7:0, the SRC2 and DST enables in bits 15:12
 #define GEO_SC_RAIL_LO(I) "s_and_b32 m0, %[" I "], 0xffff\n"
 #define GEO_SC_RAIL_HI(I) "s_lshr_b32 m0, %[" I "], 16\n"
+#define GEO_SC_RAIL_OPERANDS                                                                                           \
+    [w0] "s"(w[0]), [w1] "s"(w[1]), [w2] "s"(w[2]), [w3] "s"(w[3]), [w4] "s"(w[4]), [w5] "s"(w[5]), [w6] "s"(w[6]),     \
+        [w7] "s"(w[7]), [w8] "s"(w[8]), [w9] "s"(w[9]), [w10] "s"(w[10]), [w11] "s"(w[11]), [w12] "s"(w[12]),           \
+        [w13] "s"(w[13]), [w14] "s"(w[14]), [w15] "s"(w[15]), [i0] "s"(ix[0]), [i1] "s"(ix[1]), [i2] "s"(ix[2]),        \
+        [i3] "s"(ix[3]), [i4] "s"(ix[4]), [i5] "s"(ix[5]), [i6] "s"(ix[6]), [i7] "s"(ix[7]), [a0] "v"(a0), [a1] "v"(a1)
+// 16 channels x PAIR, the M0 update of every channel but the first in front of its pair
+#define GEO_SC_RAIL_16(PAIR)                                                                                           \
+    PAIR("w0", "") PAIR("w1", GEO_SC_RAIL_HI("i0")) PAIR("w2", GEO_SC_RAIL_LO("i1")) PAIR("w3", GEO_SC_RAIL_HI("i1"))   \
+    PAIR("w4", GEO_SC_RAIL_LO("i2")) PAIR("w5", GEO_SC_RAIL_HI("i2")) PAIR("w6", GEO_SC_RAIL_LO("i3"))                  \
+    PAIR("w7", GEO_SC_RAIL_HI("i3")) PAIR("w8", GEO_SC_RAIL_LO("i4")) PAIR("w9", GEO_SC_RAIL_HI("i4"))                  \
+    PAIR("w10", GEO_SC_RAIL_LO("i5")) PAIR("w11", GEO_SC_RAIL_HI("i5")) PAIR("w12", GEO_SC_RAIL_LO("i6"))               \
+    PAIR("w13", GEO_SC_RAIL_HI("i6")) PAIR("w14", GEO_SC_RAIL_LO("i7")) PAIR("w15", GEO_SC_RAIL_HI("i7"))
 
-// one weight line (16 channels) against the two activation words of the lane's two rows
-__device__ __forceinline__ void rail_line(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1, const uint32_t (&w)[kCoTile],
-                                          const uint32_t (&ix)[kCoTile / 2], uint32_t a0, uint32_t a1)
-{
-    // not volatile: every effect goes through the operands, and a volatile asm would count as a possible
-    // store, after which the compiler no longer reads the weight lines with scalar loads
-    asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n"
-        GEO_SC_RAIL_PAIR("w0", "") GEO_SC_RAIL_PAIR("w1", GEO_SC_RAIL_HI("i0"))
-        GEO_SC_RAIL_PAIR("w2", GEO_SC_RAIL_LO("i1")) GEO_SC_RAIL_PAIR("w3", GEO_SC_RAIL_HI("i1"))
-        GEO_SC_RAIL_PAIR("w4", GEO_SC_RAIL_LO("i2")) GEO_SC_RAIL_PAIR("w5", GEO_SC_RAIL_HI("i2"))
-        GEO_SC_RAIL_PAIR("w6", GEO_SC_RAIL_LO("i3")) GEO_SC_RAIL_PAIR("w7", GEO_SC_RAIL_HI("i3"))
-        GEO_SC_RAIL_PAIR("w8", GEO_SC_RAIL_LO("i4")) GEO_SC_RAIL_PAIR("w9", GEO_SC_RAIL_HI("i4"))
-        GEO_SC_RAIL_PAIR("w10", GEO_SC_RAIL_LO("i5")) GEO_SC_RAIL_PAIR("w11", GEO_SC_RAIL_HI("i5"))
-        GEO_SC_RAIL_PAIR("w12", GEO_SC_RAIL_LO("i6")) GEO_SC_RAIL_PAIR("w13", GEO_SC_RAIL_HI("i6"))
-        GEO_SC_RAIL_PAIR("w14", GEO_SC_RAIL_LO("i7")) GEO_SC_RAIL_PAIR("w15", GEO_SC_RAIL_HI("i7"))
-        "s_set_gpr_idx_off\n"
-        : "+{v[64:79]}"(p0), "+{v[80:95]}"(p1), "+{v[96:111]}"(n0), "+{v[112:127]}"(n1)
-        : [w0] "s"(w[0]), [w1] "s"(w[1]), [w2] "s"(w[2]), [w3] "s"(w[3]), [w4] "s"(w[4]), [w5] "s"(w[5]), [w6] "s"(w[6]),
-          [w7] "s"(w[7]), [w8] "s"(w[8]), [w9] "s"(w[9]), [w10] "s"(w[10]), [w11] "s"(w[11]), [w12] "s"(w[12]),
-          [w13] "s"(w[13]), [w14] "s"(w[14]), [w15] "s"(w[15]), [i0] "s"(ix[0]), [i1] "s"(ix[1]), [i2] "s"(ix[2]),
-          [i3] "s"(ix[3]), [i4] "s"(ix[4]), [i5] "s"(ix[5]), [i6] "s"(ix[6]), [i7] "s"(ix[7]), [a0] "v"(a0), [a1] "v"(a1)
-        : "m0", "scc");
-}
-// The first weight line of an OR group: assigns instead of accumulating, and clears the channel's other
-// rail (index ^ 32), so that the 64 accumulators need no zeroing pass.  v_and_b32 and v_mov_b32 are
-// two-operand instructions, which issue at twice the rate of v_and_or_b32: the line costs what an
-// accumulating line costs.
-#define GEO_SC_RAIL_FIRST(W, SET)                                                                                      \
+// Defines, for accumulators pinned at v[B0 : B0 + 63] (V0 = "vB0", V1 = "v(B0 + 1)" name the first pair):
+//  LINE : one weight line (16 channels) against the two activation words of the lane's two rows;
+//  FIRST: the first weight line of an OR group, which assigns instead of accumulating and clears the channel's
+//         other rail (index ^ 32), so that the 64 accumulators need no zeroing pass.  v_and_b32 and v_mov_b32
+//         are two-operand instructions, which issue at twice the rate of v_and_or_b32: the line costs what an
+//         accumulating line costs.
+// Not volatile: every effect goes through the operands, and a volatile asm would count as a possible store,
+// after which the compiler no longer reads the weight lines with scalar loads.
+#define GEO_SC_DEFINE_RAIL_LINES(LINE, FIRST, V0, V1, RP0, RP1, RN0, RN1)                                              \
+    __device__ __forceinline__ void LINE(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1, const uint32_t (&w)[kCoTile],  \
+                                         const uint32_t (&ix)[kCoTile / 2], uint32_t a0, uint32_t a1)                  \
+    {                                                                                                                  \
+        asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n" GEO_SC_RAIL_16(GEO_SC_RAIL_PAIR_##LINE) "s_set_gpr_idx_off\n" \
+            : "+{" RP0 "}"(p0), "+{" RP1 "}"(p1), "+{" RN0 "}"(n0), "+{" RN1 "}"(n1)                                   \
+            : GEO_SC_RAIL_OPERANDS                                                                                     \
+            : "m0", "scc");                                                                                            \
+    }                                                                                                                  \
+    __device__ __forceinline__ void FIRST(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1, const uint32_t (&w)[kCoTile], \
+                                          const uint32_t (&ix)[kCoTile / 2], uint32_t a0, uint32_t a1)                 \
+    {                                                                                                                  \
+        asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n" GEO_SC_RAIL_16(GEO_SC_RAIL_PAIR_##FIRST) "s_set_gpr_idx_off\n" \
+            : "={" RP0 "}"(p0), "={" RP1 "}"(p1), "={" RN0 "}"(n0), "={" RN1 "}"(n1)                                   \
+            : GEO_SC_RAIL_OPERANDS                                                                                     \
+            : "m0", "scc");                                                                                            \
+    }
+
+// accumulators at v[64:127]: the kernels with four waves per SIMD
+#define GEO_SC_RAIL_PAIR_rail_line(W, SET)                                                                             \
+    SET "v_and_or_b32 v64, %[" W "], %[a0], v64\n"                                                                     \
+        "v_and_or_b32 v65, %[" W "], %[a1], v65\n"
+#define GEO_SC_RAIL_PAIR_rail_line_first(W, SET)                                                                       \
     SET "v_and_b32 v64, %[" W "], %[a0]\n"                                                                            \
         "v_and_b32 v65, %[" W "], %[a1]\n"                                                                            \
         "s_xor_b32 m0, m0, 32\n"                                                                                      \
         "v_mov_b32 v64, 0\n"                                                                                          \
         "v_mov_b32 v65, 0\n"
-__device__ __forceinline__ void rail_line_first(u32x16& p0, u32x16& p1, u32x16& n0, u32x16& n1,
-                                                const uint32_t (&w)[kCoTile], const uint32_t (&ix)[kCoTile / 2],
-                                                uint32_t a0, uint32_t a1)
-{
-    asm("s_set_gpr_idx_on %[i0], gpr_idx(SRC2,DST)\n"
-        GEO_SC_RAIL_FIRST("w0", "") GEO_SC_RAIL_FIRST("w1", GEO_SC_RAIL_HI("i0"))
-        GEO_SC_RAIL_FIRST("w2", GEO_SC_RAIL_LO("i1")) GEO_SC_RAIL_FIRST("w3", GEO_SC_RAIL_HI("i1"))
-        GEO_SC_RAIL_FIRST("w4", GEO_SC_RAIL_LO("i2")) GEO_SC_RAIL_FIRST("w5", GEO_SC_RAIL_HI("i2"))
-        GEO_SC_RAIL_FIRST("w6", GEO_SC_RAIL_LO("i3")) GEO_SC_RAIL_FIRST("w7", GEO_SC_RAIL_HI("i3"))
-        GEO_SC_RAIL_FIRST("w8", GEO_SC_RAIL_LO("i4")) GEO_SC_RAIL_FIRST("w9", GEO_SC_RAIL_HI("i4"))
-        GEO_SC_RAIL_FIRST("w10", GEO_SC_RAIL_LO("i5")) GEO_SC_RAIL_FIRST("w11", GEO_SC_RAIL_HI("i5"))
-        GEO_SC_RAIL_FIRST("w12", GEO_SC_RAIL_LO("i6")) GEO_SC_RAIL_FIRST("w13", GEO_SC_RAIL_HI("i6"))
-        GEO_SC_RAIL_FIRST("w14", GEO_SC_RAIL_LO("i7")) GEO_SC_RAIL_FIRST("w15", GEO_SC_RAIL_HI("i7"))
-        "s_set_gpr_idx_off\n"
-        : "={v[64:79]}"(p0), "={v[80:95]}"(p1), "={v[96:111]}"(n0), "={v[112:127]}"(n1)
-        : [w0] "s"(w[0]), [w1] "s"(w[1]), [w2] "s"(w[2]), [w3] "s"(w[3]), [w4] "s"(w[4]), [w5] "s"(w[5]), [w6] "s"(w[6]),
-          [w7] "s"(w[7]), [w8] "s"(w[8]), [w9] "s"(w[9]), [w10] "s"(w[10]), [w11] "s"(w[11]), [w12] "s"(w[12]),
-          [w13] "s"(w[13]), [w14] "s"(w[14]), [w15] "s"(w[15]), [i0] "s"(ix[0]), [i1] "s"(ix[1]), [i2] "s"(ix[2]),
-          [i3] "s"(ix[3]), [i4] "s"(ix[4]), [i5] "s"(ix[5]), [i6] "s"(ix[6]), [i7] "s"(ix[7]), [a0] "v"(a0), [a1] "v"(a1)
-        : "m0", "scc");
-}
-#undef GEO_SC_RAIL_FIRST
-#undef GEO_SC_RAIL_PAIR
+GEO_SC_DEFINE_RAIL_LINES(rail_line, rail_line_first, "v64", "v65", "v[64:79]", "v[80:95]", "v[96:111]", "v[112:127]")
+// accumulators at v[32:95]: the kernel with five waves per SIMD (96 registers in all)
+#define GEO_SC_RAIL_PAIR_rail_line_lo(W, SET)                                                                          \
+    SET "v_and_or_b32 v32, %[" W "], %[a0], v32\n"                                                                     \
+        "v_and_or_b32 v33, %[" W "], %[a1], v33\n"
+#define GEO_SC_RAIL_PAIR_rail_line_first_lo(W, SET)                                                                    \
+    SET "v_and_b32 v32, %[" W "], %[a0]\n"                                                                            \
+        "v_and_b32 v33, %[" W "], %[a1]\n"                                                                            \
+        "s_xor_b32 m0, m0, 32\n"                                                                                      \
+        "v_mov_b32 v32, 0\n"                                                                                          \
+        "v_mov_b32 v33, 0\n"
+GEO_SC_DEFINE_RAIL_LINES(rail_line_lo, rail_line_first_lo, "v32", "v33", "v[32:47]", "v[48:63]", "v[64:79]", "v[80:95]")
+#undef GEO_SC_DEFINE_RAIL_LINES
+#undef GEO_SC_RAIL_16
+#undef GEO_SC_RAIL_OPERANDS
 #undef GEO_SC_RAIL_LO
 #undef GEO_SC_RAIL_HI
 
@@ -871,6 +875,114 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 #pragma unroll
         for (int r = 0; r < R; r++)
             if (a0 + r < q.wo) atomicAdd(yo + (size_t)r * q.ho, sum[2 * c + r]);  // integer adds: order does not matter
+    }
+}
+
+// k_conv_fwd_split_rail for launches in which every wave sums exactly one (pack, add group) pair (blockIdx.y =
+// the pair): small layers split as far as they go.  Without running sums a wave needs 96 registers instead of
+// 128 - the 64 accumulators sit at v[32:95], the counts go from the popcounts straight into the atomics - so
+// five waves fit a SIMD instead of four: 5120 waves (the 32 -> 64 5 x 5 layer at 8 x 8, batch 256) are one
+// round instead of two, of which the second would run a quarter full and bound by load latency.
+// Two waves per workgroup, each with a tile of its own: a CU takes at most 16 workgroups, which single-wave
+// workgroups would hit at four waves per SIMD.
+constexpr int kPairWaves = 2;
+template <int WK, int CU>
+__global__ __launch_bounds__(64 * kPairWaves) __attribute__((amdgpu_waves_per_eu(5, 5))) void k_conv_fwd_pair_rail(FwdParams q, unsigned n_tiles)
+{
+    constexpr int C = kCoTile, R = 2, NW = R + WK - 1;
+    const unsigned tile = blockIdx.x * kPairWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (tile >= n_tiles) return;
+    const int cot = tile % q.n_cotile;
+    const long long slot0 = (long long)(tile / q.n_cotile) * 64 + (threadIdx.x & 63);
+    const bool live = slot0 < q.slots;
+    const long long slot = live ? slot0 : 0;
+    const int b = (int)(slot % q.ho);
+    const long long t = slot / q.ho;
+    const int a0 = (int)(t % q.row_groups) * R;
+    const long long n = t / q.row_groups;
+    const unsigned item_stride = (unsigned)q.packs * q.act_plane;
+    unsigned voff[NW];
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+        const int row = a0 + j < q.wi ? a0 + j : q.wi - 1;
+        voff[j] = 4u * ((unsigned)n * item_stride + (unsigned)b + (unsigned)row * q.hi);
+    }
+    const __amdgpu_buffer_rsrc_t act = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(q.act), 0, (int)(4u * (unsigned)q.n * item_stride), 0x00020000);
+    const unsigned plane_b = 4u * q.act_plane, add_b = 4u * q.add_stride, or_b = 4u * q.or_stride;
+
+    const int groups = q.add_outer * q.add_inner;
+    const int pv = blockIdx.y;
+    const int p = pv / groups;
+    const int go = (pv - p * groups) / q.add_inner;
+    const int gi = pv - p * groups - go * q.add_inner;
+    const int ch0 = go * q.or_ch_per_group;
+    const int chs = min(q.or_ch_per_group, q.or_ch_total - ch0);
+    const size_t lines_per_pack = (size_t)q.or_rows * q.add_inner * q.or_ch_total * q.w_k;
+    const size_t line = (size_t)cot * q.rail_lines + p * lines_per_pack + (size_t)ch0 * q.add_inner * q.w_k +
+                        (size_t)gi * chs * q.w_k;
+    const uint32_t* wp = q.wgt_rail + line * C;
+    const uint32_t* ip = q.wgt_rail_idx + line * (C / 2);
+    u32x16 p0, p1, n0, n1;  // written by the group's first line
+    bool first = true;
+    const unsigned group_off = (unsigned)p * plane_b + (unsigned)gi * add_b + (unsigned)ch0 * or_b;
+    for (int row = 0; row < q.or_rows; row++) {
+        unsigned ch_off = group_off + 4u * (unsigned)row;  // next kernel row: one word further
+        auto channels_of = [&](auto cu_tag, auto first_tag) {
+            constexpr int N = decltype(cu_tag)::value;
+            constexpr bool FIRST = decltype(first_tag)::value;
+            uint32_t aw[N][NW];
+#pragma unroll
+            for (int cu = 0; cu < N; cu++)
+#pragma unroll
+                for (int j = 0; j < NW; j++)
+                    aw[cu][j] = __builtin_amdgcn_raw_buffer_load_b32(act, (int)voff[j], (int)(ch_off + (unsigned)cu * or_b), 0);
+            uint32_t wv[N * WK][C], iv[N * WK][C / 2];
+#pragma unroll
+            for (int l = 0; l < N * WK; l++) {
+#pragma unroll
+                for (int c = 0; c < C; c++) wv[l][c] = wp[l * C + c];
+#pragma unroll
+                for (int c = 0; c < C / 2; c++) iv[l][c] = ip[l * (C / 2) + c];
+            }
+#pragma unroll
+            for (int cu = 0; cu < N; cu++)
+#pragma unroll
+                for (int u = 0; u < WK; u++) {
+                    if (FIRST && cu == 0 && u == 0)
+                        rail_line_first_lo(p0, p1, n0, n1, wv[0], iv[0], aw[0][0], aw[0][1]);
+                    else
+                        rail_line_lo(p0, p1, n0, n1, wv[cu * WK + u], iv[cu * WK + u], aw[cu][u], aw[cu][u + 1]);
+                }
+            wp += N * WK * C;
+            ip += N * WK * (C / 2);
+            ch_off += (unsigned)N * or_b;
+        };
+        auto channels = [&](auto cu_tag) {
+            if (first)
+                channels_of(cu_tag, std::true_type());
+            else
+                channels_of(cu_tag, std::false_type());
+            first = false;
+        };
+        int ci = 0;
+        for (; ci + CU <= chs; ci += CU) channels(std::integral_constant<int, CU>());
+        if constexpr (CU > 1)
+            for (; ci < chs; ci++) channels(std::integral_constant<int, 1>());
+    }
+    if (!live) return;
+    const size_t out_plane = (size_t)q.wo * q.ho;
+    int32_t* yo = q.y + ((size_t)n * q.c_out + (size_t)cot * C) * out_plane + (size_t)a0 * q.ho + b;
+    const bool row1 = a0 + 1 < q.wo;
+    // accumulator (channel c, row r) is element 2 c + r of the 32: p0 / n0 hold channels 0 - 7, p1 / n1 8 - 15
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        if (cot * C + c >= q.c_out) break;
+        const u32x16& pv16 = c < C / 2 ? p0 : p1;
+        const u32x16& nv16 = c < C / 2 ? n0 : n1;
+        const int e = 2 * (c % (C / 2));
+        atomicAdd(yo + (size_t)c * out_plane, __popc(pv16[e]) - __popc(nv16[e]));  // integer adds: order does not matter
+        if (row1) atomicAdd(yo + (size_t)c * out_plane + q.ho, __popc(pv16[e + 1]) - __popc(nv16[e + 1]));
     }
 }
 
@@ -1355,6 +1467,11 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
                     hipLaunchKernelGGL((k_conv_fwd_rail_lds<4, 1>), grid_lds, dim3(256), 0, s, q);
             } else if (plain)
                 hipLaunchKernelGGL((k_conv_fwd_rail<WK, CR>), grid, dim3(64), 0, s, q);
+            else if (q.pv_per_block == 1 && waves * splits > 4096)
+                // one pair per wave and more than a round of waves: the form with five waves per SIMD
+                hipLaunchKernelGGL((k_conv_fwd_pair_rail<WK, CR>),
+                                   dim3((unsigned)((blocks + kPairWaves - 1) / kPairWaves), (unsigned)splits),
+                                   dim3(64 * kPairWaves), 0, s, q, (unsigned)blocks);
             else
                 hipLaunchKernelGGL((k_conv_fwd_split_rail<WK, CR>), grid, dim3(64), 0, s, q);
         } else
