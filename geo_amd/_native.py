@@ -69,6 +69,8 @@ C_API = {
                                [_P] * 7),
     "geo_sc_bn_fixed_from_counts": (ctypes.c_int, [_P] + [ctypes.c_int] * 5 + [_P, _P, ctypes.c_float, ctypes.c_float] +
                                     [_P] * 9 + [ctypes.c_size_t, _P]),
+    "geo_sc_quantize_many": (ctypes.c_int, [ctypes.c_int, _P, _P, _P, ctypes.c_int, _P]),
+    "geo_sc_copy_back_clamp": (ctypes.c_int, [ctypes.c_int, _P, _P, _P, _P, ctypes.c_float, ctypes.c_float, _P]),
     "geo_sc_conv2d_add_partial_forward_q7": (ctypes.c_int, [_D, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "geo_sc_quantize": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.c_int, _P]),
     "geo_sc_weight_streams_finish": (ctypes.c_int, [_D, _P, _P]),

@@ -285,6 +285,40 @@ def bn_fixed_from_counts(counts, bit_length, gamma, beta, eps, running_mean=None
     return mean, var, w_n, b_n, invstd, scale
 
 
+def quantize_many(tensors, prec, stream=None):
+    """geo_sc_quantize_many: quantize() of every tensor of the list (contiguous fp32 GPU tensors) in one launch;
+    returns the new tensors."""
+    for t in tensors:
+        _require_gpu_f32(t, "tensor")
+    outs = [torch.empty_like(t) for t in tensors]
+    n = len(tensors)
+    if n:
+        arr = ctypes.c_void_p * n
+        sizes = (ctypes.c_size_t * n)(*[t.numel() for t in tensors])
+        _check(_native.lib().geo_sc_quantize_many(n, arr(*[t.data_ptr() for t in tensors]),
+                                                  arr(*[o.data_ptr() for o in outs]), sizes, int(prec),
+                                                  _stream_ptr(stream)), "geo_sc_quantize_many")
+    return outs
+
+
+def copy_back_clamp(masters, params, orgs, lo, hi, stream=None):
+    """geo_sc_copy_back_clamp: params[i] <- masters[i], and orgs[i] <- clamp(masters[i], lo, hi) where orgs[i] is
+    not None, for all i in one launch (contiguous float32 GPU tensors of equal sizes per i)."""
+    n = len(masters)
+    if n == 0:
+        return
+    for m, p, o in zip(masters, params, orgs):
+        for t in (m, p) + ((o,) if o is not None else ()):
+            if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == m.numel()):
+                raise ValueError("master copies, parameters and buffers must be contiguous float32 GPU tensors")
+    arr = ctypes.c_void_p * n
+    sizes = (ctypes.c_size_t * n)(*[m.numel() for m in masters])
+    _check(_native.lib().geo_sc_copy_back_clamp(n, arr(*[m.data_ptr() for m in masters]),
+                                                arr(*[p.data_ptr() for p in params]),
+                                                arr(*[o.data_ptr() if o is not None else None for o in orgs]), sizes,
+                                                float(lo), float(hi), _stream_ptr(stream)), "geo_sc_copy_back_clamp")
+
+
 def quantize(x, prec, out=None, stream=None):
     """geo_sc_quantize: round(x * 2^prec) clamped to +-(2^prec - 1), over 2^prec, in one launch.
     ``x`` is a contiguous fp32 GPU tensor; ``out`` may be ``x`` itself."""

@@ -505,6 +505,49 @@ __global__ __launch_bounds__(256) void k_quantize(const float* __restrict__ src,
 
 constexpr int kTailMaxChannels = 4096;
 
+// The end of the reference's training step (utils_own.py:108-113) for up to kMaxStepTensors parameters in one
+// launch: every parameter takes its master copy's value, and where the layer keeps a full-precision buffer
+// (weight_org) that buffer becomes the new value clamped to [lo, hi].  blockIdx.y = parameter.
+constexpr int kMaxStepTensors = 24;
+struct StepTensors {
+    const float* master[kMaxStepTensors];
+    float* param[kMaxStepTensors];
+    float* org[kMaxStepTensors];   // null: no such buffer
+    size_t n[kMaxStepTensors];
+};
+__global__ __launch_bounds__(256) void k_copy_back_clamp(StepTensors t, float lo, float hi)
+{
+    const int i = blockIdx.y;
+    const float* __restrict__ src = t.master[i];
+    float* __restrict__ dst = t.param[i];
+    float* __restrict__ org = t.org[i];
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < t.n[i]; e += (size_t)gridDim.x * 256) {
+        const float v = src[e];
+        dst[e] = v;
+        // torch.clamp: NaN stays NaN
+        if (org) org[e] = v < lo ? lo : (v > hi ? hi : v);
+    }
+}
+
+// quantize for several tensors in one launch (the weights of all layers of a network); blockIdx.y = tensor
+struct QuantTensors {
+    const float* src[kMaxStepTensors];
+    float* dst[kMaxStepTensors];
+    size_t n[kMaxStepTensors];
+};
+__global__ __launch_bounds__(256) void k_quantize_many(QuantTensors t, float scale, float inv_scale)
+{
+    const int i = blockIdx.y;
+    const float* __restrict__ src = t.src[i];
+    float* __restrict__ dst = t.dst[i];
+    const float hi = scale - 1.0f;
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < t.n[i]; e += (size_t)gridDim.x * 256) {
+        float v = rintf(src[e] * scale);
+        v = v < -hi ? -hi : (v > hi ? hi : v);
+        dst[e] = v * inv_scale;
+    }
+}
+
 int tail_splits(int n, int c, int w, int h)
 {
     // enough blocks to fill the GPU, not more than the channel has 256-element chunks
@@ -732,5 +775,56 @@ extern "C" int geo_sc_quantize(const float* src, float* dst, size_t n, int prec,
     if (blocks > 256 * 16) blocks = 256 * 16;
     hipLaunchKernelGGL(k_quantize, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, src, dst, n, scale,
                        1.0f / scale);
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_copy_back_clamp(int count, const float* const* master, float* const* param, float* const* org,
+                                      const size_t* elements, float lo, float hi, geo_sc_stream_t stream)
+{
+    if (count < 0 || (count > 0 && (!master || !param || !elements))) return GEO_SC_ERR_INVALID_ARGUMENT;
+    for (int first = 0; first < count; first += kMaxStepTensors) {
+        const int m = count - first < kMaxStepTensors ? count - first : kMaxStepTensors;
+        StepTensors t = {};
+        size_t most = 0;
+        for (int i = 0; i < m; i++) {
+            if (!master[first + i] || !param[first + i]) return GEO_SC_ERR_INVALID_ARGUMENT;
+            t.master[i] = master[first + i];
+            t.param[i] = param[first + i];
+            t.org[i] = org ? org[first + i] : nullptr;
+            t.n[i] = elements[first + i];
+            if (t.n[i] > most) most = t.n[i];
+        }
+        size_t blocks = (most + 255) / 256;
+        if (blocks < 1) blocks = 1;
+        if (blocks > 1024) blocks = 1024;
+        hipLaunchKernelGGL(k_copy_back_clamp, dim3((unsigned)blocks, (unsigned)m), dim3(256), 0, (hipStream_t)stream, t, lo,
+                           hi);
+    }
+    return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
+}
+
+extern "C" int geo_sc_quantize_many(int count, const float* const* src, float* const* dst, const size_t* elements,
+                                    int prec, geo_sc_stream_t stream)
+{
+    if (prec < 1 || prec > 23 || count < 0 || (count > 0 && (!src || !dst || !elements)))
+        return GEO_SC_ERR_INVALID_ARGUMENT;
+    const float scale = (float)(1u << prec);
+    for (int first = 0; first < count; first += kMaxStepTensors) {
+        const int m = count - first < kMaxStepTensors ? count - first : kMaxStepTensors;
+        QuantTensors t = {};
+        size_t most = 0;
+        for (int i = 0; i < m; i++) {
+            if (!src[first + i] || !dst[first + i]) return GEO_SC_ERR_INVALID_ARGUMENT;
+            t.src[i] = src[first + i];
+            t.dst[i] = dst[first + i];
+            t.n[i] = elements[first + i];
+            if (t.n[i] > most) most = t.n[i];
+        }
+        size_t blocks = (most + 255) / 256;
+        if (blocks < 1) blocks = 1;
+        if (blocks > 1024) blocks = 1024;
+        hipLaunchKernelGGL(k_quantize_many, dim3((unsigned)blocks, (unsigned)m), dim3(256), 0, (hipStream_t)stream, t,
+                           scale, 1.0f / scale);
+    }
     return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
 }

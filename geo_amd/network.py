@@ -73,7 +73,7 @@ class CONV_tiny_add_partial(nn.Module):
         return utils_class.sc_conv_block(conv, bn, x, err=self.err[i], forward=self.compute,
                                          z_unit=2 ** self.z_unit[i], load_unit=self.load_unit[i],
                                          load_wait_w=self.load_wait[j], load_wait_a=self.load_wait[i],
-                                         torch_stats=self.fused_torch_stats, **tail)
+                                         torch_stats=self.fused_torch_stats, weight_ready=True, **tail)
 
     def _block(self, conv, bn, x, i):
         if self._fusable(x):
@@ -84,6 +84,9 @@ class CONV_tiny_add_partial(nn.Module):
         return self.tanh(self.pool(x))
 
     def forward(self, x_in, target=None):
+        if self._fusable(x_in):
+            # the four layers' weight quantisation (utils_class.py:33) in one launch
+            utils_class.quantize_weights([self.conv1, self.conv2, self.conv3, self.fc1])
         x = self._block(self.conv1, self.bn1, x_in, 0)
         x = self._block(self.conv2, self.bn2, x, 1)
         x = self._block(self.conv3, self.bn3, x, 2)
@@ -280,10 +283,17 @@ def apply_update(model, optimizer, param_copy):
         for (master, _), g in zip(with_grad, scaled):
             master.grad = g
     optimizer.step()
-    torch._foreach_copy_([p.data for p in params], [master.data for master in param_copy])
-    for m in model.modules():
-        if hasattr(m, "weight_org"):
-            torch.clamp(m.weight.data, -1, 0.999, out=m.weight_org)
+    orgs = {id(m.weight): m.weight_org for m in model.modules() if hasattr(m, "weight_org")}
+    if all(p.is_cuda and p.dtype == torch.float32 and p.data.is_contiguous() for p in params):
+        # copy back and refresh weight_org, all parameters in one launch
+        from . import capi
+        capi.copy_back_clamp([master.data for master in param_copy], [p.data for p in params],
+                             [orgs.get(id(p)) for p in params], -1, 0.999)
+    else:
+        torch._foreach_copy_([p.data for p in params], [master.data for master in param_copy])
+        for p in params:
+            if id(p) in orgs:
+                torch.clamp(p.data, -1, 0.999, out=orgs[id(p)])
     optimizer.zero_grad()
 
 

@@ -139,8 +139,20 @@ class _SCConvBlock(torch.autograd.Function):
                 None)
 
 
+def quantize_weights(convs, prec=7):
+    """``conv.weight.data = quantize(conv.weight_org, prec)`` (utils_class.py:33) for several layers in one launch;
+    ``sc_conv_block(..., weight_ready=True)`` then skips its own."""
+    if all(c.weight_org.is_cuda and c.weight_org.dtype == torch.float32 and c.weight_org.is_contiguous() for c in convs):
+        from . import capi
+        for c, q in zip(convs, capi.quantize_many([c.weight_org for c in convs], prec)):
+            c.weight.data = q
+    else:
+        for c in convs:
+            c.weight.data = utils_functional.quantize(c.weight_org, prec=prec)
+
+
 def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_unit=8, load_wait_w=2, load_wait_a=2,
-                  prec=7, relu=False, pool=True, hardtanh=True, quant7=True, torch_stats=False):
+                  prec=7, relu=False, pool=True, hardtanh=True, quant7=True, torch_stats=False, weight_ready=False):
     """``hardtanh(pool(relu(bn(conv(input)))))`` of a ``Conv2d_Add_Partial`` and a
     ``BatchNorm2d_fixed`` / ``BatchNorm1d_fixed`` in training mode, fused (LFSR generators, GPU
     tensors).  Same in-place quantisation of ``input.data`` and ``conv.weight.data`` as
@@ -156,7 +168,8 @@ def sc_conv_block(conv, bn, input, *, err=7, forward="1d_bin", z_unit=8, load_un
     # an input that is the untouched 7-bit output of a fused block already holds quantize(input, 7)
     if not (prec == 7 and getattr(input, "_geo_q7_version", None) == input._version):
         input.data = utils_functional.quantize(input.data, prec=prec)
-    conv.weight.data = utils_functional.quantize(conv.weight_org, prec=prec)
+    if not weight_ready:   # (quantize_weights has done it for all layers of the network)
+        conv.weight.data = utils_functional.quantize(conv.weight_org, prec=prec)
     mode = {"1d_bin": "y", "z_bin": "z", "yz_bin": "yz"}[forward]
     kw = dict(bit_length=2 ** err, padding=(int(conv.padding[0]), int(conv.padding[1])),
               total_width=utils_functional.prec_default, load_width=int(load_unit), load_wait_w=int(load_wait_w),
