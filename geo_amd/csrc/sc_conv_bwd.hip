@@ -479,7 +479,10 @@ struct SplitStager {
 // its own position, shifted once); as the I-major operand of the weight-gradient product they are the k
 // dimension: a thread's eight positions and a whole chunk lie inside one item (a_item is a multiple of
 // kChunk), and the pointer jumps by a_skip when it passes an item's end.
-template <bool KMAJOR>
+// AHEAD (K-major only): the table entries of a chunk are read when the chunk before it is fetched, so that a
+// fetch issues its loads without waiting for the table first; the entries read for the chunk behind the last
+// one (up to 2 * kChunk + 8 entries behind the member's part of the table) are never used.
+template <bool KMAJOR, bool AHEAD = false>
 struct ViewStager {
     const float* base;
     const long long* rows;  // K-major: the table of this batch member (uniform)
@@ -488,6 +491,15 @@ struct ViewStager {
     int kr;                 // K-major: first row of this thread's half of the current chunk
     int in_item, item, skip;
     int half, ii;
+    long long ahead[(KMAJOR && AHEAD) ? 8 : 1];  // the rows' starts of the chunk to fetch next
+
+    __device__ __forceinline__ void read_ahead()
+    {
+        if constexpr (KMAJOR && AHEAD) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) ahead[c] = rows[kr + c];
+        }
+    }
 
     __device__ __forceinline__ void init(const GemmParams& q, int batch, int i0, int k_begin, int I, int ii_, int half_)
     {
@@ -501,6 +513,13 @@ struct ViewStager {
             const int m = min(i0 + ii, I - 1);
             off = m + (m / item) * skip;
             kr = k_begin + 8 * half;
+            read_ahead();
+            if constexpr (AHEAD) {
+                // wait for these entries here, where a tile is opened, and not where this path meets the one
+                // of the later fetches: there the wait would also take in the data loads of the fetch before
+#pragma unroll
+                for (int c = 0; c < 8; c++) asm volatile("" ::"v"(ahead[c]));
+            }
         } else {
             const int m = k_begin + 8 * half;
             in_item = m % item;
@@ -520,9 +539,20 @@ struct ViewStager {
             }
         }
     }
-    __device__ __forceinline__ void skip_chunk() { advance(); }
+    __device__ __forceinline__ void skip_chunk()
+    {
+        advance();
+        read_ahead();
+    }
     __device__ __forceinline__ void fetch_whole(float (&r)[8])
     {
+        if constexpr (KMAJOR && AHEAD) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) r[c] = (base + ahead[c])[off];
+            advance();
+            read_ahead();
+            return;
+        }
         if (KMAJOR) {
 #pragma unroll
             for (int c = 0; c < 8; c++) r[c] = (base + rows[kr + c])[off];
@@ -880,7 +910,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int a_ii = A_KMAJOR ? (wa % NX) * 64 + lane : ta / (2 * KC);
     const int a_q = A_KMAJOR ? wa / NX : ta % (2 * KC);  // which eight k of the trip
     const int b_ii = BK ? (t & 255) : (t >> 1), b_half = BK ? (wave >> 2) : (t & 1);
-    typename std::conditional<VA, ViewStager<A_KMAJOR>, SplitStager<A_KMAJOR>>::type sa;
+    typename std::conditional<VA, ViewStager<A_KMAJOR, true>, SplitStager<A_KMAJOR>>::type sa;
     typename std::conditional<VB, ShiftStager, SplitStager<B_KMAJOR>>::type sb;
 
     const int n_tiles = q.ni * q.nj * q.nz;
@@ -902,11 +932,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         else
             sb.init(q.b + batch * q.b_batch_stride, q.ldb, jt * kBigJ, k_begin, q.J, b_ii, b_half);
     };
-    // the next trip's worth of the stream into a register set; nothing once the last tile is through
+    // The next trip's worth of the stream into a register set.  Once the last tile is through, the fetches go
+    // round that tile again (loads of valid addresses that nobody uses): every path through here issues the
+    // same loads, so the waits that the compiler places in front of the split count only the loads of the
+    // set they need - with a path that issues none, they would wait for the newest loads as well.
     auto fetch_next = [&](float (&ra)[8], float (&rb)[KC][8]) {
         if (left_f == 0) {
-            if (w_f + (int)gridDim.x >= n_tiles) return;
-            w_f += gridDim.x;
+            if (w_f + (int)gridDim.x < n_tiles) w_f += gridDim.x;
             open_tile();
         }
         sa.fetch_whole(ra);
@@ -1025,21 +1057,36 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         fetch_next(ra[R], rb[R]);
         __syncthreads();
     };
-    // after a trip: was that the tile's last?  Then its results go out; true when it was the last tile.
-    auto tile_done = [&]() -> bool {
-        if (--left_m > 0) return false;
+    // after a trip: was that the tile's last?  Then its results go out.  Behind the last tile nothing is stored
+    // any more (a trip that still follows multiplies what the fetches past the end left in LDS).
+    auto tile_done = [&]() {
+        if (--left_m > 0) return;
         store_tile<EPI, NX, 2, 2, true>(q, acc, out_m, i0_m + wi, j0_m + wj, l32, lk);
-        if (w_m + (int)gridDim.x >= n_tiles) return true;
+        if (w_m + (int)gridDim.x >= n_tiles) {
+            left_m = 0x7fffffff;
+            return;
+        }
         w_m += gridDim.x;
         describe_m();
         zero_acc();
-        return false;
     };
-    for (;;) {
+    // The loop leaves at its end only, after a counted number of trip pairs (one trip more than the stream has
+    // when that number is odd).  With an exit between the two trips the compiler's structured form of the loop
+    // has a path from the first trip straight back to itself, and on that path the register set that the
+    // first trip splits is the newest one loaded: its waits would then cover the loads of the trip before
+    // instead of those of two trips before.
+    int trips = 0;
+    for (int w = blockIdx.x; w < n_tiles; w += gridDim.x) {
+        int it, jt, z;
+        gemm_tile_of(q, w, it, jt, z);
+        const int k_begin = (z % q.splits) * q.k_per_split;
+        trips += (min(q.K, k_begin + q.k_per_split) - k_begin) / kUnit;
+    }
+    for (int n = (trips + 1) >> 1; n > 0; n--) {
         trip(std::integral_constant<int, 0>());
-        if (tile_done()) break;
+        tile_done();
         trip(std::integral_constant<int, 1>());
-        if (tile_done()) break;
+        tile_done();
     }
 }
 
@@ -2511,7 +2558,8 @@ BwdLayout bwd_layout(const Geometry& g, int groups_per_round)
         o += align256(sizeof(float) * (b.fused_k && tiled > plain ? tiled : plain));
     }
     b.off_rows = o;
-    o += align256(sizeof(long long) * (size_t)b.G.n_groups * b.view_k_pad);
+    // (and behind it the entries that the eight-wave kernel reads ahead of the last chunk)
+    o += align256(sizeof(long long) * ((size_t)b.G.n_groups * b.view_k_pad + 2 * kChunk + 8));
     b.off_zero = o;
     o += 256;
     b.bytes = o;
