@@ -741,8 +741,10 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
     };
     int c = 0;
     // Whole chunks, no branches in the trip.  The split of chunk c + 1 (vector ALU, 24 steps: three per
-    // pair of elements) is written between the MFMAs of chunk c, one step per MFMA with four blocks, and
-    // scheduling barriers keep that order, so that it issues while the matrix pipe is busy.
+    // pair of elements) is written between the MFMAs of chunk c, one step per MFMA with four blocks, so
+    // that it issues while the matrix pipe is busy.  (Scheduling barriers that spelled this order out held in
+    // the first of the loop's two trips only: in the second the compiler chained the six MFMAs of each
+    // block back to back.  Without them both trips keep the written order.)
     const int n_whole = k_len > 0 ? k_len / kChunk : 0;
     constexpr int kMfmas = NX * NY > 0 ? 6 * NX * NY : 1;  // per trip
     constexpr int kStepsPerMfma = (24 + kMfmas - 1) / kMfmas;
@@ -792,14 +794,6 @@ __device__ __forceinline__ void gemm_wave_split(const GemmParams& q, uint4 (*as)
         bs[S ^ 1][0][sb.half][sb.ii] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
         bs[S ^ 1][1][sb.half][sb.ii] = make_uint4(mid[4], mid[5], mid[6], mid[7]);
         bs[S ^ 1][2][sb.half][sb.ii] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-        // order asked of the scheduler: LDS reads, then one MFMA and a share of the vector ALU work in turn
-        __builtin_amdgcn_sched_group_barrier(0x100, 3 * (NX + NY), 0);
-#pragma unroll
-        for (int m = 0; m < kMfmas; m++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, (88 + kMfmas - 1) / kMfmas, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x200, 6, 0);
         __syncthreads();
     };
     if (NX * NY > 0) {
