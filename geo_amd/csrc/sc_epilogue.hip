@@ -787,7 +787,7 @@ extern "C" int geo_sc_copy_back_clamp(int count, const float* const* master, flo
         StepTensors t = {};
         size_t most = 0;
         for (int i = 0; i < m; i++) {
-            if (!master[first + i] || !param[first + i]) return GEO_SC_ERR_INVALID_ARGUMENT;
+            if (elements[first + i] && (!master[first + i] || !param[first + i])) return GEO_SC_ERR_INVALID_ARGUMENT;
             t.master[i] = master[first + i];
             t.param[i] = param[first + i];
             t.org[i] = org ? org[first + i] : nullptr;
@@ -814,7 +814,7 @@ extern "C" int geo_sc_quantize_many(int count, const float* const* src, float* c
         QuantTensors t = {};
         size_t most = 0;
         for (int i = 0; i < m; i++) {
-            if (!src[first + i] || !dst[first + i]) return GEO_SC_ERR_INVALID_ARGUMENT;
+            if (elements[first + i] && (!src[first + i] || !dst[first + i])) return GEO_SC_ERR_INVALID_ARGUMENT;
             t.src[i] = src[first + i];
             t.dst[i] = dst[first + i];
             t.n[i] = elements[first + i];

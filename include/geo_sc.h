@@ -382,13 +382,14 @@ GEO_SC_API int geo_sc_bn_fixed_from_counts(const int32_t* counts, int n, int c, 
  * and to weight_org on every call (utils_class.py:32-33).  n fp32 elements on the device; dst may be src.
  */
 GEO_SC_API int geo_sc_quantize(const float* src, float* dst, size_t n, int prec, geo_sc_stream_t stream);
-/* The same for `count` tensors in one launch (the weight_org buffers of all layers of a network at the start of
- * a forward): src, dst and elements are HOST arrays of `count` entries, the tensors are on the device. */
+/* The same for `count` tensors in one launch per 24 of them (the weight_org buffers of all layers of a network
+ * at the start of a forward): src, dst and elements are HOST arrays of `count` entries, the tensors are on the
+ * device; a tensor of no elements may have null pointers. */
 GEO_SC_API int geo_sc_quantize_many(int count, const float* const* src, float* const* dst, const size_t* elements,
                                     int prec, geo_sc_stream_t stream);
 
 /*
- * The end of the reference's training step (utils_own.py:108-113) in one launch for `count` parameters:
+ * The end of the reference's training step (utils_own.py:108-113) in one launch per 24 of `count` parameters:
  * param[i] <- master[i] (the optimiser's full-precision copy, `elements[i]` floats), and where org[i] is not
  * NULL (a layer's weight_org buffer) org[i] <- clamp(master[i], lo, hi).  master, param, org (may be NULL
  * altogether) and elements are HOST arrays of `count` entries; the tensors are on the device.

@@ -193,3 +193,75 @@ def test_quantize_kernel_equals_the_torch_op_chain():
     y = xd.clone()
     assert capi.quantize(y, 7, out=y) is y and torch.equal(torch.nan_to_num(y), torch.nan_to_num(capi.quantize(xd, 7)))
     assert capi.quantize(torch.empty(0, device="cuda"), 7).numel() == 0
+
+
+def test_quantize_many_equals_quantize_per_tensor(capi):
+    """geo_sc_quantize_many: every tensor of the list as geo_sc_quantize gives it (odd sizes, an empty one, more
+    tensors than one launch takes)."""
+    g = torch.Generator().manual_seed(11)
+    sizes = [1, 3, 1000, 4097, 0, 25 * 32 * 32, 7] + [5] * 23
+    xs = [(torch.rand(n, generator=g) * 4 - 2).cuda() for n in sizes]
+    assert len(xs) == 30
+    xs[2][:4] = torch.tensor([0.5 / 128, 1.5 / 128, -2.5 / 128, 127.5 / 128], device="cuda")   # ties
+    for prec in (7, 3):
+        got = capi.quantize_many(xs, prec)
+        for x, q in zip(xs, got):
+            assert q.shape == x.shape and torch.equal(q, capi.quantize(x, prec))
+    assert capi.quantize_many([], 7) == []
+    with pytest.raises(Exception):
+        capi.quantize_many(xs, 0)   # precision out of range
+
+
+def test_copy_back_clamp_equals_the_torch_ops(capi):
+    """geo_sc_copy_back_clamp against the end of the reference's training step (utils_own.py:108-113):
+    p.data <- master, weight_org <- master.clamp(-1, 0.999), for parameters with and without such a buffer."""
+    g = torch.Generator().manual_seed(12)
+    sizes = [25 * 3 * 32, 10, 4099, 64, 1]
+    masters = [(torch.rand(n, generator=g) * 3 - 1.5).cuda() for n in sizes]
+    masters[1][:4] = torch.tensor([-1.0, 0.999, 1.0, -1.0000001], device="cuda")
+    params = [torch.full((n,), 7.0, device="cuda") for n in sizes]
+    orgs = [torch.full((n,), 9.0, device="cuda") if i % 2 == 0 else None for i, n in enumerate(sizes)]
+    capi.copy_back_clamp(masters, params, orgs, -1.0, 0.999)
+    torch.cuda.synchronize()
+    for m, p, o in zip(masters, params, orgs):
+        assert torch.equal(p, m)
+        if o is not None:
+            assert torch.equal(o, m.clamp(-1.0, 0.999))
+    capi.copy_back_clamp([], [], [], -1.0, 0.999)
+    with pytest.raises(ValueError):
+        capi.copy_back_clamp(masters[:1], [params[1]], [None], -1.0, 0.999)   # sizes differ
+    # more tensors than one launch takes
+    many_m = [(torch.rand(9, generator=g) * 3 - 1.5).cuda() for _ in range(30)]
+    many_p, many_o = [torch.zeros(9, device="cuda") for _ in many_m], [torch.zeros(9, device="cuda") for _ in many_m]
+    capi.copy_back_clamp(many_m, many_p, many_o, -1.0, 0.999)
+    for m, p, o in zip(many_m, many_p, many_o):
+        assert torch.equal(p, m) and torch.equal(o, m.clamp(-1.0, 0.999))
+
+
+@pytest.mark.parametrize("shape,L", [((64, 32, 16, 16), 64), ((37, 10, 1, 1), 64), ((8, 700, 4, 4), 128), ((256, 64, 4, 4), 256)])
+def test_bn_fixed_from_counts_is_statistics_plus_affine(capi, shape, L):
+    """geo_sc_bn_fixed_from_counts = geo_sc_count_stats + geo_sc_bn_fixed_affine (two launches instead of three,
+    the partial sums handed over in the workspace): the same bits in every output, and the exact statistics
+    against float64 sums of the integers."""
+    g = torch.Generator().manual_seed(shape[1])
+    counts = torch.randint(-5 * L, 5 * L + 1, shape, generator=g, dtype=torch.int32).cuda()
+    c = shape[1]
+    gamma, beta = (torch.rand(c, generator=g) + 0.5).cuda(), (torch.rand(c, generator=g) - 0.5).cuda()
+    rm0, rv0 = torch.rand(c, generator=g).cuda(), (torch.rand(c, generator=g) + 0.5).cuda()
+    rm1, rv1 = rm0.clone(), rv0.clone()
+    mean, var, w_n, b_n, invstd, scale = capi.bn_fixed_from_counts(counts, L, gamma, beta, 1e-5, rm1, rv1)
+    m2, v2 = capi.count_stats(counts, L)
+    n_per = counts.numel() // c
+    rm2, rv2 = rm0.clone(), rv0.clone()
+    w2, b2, i2, s2 = capi.bn_fixed_affine(m2, v2, gamma, beta, 1e-5, n_per, rm2, rv2)
+    torch.cuda.synchronize()
+    for a, b in ((mean, m2), (var, v2), (w_n, w2), (b_n, b2), (invstd, i2), (scale, s2), (rm1, rm2), (rv1, rv2)):
+        assert torch.equal(a, b)
+    # the statistics from the integers themselves: sums in int64 (exact), one division in float64
+    ci = counts.cpu().long().permute(1, 0, 2, 3).reshape(c, -1)
+    s1, s2 = ci.sum(1), (ci * ci).sum(1)
+    exact_mean = (s1.double() / (n_per * L)).float()
+    exact_var = ((n_per * s2 - s1 * s1).double() / (float(n_per) ** 2 * float(L) ** 2)).float()
+    assert torch.equal(mean.cpu(), exact_mean)
+    ulp = torch.abs(torch.nextafter(exact_var, torch.full_like(exact_var, float("inf"))) - exact_var)
+    assert bool((torch.abs(var.cpu() - exact_var) <= ulp).all())
