@@ -885,13 +885,24 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 // round instead of two, of which the second would run a quarter full and bound by load latency.
 // Two waves per workgroup, each with a tile of its own: a CU takes at most 16 workgroups, which single-wave
 // workgroups would hit at four waves per SIMD.
-constexpr int kPairWaves = 2;
-template <int WK, int CU>
-__global__ __launch_bounds__(64 * kPairWaves) __attribute__((amdgpu_waves_per_eu(5, 5))) void k_conv_fwd_pair_rail(FwdParams q, unsigned n_tiles)
+// WG: the pairs of one tile as the waves of one workgroup (at most 16 pairs): their counts meet in LDS
+// (ds_add_u32) and the workgroup stores the sums - no zeroing launch over y and no global atomics, whose
+// drain is what such a launch otherwise ends with (the 32 -> 64 layer: waves live 59 us of the 88 us that
+// the launch with atomics takes).
+constexpr int kPairWaves = 2, kPairWgMax = 16;
+template <int WK, int CU, bool WG = false>
+__global__ __launch_bounds__(WG ? 64 * kPairWgMax : 64 * kPairWaves) __attribute__((amdgpu_waves_per_eu(5, 5)))
+void k_conv_fwd_pair_rail(FwdParams q, unsigned n_tiles)
 {
     constexpr int C = kCoTile, R = 2, NW = R + WK - 1;
-    const unsigned tile = blockIdx.x * kPairWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (tile >= n_tiles) return;
+    __shared__ int red[WG ? 2 * C * 64 : 1];  // [2 c + r][lane]
+    const int wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned tile = WG ? blockIdx.x : blockIdx.x * kPairWaves + wave_in_wg;
+    if (!WG && tile >= n_tiles) return;
+    if constexpr (WG) {
+        for (int i = threadIdx.x; i < 2 * C * 64; i += blockDim.x) red[i] = 0;
+        __syncthreads();
+    }
     const int cot = tile % q.n_cotile;
     const long long slot0 = (long long)(tile / q.n_cotile) * 64 + (threadIdx.x & 63);
     const bool live = slot0 < q.slots;
@@ -912,7 +923,7 @@ __global__ __launch_bounds__(64 * kPairWaves) __attribute__((amdgpu_waves_per_eu
     const unsigned plane_b = 4u * q.act_plane, add_b = 4u * q.add_stride, or_b = 4u * q.or_stride;
 
     const int groups = q.add_outer * q.add_inner;
-    const int pv = blockIdx.y;
+    const int pv = WG ? wave_in_wg : blockIdx.y;
     const int p = pv / groups;
     const int go = (pv - p * groups) / q.add_inner;
     const int gi = pv - p * groups - go * q.add_inner;
@@ -970,11 +981,28 @@ __global__ __launch_bounds__(64 * kPairWaves) __attribute__((amdgpu_waves_per_eu
         if constexpr (CU > 1)
             for (; ci < chs; ci++) channels(std::integral_constant<int, 1>());
     }
-    if (!live) return;
     const size_t out_plane = (size_t)q.wo * q.ho;
     int32_t* yo = q.y + ((size_t)n * q.c_out + (size_t)cot * C) * out_plane + (size_t)a0 * q.ho + b;
     const bool row1 = a0 + 1 < q.wo;
     // accumulator (channel c, row r) is element 2 c + r of the 32: p0 / n0 hold channels 0 - 7, p1 / n1 8 - 15
+    if constexpr (WG) {
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int e = 0; e < 2 * C; e++) {
+            const u32x16& pv16 = e < C ? p0 : p1;
+            const u32x16& nv16 = e < C ? n0 : n1;
+            atomicAdd(&red[e * 64 + lane], __popc(pv16[e % C]) - __popc(nv16[e % C]));  // result unused: ds_add_u32
+        }
+        __syncthreads();
+        if (!live) return;
+        const int n_waves = blockDim.x >> 6;
+        for (int e = wave_in_wg; e < 2 * C; e += n_waves) {
+            const int c = e >> 1, r = e & 1;
+            if (cot * C + c < q.c_out && (r == 0 || row1)) yo[(size_t)c * out_plane + (size_t)r * q.ho] = red[e * 64 + lane];
+        }
+        return;
+    }
+    if (!live) return;
 #pragma unroll
     for (int c = 0; c < C; c++) {
         if (cot * C + c >= q.c_out) break;
@@ -1439,7 +1467,13 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
         hipLaunchKernelGGL((k_conv_fwd_items_rail_wg<WK, CU, S>), dim3((unsigned)blocks), dim3(64 * S), 0, s, q);
         return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
     }
-    if (!plain) {
+    // one (pack, add group) pair per wave and more than a round of waves: the form with five waves per SIMD,
+    // with the pairs of a tile in one workgroup where they are few enough
+    const bool pair = g.rail && R == 2 && WK > 0 && !lds && !plain && q.pv_per_block == 1 && waves * splits > 4096;
+    // (in one round of five waves per SIMD only: with a second round, whole workgroups wait for ten free wave
+    // slots of one CU, and the 32 -> 32 layer at 16 x 16 takes 161 us instead of 135 us)
+    const bool pair_wg = pair && splits <= kPairWgMax && waves * splits <= 5 * 4 * 256;
+    if (!plain && !pair_wg) {
         const size_t n_out = (size_t)g.n * g.c_out * g.wo * g.ho;
         size_t zb = (n_out + 255) / 256;
         hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)(zb > 4096 ? 4096 : zb)), dim3(256), 0, s, q.y, n_out);
@@ -1467,8 +1501,10 @@ int launch(const Geometry& g, FwdParams q, hipStream_t s)
                     hipLaunchKernelGGL((k_conv_fwd_rail_lds<4, 1>), grid_lds, dim3(256), 0, s, q);
             } else if (plain)
                 hipLaunchKernelGGL((k_conv_fwd_rail<WK, CR>), grid, dim3(64), 0, s, q);
-            else if (q.pv_per_block == 1 && waves * splits > 4096)
-                // one pair per wave and more than a round of waves: the form with five waves per SIMD
+            else if (pair_wg)
+                hipLaunchKernelGGL((k_conv_fwd_pair_rail<WK, CR, true>), dim3((unsigned)blocks), dim3(64 * splits), 0, s, q,
+                                   (unsigned)blocks);
+            else if (pair)
                 hipLaunchKernelGGL((k_conv_fwd_pair_rail<WK, CR>),
                                    dim3((unsigned)((blocks + kPairWaves - 1) / kPairWaves), (unsigned)splits),
                                    dim3(64 * kPairWaves), 0, s, q, (unsigned)blocks);

@@ -453,6 +453,31 @@ def test_large_y_mode_launches_skip_the_zero_rail(capi, so, shape_x, shape_w, pa
         capi.conv2d_add_partial_from_streams(capi.act_streams(x.cuda(), d), short, d)
 
 
+# ------------------------------------------------------------------ launches split over (pack, kernel row) pairs
+@pytest.mark.parametrize("shape_x,shape_w,pad,L,loading", [
+    ((256, 32, 8, 8), (64, 32, 5, 5), (2, 2), 64, (7, 2, 2, 2)),     # 5120 waves, one pair each: the pairs of a tile in one workgroup
+    ((250, 32, 8, 8), (60, 32, 5, 5), (2, 2), 64, (7, 8, 1, 1)),     # the same with a ragged last tile and a partial c_out tile
+    ((256, 32, 16, 16), (32, 32, 5, 5), (2, 2), 64, (7, 2, 2, 2)),   # 10240 waves: two rounds, one pair per wave with atomics
+    ((200, 16, 8, 9), (48, 16, 3, 3), (1, 1), 256, (7, 8, 1, 1)),    # 24 pairs: more than a workgroup takes
+    ((64, 32, 8, 8), (64, 32, 5, 5), (2, 2), 64, (7, 8, 1, 1)),      # 1280 waves: under a round, several pairs per wave
+])
+def test_split_launches_match_oracle(capi, so, shape_x, shape_w, pad, L, loading):
+    """Small layers whose (pack, kernel row) passes are split over waves (the 4-layer CNN's second and third
+    layer at batch 256): every form of the split launch against the oracle, bit for bit, twice in a row (the
+    second call finds the first one's counts in y)."""
+    x, w = wl.make_inputs(shape_x, shape_w, "q7", seed=shape_w[0] + L)
+    w.view(-1)[::7] = 0.0
+    tw, lw, ww, wa = loading
+    exp = so.conv2d_add_partial(x.numpy(), w.numpy(), L, pad, tw, lw, ww, wa)
+    d = capi.make_desc(x.shape, w.shape, L, pad, tw, lw, ww, wa)
+    y = torch.full(capi.output_shape(d), 12345, dtype=torch.int32, device="cuda")
+    act, wgt = capi.act_streams(x.cuda(), d), capi.weight_streams(w.cuda(), d)
+    for _ in range(2):
+        capi.conv2d_add_partial_from_streams(act, wgt, d, out=y)
+        assert np.array_equal(y.cpu().numpy(), exp)
+    assert np.array_equal(capi.conv2d_add_partial_forward(x.cuda(), w.cuda(), L, pad, tw, lw, ww, wa).cpu().numpy(), exp)
+
+
 # ------------------------------------------------------------------ batches cut into chunks
 @pytest.mark.parametrize("shape_x,shape_w,pad,L,kw", [
     ((11, 6, 9, 8), (20, 6, 3, 3), (1, 1), 64, {}),                                   # position-major, 3-wide
