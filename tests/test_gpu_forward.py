@@ -551,3 +551,40 @@ def test_forward_uncut_at_the_resnet_shape(capi, checksums):
     a = capi.conv2d_add_partial_forward_q7(k, wq7.cuda(), 256, (pad, pad))
     b = capi.conv2d_add_partial_forward(xq7.cuda(), wq7.cuda(), 256, (pad, pad), options=whole)
     assert torch.equal(a, b) and int(a.abs().max()) > 0
+
+
+def test_chunked_forward_in_a_hip_graph(capi):
+    """A cut batch alternates between the caller's stream and a second stream of the library (forked and joined
+    with events): captured after geo_sc_init, the whole fork-join becomes part of the graph.  Replayed three
+    times, with eager calls (which overwrite the workspace) and synchronisations between the replays, every
+    replay against the eager result."""
+    L, pad = 64, (1, 1)
+    x, w = wl.make_inputs((12, 6, 9, 8), (20, 6, 3, 3), "q7", seed=21)
+    xd, wd = x.cuda(), w.cuda()
+    d = capi.make_desc(x.shape, w.shape, L, pad)
+    item = 4 * 2 * 6 * 11 * 10
+    opt = capi.make_options(forward_stream_bytes=6 * item)       # chunks of three items: four chunks, two per stream
+    assert capi.forward_chunk(d, opt) == 3
+    ws = torch.empty(capi.workspace_size(d, opt), dtype=torch.uint8, device="cuda")
+    ref = capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d)
+    capi.init()
+    out = torch.zeros_like(ref)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d, out=out, workspace=ws, options=opt)   # warm-up
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        capi.conv2d_add_partial_forward(xd, wd, L, pad, desc=d, out=out, workspace=ws, options=opt)
+    x2 = torch.rand_like(xd)
+    for i in range(3):
+        out.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), i
+        # eager work on the same workspace between the replays
+        other = capi.conv2d_add_partial_forward(x2, wd, L, pad, desc=d, workspace=ws, options=opt)
+        torch.cuda.synchronize()
+        assert not torch.equal(other, ref)
