@@ -70,7 +70,7 @@ struct GemmParams {
     long long c_split_stride;
     long long a_batch_stride, b_batch_stride, c_batch_stride;
     // EPI_EXP_TIMES_G: c[i][j] = g[i * c_out + (j % c_out)] * exp(-acc), g = upstream gradient stored [m][c_out]
-    // EPI_EXP_TIMES_G_PLANES (g_planes set, eight-wave kernel only): the same from the gradient as the caller
+    // EPI_EXP_TIMES_G_PLANES (g_planes set; whole tiles only): the same from the gradient as the caller
     // has it, [n][c_out][npos] with i = n * npos + position; npos a multiple of 32, g 16-byte aligned
     const float* __restrict__ g;
     int c_out, npos, g_planes;
@@ -2324,6 +2324,23 @@ inline int big_tile_nx(const GemmParams& q, int batch, bool b_along_k)
     return ok ? nx : 0;
 }
 
+// Tile extents of the 128 x 128 kernel.  A dimension of at most 192 whose last (or only) 128-tile would be at
+// most half full takes tiles of 64: the 2 x 2 wave arrangement would leave half of the waves of such a tile
+// without work (one dimension only, j first).
+inline void split_tile_extents(int I, int J, int& tile_i, int& tile_j)
+{
+    auto half_tiles = [](int n) { return n <= 3 * kTile / 2 && (n - 1) % kTile < kTile / 2; };
+    tile_j = half_tiles(J) ? kTile / 2 : kTile;
+    tile_i = tile_j == kTile && half_tiles(I) ? kTile / 2 : kTile;
+}
+// its tiles are all whole: what the epilogue that reads the upstream gradient in the caller's layout asks for
+inline bool split_tiles_whole(int I, int J)
+{
+    int ti, tj;
+    split_tile_extents(I, J, ti, tj);
+    return I % ti == 0 && J % tj == 0;
+}
+
 template <bool AK, bool BK, int EPI, bool VA = false, bool VB = false>
 int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
 {
@@ -2373,13 +2390,10 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
             return hipGetLastError() == hipSuccess ? GEO_SC_OK : GEO_SC_ERR_LAUNCH;
         }
     }
-    if (EPI == EPI_EXP_TIMES_G && q.g_planes) return GEO_SC_ERR_UNSUPPORTED;  // (the caller decides with big_tile_nx)
-    // A dimension of at most 192 whose last (or only) 128-tile would be at most half full takes tiles of
-    // 64: the 2 x 2 wave arrangement would leave half of the waves of such a tile without work (one
-    // dimension only, j first).
-    auto half_tiles = [](int n) { return n <= 3 * kTile / 2 && (n - 1) % kTile < kTile / 2; };
-    q.tile_j = half_tiles(q.J) ? kTile / 2 : kTile;
-    q.tile_i = q.tile_j == kTile && half_tiles(q.I) ? kTile / 2 : kTile;
+    // the gradient in the caller's layout: views with whole tiles only (the caller decides with big_tile_nx and
+    // split_tiles_whole)
+    if (EPI == EPI_EXP_TIMES_G && q.g_planes && !(VA && split_tiles_whole(q.I, q.J))) return GEO_SC_ERR_UNSUPPORTED;
+    split_tile_extents(q.I, q.J, q.tile_i, q.tile_j);
     q.ni = (q.I + q.tile_i - 1) / q.tile_i;
     q.nj = (q.J + q.tile_j - 1) / q.tile_j;
     q.nz = q.splits * batch;
@@ -2408,7 +2422,14 @@ int launch_gemm(const GemmParams& q0, int batch, hipStream_t s)
         hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, false, true>), grid, dim3(256), 0, s, q);
     } else if constexpr (VA) {
         if (!b_vec) return GEO_SC_ERR_UNSUPPORTED;
-        hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
+        if constexpr (EPI == EPI_EXP_TIMES_G) {
+            if (q.g_planes)
+                hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI_EXP_TIMES_G_PLANES, true>), grid, dim3(256), 0, s, q);
+            else
+                hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
+        } else {
+            hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI, true>), grid, dim3(256), 0, s, q);
+        }
     } else if constexpr (AK && BK) {
         hipLaunchKernelGGL((k_gemm_split<AK, BK, EPI>), grid, dim3(256), 0, s, q);
     } else {
@@ -2599,10 +2620,13 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
     if (fused || !view)
         hipLaunchKernelGGL(k_position_table, dim3(m_blocks), dim3(256), 0, s, pos_base, pos_arow, pos_bcol, M,
                            g.c_in, g.c_out, g.w_in, g.h_in, g.pad_w, g.pad_h, g.wo, g.ho);
-    // Where the first product takes the eight-wave kernel in every round, its epilogue reads the upstream
-    // gradient as it is (items of whole 32-position blocks, 16-byte aligned): no transposed copy.
+    // Where the first product reads col as a view and its tiles are whole (the eight-wave kernel in every round,
+    // or the 128 x 128 kernel), its epilogue reads the upstream gradient as it is (items of whole 32-position
+    // blocks, 16-byte aligned): no transposed copy.
+    // (the 128 x 128 kernel with full-width tiles only: with tiles of 64 columns the strided loads cost what the
+    // small transposed copy does)
     bool g_planes = !fused && view && (g.wo * g.ho) % 32 == 0 && ((uintptr_t)gy & 15) == 0;
-    if (g_planes) {
+    if (g_planes && !(split_tiles_whole(M, J) && J % kTile == 0)) {
         GemmParams t = {};
         t.I = M; t.J = J; t.K = K; t.splits = 1; t.k_per_split = K;
         for (int v0 = 0; v0 < G.n_groups; v0 += L.rows_per_chunk) {
