@@ -54,7 +54,7 @@ constexpr int kTile = 128;   // block tile in I and J
 constexpr int kChunk = 16;   // K per LDS stage
 constexpr int kLd = 132;     // LDS row stride in floats: rows stay 16-byte aligned for float4 stores
 
-enum Epilogue { EPI_STORE = 0, EPI_EXP_TIMES_G = 1, EPI_EXP_TIMES_G_PLANES = 2 };
+enum Epilogue { EPI_STORE = 0, EPI_EXP_TIMES_G = 1, EPI_EXP_TIMES_G_PLANES = 2, EPI_STORE_ITEMS = 3 };
 
 struct GemmParams {
     const float* __restrict__ a;
@@ -81,12 +81,17 @@ struct GemmParams {
     const long long* __restrict__ a_rows;
     long long a_rows_batch;
     int a_item, a_skip;
-    // B as a view of E shifted by whole image rows (kernels with VB; the input-gradient product summed over
-    // the sh_wk kernel rows u): chunk c of the k dimension holds the columns j = (c / sh_wk) * kChunk ... of kernel
-    // row u = c % sh_wk, and column i = (n, p, b) of B is row (n, p + sh_pad - u, b) of E (sh_j floats per row
-    // of E, ldb apart) where that output row exists, zero elsewhere (read from sh_zero).
+    // B as a view of E shifted by image rows and columns (kernels with VB; the input-gradient product summed
+    // over all sh_wk x sh_hk kernel taps (u, v) inside the GEMM): chunk c of the k dimension holds the columns
+    // j = (c / (sh_wk sh_hk)) * kChunk ... of tap t = c % (sh_wk sh_hk), u = t % sh_wk, v = t / sh_wk, and column
+    // i = (n, p, c) of B (an element of the input: sh_win rows of sh_hin) is row (n, p + sh_pad - u, c + sh_padh - v)
+    // of E_v (sh_j floats per row, ldb apart; E_v starts v * b_batch_stride into b) where that output position
+    // exists, zero elsewhere (read from sh_zero).
     const float* __restrict__ sh_zero;
-    int sh_j, sh_wo, sh_ho, sh_win, sh_pad, sh_wk;
+    int sh_j, sh_wo, sh_ho, sh_win, sh_hin, sh_pad, sh_padh, sh_wk, sh_hk;
+    // EPI_STORE_ITEMS: column j = (n, rest) of the result goes to c[(n * I + i) * c_plane + rest] (c_plane
+    // columns per item): the input gradient in the caller's layout (n, c_in, w_in, h_in)
+    int c_plane;
     // tile extent per workgroup in i and j: kTile, or kTile / 2 in at most one of them (set by
     // launch_gemm): the four waves then line up along the other dimension
     int tile_i, tile_j;
@@ -241,11 +246,24 @@ __device__ __forceinline__ void store_tile(const GemmParams& q, const floatx16 (
             const int x = (b0 + bb) / NYd, y = (b0 + bb) % NYd;
             const int j = jw + y * 32 + l32, ib = iw + x * 32 + 4 * lk;
             const bool j_ok = WHOLE || j < q.J;
+            if constexpr (EPI == EPI_STORE_ITEMS) {
+                // the lane's column is one element of one item: rows are c_plane apart
+                const int jc = j_ok ? j : 0;
+                const int item = jc / q.c_plane;
+                float* op = out + ((long long)item * q.I + ib) * q.c_plane + (jc - item * q.c_plane);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int di = 8 * (r >> 2) + (r & 3);
+                    if (WHOLE || (j_ok && ib + di < q.I)) op[(long long)di * q.c_plane] = acc[x][y][r];
+                }
+                continue;
+            }
             float* op = out + (long long)ib * q.ldc + j;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int di = 8 * (r >> 2) + (r & 3);
-                const float v = EPI != EPI_STORE ? gv[bb][r] * exp_neg(acc[x][y][r]) : acc[x][y][r];
+                const float v = (EPI == EPI_EXP_TIMES_G || EPI == EPI_EXP_TIMES_G_PLANES) ? gv[bb][r] * exp_neg(acc[x][y][r])
+                                                                                        : acc[x][y][r];
                 if (WHOLE)
                     op[(long long)di * q.ldc] = v;
                 else if (j_ok && ib + di < q.I)
@@ -600,56 +618,66 @@ struct ViewStager {
     }
 };
 
-// Stager of the B operand of the input-gradient product when it sums over the kernel rows inside the GEMM
-// (GemmParams::sh_*): the k dimension runs over chunks of kChunk columns j of E with the kernel row u as the
-// fast index, and for kernel row u the column (n, p, b) of B is the row (n, p + pad - u, b) of E.  I-major: a
-// thread keeps one column and eight consecutive j; from chunk to chunk it moves one image row up, and after the
-// last kernel row on to the next columns - so the rows of E that the kernel rows share are read in consecutive
-// chunks, while they are still in the CU's cache.  Columns whose output row does not exist for a u read a block
-// of zeros instead (no select on the loaded data, so nothing waits for the load).  sh_j is a multiple of
-// kChunk: there are no partial chunks.
+// Stager of the B operand of the input-gradient product when it sums over the kernel taps inside the GEMM
+// (GemmParams::sh_*): the k dimension runs over chunks of kChunk columns j of E with the tap (u, v) as the fast
+// index (u fastest), and for tap (u, v) the column (n, p, c) of B - an element of the input - is the row
+// (n, p + pad_w - u, c + pad_h - v) of E_v.  I-major: a thread keeps one column and eight consecutive j; from
+// chunk to chunk it moves one image row up, then one column left, and after the last tap on to the next columns
+// j - so the rows of E that the taps share are read in consecutive chunks, while they are still in the CU's
+// cache.  Columns whose output position does not exist for a tap read a block of zeros instead (no select on the
+// loaded data, so nothing waits for the load).  sh_j is a multiple of kChunk: there are no partial chunks.
 struct ShiftStager {
-    const float* e_rows;   // E of this batch member
+    const float* e0;       // E_0; E_v is group_stride floats further per v
     const float* zero;
     const float* p;
-    long long ld;
-    int j, u, prow, wo;  // j: this thread's first column of E in the current chunk; prow: p + pad
-    long long row0;                 // (n * wo + prow + pad) * ho + b: the row of E for u = 0
-    int half, ii, sh_j, ho, n_u;
+    long long ld, group_stride;
+    int j, u, v, prow, pcol, wo, ho;  // j: this thread's first column of E in the current chunk; prow = p + pad_w, pcol = c + pad_h
+    long long row0;                   // (n * wo + prow) * ho + pcol: the row of E for the tap (0, 0)
+    int half, ii, n_u, n_v;
 
     __device__ __forceinline__ void point()
     {
-        const int r = prow - u;  // prow already holds p + pad
-        p = (r >= 0 && r < wo) ? e_rows + (row0 - (long long)u * ho) * ld + j : zero;
+        const int r = prow - u, c = pcol - v;
+        p = (r >= 0 && r < wo && c >= 0 && c < ho)
+                ? e0 + (long long)v * group_stride + (row0 - (long long)u * ho - v) * ld + j
+                : zero;
     }
     __device__ __forceinline__ void init(const GemmParams& q, int batch, int j0, int k_begin, int Jn, int ii_, int half_)
     {
         ii = ii_;
         half = half_;
         n_u = q.sh_wk;
-        e_rows = q.b + batch * q.b_batch_stride;
+        n_v = q.sh_hk;
+        // all taps in one product (E_v chosen by the tap), or one product per kernel column (batch member) over
+        // its kernel rows (sh_hk = 1, sh_hin = ho, sh_padh = 0)
+        e0 = q.b + (n_v == 1 ? (long long)batch * q.b_batch_stride : 0);
+        group_stride = q.b_batch_stride;
         zero = q.sh_zero;
         ld = q.ldb;
-        sh_j = q.sh_j;
         wo = q.sh_wo;
         ho = q.sh_ho;
         const int m = min(j0 + ii, Jn - 1);
-        const int per_item = q.sh_win * q.sh_ho;
+        const int per_item = q.sh_win * q.sh_hin;
         const int n = m / per_item, rem = m - n * per_item;
-        const int pr = rem / q.sh_ho, b = rem - pr * q.sh_ho;
+        const int pr = rem / q.sh_hin, c = rem - pr * q.sh_hin;
         prow = pr + q.sh_pad;
-        row0 = ((long long)n * wo + prow) * ho + b;
-        // chunk c of the k dimension: kernel row c % w_k of the columns (c / w_k) * kChunk ...
-        const int chunk = k_begin / kChunk;
-        u = chunk % n_u;
-        j = (chunk / n_u) * kChunk + 8 * half;
+        pcol = c + q.sh_padh;
+        row0 = ((long long)n * wo + prow) * ho + pcol;
+        // chunk c of the k dimension: tap c % (w_k h_k) of the columns (c / (w_k h_k)) * kChunk ...
+        const int chunk = k_begin / kChunk, taps = n_u * n_v, t = chunk % taps;
+        u = t % n_u;
+        v = t / n_u;
+        j = (chunk / taps) * kChunk + 8 * half;
         point();
     }
     __device__ __forceinline__ void advance()
     {
         if (++u == n_u) {
             u = 0;
-            j += kChunk;
+            if (++v == n_v) {
+                v = 0;
+                j += kChunk;
+            }
         }
         point();
     }
@@ -1584,11 +1612,14 @@ __global__ __launch_bounds__(256) void k_reduce_wgrad_tiled(const float* __restr
 
 // What a round of GEMM launches needs beforehand, in one launch (grid: blocks x groups of the round):
 //  * the weight operands wcat / wd of k_weight_operands, for group g0 + blockIdx.y;
-//  * with dx_rows, in wd's place, the A operand of the input-gradient product that sums the kernel rows inside
-//    the GEMM (y accumulation: group = kernel column v, members (ci, u)): wdx[g][k][ci] = wd[g][j][(ci, u)], i.e.
-//    clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one, with the
-//    kernel row as the fast index over chunks of kChunk columns, k = ((j / kChunk) * w_k + u) * kChunk + j % kChunk:
-//    consecutive chunks of the product then read the same columns of E one image row apart (ShiftStager);
+//  * with dx_rows, in wd's place, the A operand of the input-gradient product that sums kernel taps inside
+//    the GEMM (y accumulation: group = kernel column v, members (ci, u)): wdx[k][ci] = wd[v][j][(ci, u)], i.e.
+//    clamp(w, 0, 100) for the positive rail j < c_out and clamp(w, -100, 0) for the negative one, with the tap
+//    as the fast index over chunks of kChunk columns - dx_rows = 1: one operand per group,
+//    k = ((j / kChunk) * w_k + u) * kChunk + j % kChunk (the kernel rows inside the product); dx_rows = 2: one
+//    operand for all groups, k = (((j / kChunk) * h_k + v) * w_k + u) * kChunk + j % kChunk (all taps inside):
+//    consecutive chunks of the product then read the same columns of E one image row, then one image column
+//    apart (ShiftStager);
 //  * from the blocks of the round's first group: view_rows[g][k], where row k of group g's col starts in the
 //    planes of k_shift_planes (elements), for every group; and 64 zeros for the shifted view of E (a store
 //    rather than a memset, so that a caller may capture the launch sequence in a graph).
@@ -1599,7 +1630,7 @@ struct PrepParams {
     int g0, c_out;
     Groups G;
     size_t g_stride;
-    int dx_rows;            // wd holds the wdx operand (y accumulation: c_in, w_k, h_k from G)
+    int dx_rows;            // wd holds the wdx operand (y accumulation: c_in, w_k, h_k from G): 1 per group, 2 one for all
     long long* view_rows;   // null: no view
     int view_groups, view_k_pad, ho;
     long long plane;
@@ -1625,13 +1656,19 @@ __global__ __launch_bounds__(256) void k_bwd_prep(PrepParams q)
         }
     }
     if (q.dx_rows) {
+        // this block row's kernel column g: its own operand, or its part of the one operand (which starts where
+        // the round's wd starts)
         const int J = 2 * c_out, c_in = q.G.c_in, w_k = q.G.w_k, h_k = q.G.h_k;
         for (int e = blockIdx.x * 256 + threadIdx.x; e < w_k * J * c_in; e += gridDim.x * 256) {
             const int ci = e % c_in, r = e / c_in;
-            const int chunk = r / kChunk, u = chunk % w_k, j = (chunk / w_k) * kChunk + r % kChunk;
+            const int chunk = r / kChunk, u = chunk % w_k, jc = chunk / w_k, jj = r % kChunk, j = jc * kChunk + jj;
             const int co = j >= c_out ? j - c_out : j;
             const float wv = q.w[(((size_t)co * c_in + ci) * w_k + u) * h_k + g];
-            wdg[e] = j < c_out ? fminf(fmaxf(wv, 0.0f), 100.0f) : fminf(fmaxf(wv, -100.0f), 0.0f);
+            const float val = j < c_out ? fminf(fmaxf(wv, 0.0f), 100.0f) : fminf(fmaxf(wv, -100.0f), 0.0f);
+            if (q.dx_rows == 2)
+                q.wd[((((size_t)jc * h_k + g) * w_k + u) * kChunk + jj) * c_in + ci] = val;
+            else
+                wdg[e] = val;
         }
     }
     if (blockIdx.y == 0) {
@@ -2456,6 +2493,7 @@ struct BwdLayout {
     int rows_per_chunk;  // add groups processed by one round of launches
     int dcol_slices;     // partial dcol arrays per round (column blocks of the fused kernel), rows_per_chunk * col_v apart
     bool dx_rows;        // the input-gradient GEMM sums the kernel rows itself (E read as a view shifted by image rows)
+    bool dx_taps;        // it sums all kernel taps and writes dL/dx itself (E read as a view shifted by rows and columns)
     size_t off_zero;     // a block of zeros for that view
     bool view_col;       // the GEMMs read col as a view of the shifted input planes (k_shift_planes) kept in col's space
     int view_k_pad;      // entries per group of the view's row table
@@ -2557,6 +2595,18 @@ BwdLayout bwd_layout(const Geometry& g, int groups_per_round)
                 (2 * g.c_out) % kChunk == 0 && rows == (size_t)b.G.n_groups &&
                 (size_t)g.h_k * g.c_in * g.n * g.w_in * g.ho <= rows * b.col_v &&
                 (long long)g.n * g.w_in * g.ho < 0x7fffffffLL && (long long)g.w_k * 2 * g.c_out < 0x7fffffffLL;
+    // all kernel taps summed inside that GEMM, which then writes dL/dx itself (no per-column results, no pass that
+    // adds them): the same without the conditions of that pass, where the result alone has tiles for the GPU
+    // (a product per kernel column has h_k times as many)
+    {
+        int ti, tj;
+        const long long m2 = (long long)g.n * g.w_in * g.h_in;
+        split_tile_extents(g.c_in, m2 > 0x7fffffffLL ? 0x7fffffff : (int)m2, ti, tj);
+        const long long tiles = (long long)((g.c_in + ti - 1) / ti) * ((m2 + tj - 1) / tj);
+        b.dx_taps = !b.fused_k && g.mode == GEO_SC_ACC_Y && (2 * g.c_out) % kChunk == 0 &&
+                    rows == (size_t)b.G.n_groups && m2 < 0x7fffffffLL &&
+                    (long long)g.w_k * g.h_k * 2 * g.c_out < 0x7fffffffLL && tiles >= 2 * kBigWorkgroups;
+    }
     size_t o = 0;
     b.off_col = o;  o += align256(sizeof(float) * rows * col_alloc);
     b.off_e = o;    o += align256(sizeof(float) * rows * e_alloc);
@@ -2743,12 +2793,13 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
                                dim3(m_blocks > 1024 ? 1024 : m_blocks, (K + kIm2colMembers - 1) / kIm2colMembers, nv),
                                dim3(256), 0, s, x, col, pos_base, pos_arow, pos_bcol, v0, M, G, g.w_in, g.h_in, L.col_v);
         }
-        const bool dx_rows = gx && L.dx_rows && ((uintptr_t)gx & 15) == 0;
+        const bool dx_taps = gx && L.dx_taps;
+        const bool dx_rows = dx_taps || (gx && L.dx_rows && ((uintptr_t)gx & 15) == 0);
         {
             // weight operands of the round's groups; with the first round the view's row table and the block of zeros
             PrepParams pp = {};
             pp.w = w; pp.wcat = wcat; pp.wd = wd; pp.g0 = v0; pp.c_out = g.c_out; pp.G = G; pp.g_stride = L.w_v;
-            pp.dx_rows = dx_rows ? 1 : 0;
+            pp.dx_rows = dx_taps ? 2 : dx_rows ? 1 : 0;
             if (v0 == 0 && view) {
                 pp.view_rows = view_rows; pp.view_groups = G.n_groups; pp.view_k_pad = L.view_k_pad; pp.ho = g.ho;
                 pp.plane = (long long)g.n * (g.w_in + 2 * g.pad_w) * g.ho;
@@ -2789,6 +2840,25 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
                                L.splits, g.c_out, G, L.part_v);
         }
         if (!gx) continue;
+        if (dx_taps) {
+            // gx[n][ci][(p, c)] = sum_(u, v, j) wdx[(j, v, u)][ci] * E_v[(n, p + pad_w - u, c + pad_h - v)][j]: every
+            // kernel tap summed inside one GEMM (nine times the k of the product per tap, a ninth of its output,
+            // stored in the caller's layout); the operand wdx and the block of zeros come from k_bwd_prep
+            float* zero = (float*)(ws + L.off_zero);
+            const int k9 = g.w_k * g.h_k * J;
+            const long long m2 = (long long)g.n * g.w_in * g.h_in;
+            GemmParams q3 = {};
+            q3.a = wd; q3.b = e; q3.c = gx;
+            q3.I = g.c_in; q3.J = (int)m2; q3.K = k9;
+            q3.lda = g.c_in; q3.ldb = J; q3.ldc = m2;
+            q3.splits = 1; q3.k_per_split = k9; q3.c_split_stride = 0;
+            q3.a_batch_stride = 0; q3.b_batch_stride = (long long)L.e_v; q3.c_batch_stride = 0;
+            q3.sh_zero = zero; q3.sh_j = J; q3.sh_wo = g.wo; q3.sh_ho = g.ho; q3.sh_win = g.w_in; q3.sh_hin = g.h_in;
+            q3.sh_pad = g.pad_w; q3.sh_padh = g.pad_h; q3.sh_wk = g.w_k; q3.sh_hk = g.h_k;
+            q3.c_plane = g.w_in * g.h_in;
+            if ((rc = launch_gemm<true, false, EPI_STORE_ITEMS, false, true>(q3, 1, s)) != GEO_SC_OK) return rc;
+            continue;
+        }
         if (dx_rows) {
             // d[v][ci][(n, p, b)] = sum_(u, j) wd_v[j][(ci, u)] * E_v[(n, p + pad - u, b)][j]: the kernel rows
             // summed inside the GEMM (three times the k of the product per (ci, u), a third of its rows and of
@@ -2804,8 +2874,8 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
             q3.splits = 1; q3.k_per_split = k3; q3.c_split_stride = 0;
             q3.a_batch_stride = (long long)L.w_v; q3.b_batch_stride = (long long)L.e_v;
             q3.c_batch_stride = (long long)g.c_in * m2;
-            q3.sh_zero = zero; q3.sh_j = J; q3.sh_wo = g.wo; q3.sh_ho = g.ho; q3.sh_win = g.w_in; q3.sh_pad = g.pad_w;
-            q3.sh_wk = g.w_k;
+            q3.sh_zero = zero; q3.sh_j = J; q3.sh_wo = g.wo; q3.sh_ho = g.ho; q3.sh_win = g.w_in; q3.sh_hin = g.ho;
+            q3.sh_pad = g.pad_w; q3.sh_padh = 0; q3.sh_wk = g.w_k; q3.sh_hk = 1;
             if ((rc = launch_gemm<true, false, EPI_STORE, false, true>(q3, nv, s)) != GEO_SC_OK) return rc;
             const long long quads = (long long)g.n * g.c_in * g.w_in * g.h_in / 4;
             hipLaunchKernelGGL(k_shift_sum_v4, dim3(grid1d(quads)), dim3(256), 0, s, dcol, gx, quads, g.n, g.c_in, g.w_in,

@@ -114,6 +114,34 @@ def test_backward_through_the_gemm_kernels(capi, shape_x, shape_w, pad, scale):
     check("grad_w", gw, rw)
 
 
+@pytest.mark.parametrize("shape_x,shape_w,pad", [
+    ((40, 12, 40, 44), (8, 12, 3, 5), (1, 1)),     # 3 x 5 taps, output 40 x 42 from 40 x 44: rows and columns that do not exist for a tap, a ragged last tile
+    ((70, 40, 31, 31), (16, 40, 2, 2), (0, 0)),    # even kernel, no padding, odd extents
+    ((33, 16, 64, 32), (24, 16, 5, 1), (2, 0)),    # one kernel column: five kernel rows only
+])
+def test_input_gradient_with_all_kernel_taps_inside_the_gemm(capi, shape_x, shape_w, pad):
+    """Inputs of at least 512 tiles of 128 positions: the input-gradient product sums over every kernel tap and
+    writes dL/dx in the caller's layout itself (no per-column results, no pass that adds them).  Against float64
+    autograd over the surrogate on the GPU."""
+    from oracle import surrogate
+    x, w = wl.make_inputs(shape_x, shape_w, "kaiming", seed=shape_x[1])
+    w = (w * 3).contiguous()
+    w.view(-1)[::5] = 0.0
+    xd, wd = x.cuda(), w.cuda()
+    d = capi.make_desc(x.shape, w.shape, 128, pad)
+    g = torch.randn(capi.output_shape(d), generator=torch.Generator().manual_seed(4)).cuda()
+    gx, gw = capi.conv2d_add_partial_backward(xd, wd, g, 128, pad)
+    xr = xd.clone().double().requires_grad_(True)
+    wr = wd.clone().double().requires_grad_(True)
+    xp = torch.nn.functional.pad(xr, (pad[0], pad[0], pad[1], pad[1]))
+    p, n = surrogate.surrogate_rails(xp, wr.clamp(0, 100), -(wr.clamp(-100, 0)))
+    (p - n).backward(g.double())
+    check("grad_x", gx, xr.grad)
+    check("grad_w", gw, wr.grad)
+    gx_only, none = capi.conv2d_add_partial_backward(xd, wd, g, 128, pad, need_grad_w=False)
+    assert none is None and torch.equal(gx_only, gx)
+
+
 def test_backward_headline_shape_against_torch_fp32_and_properties(capi):
     """128->128 3x3 at 16x16, batch 256: against torch's own fp32 autograd over the surrogate
     (the float64 oracle on the CPU would take minutes), plus linearity in grad_y."""
