@@ -2610,7 +2610,8 @@ BwdLayout bwd_layout(const Geometry& g, int groups_per_round)
     size_t o = 0;
     b.off_col = o;  o += align256(sizeof(float) * rows * col_alloc);
     b.off_e = o;    o += align256(sizeof(float) * rows * e_alloc);
-    b.off_dcol = o; o += align256(sizeof(float) * rows * b.col_v * b.dcol_slices);
+    // (no per-group input gradients where the product over all taps writes dL/dx itself)
+    b.off_dcol = o; o += b.dx_taps ? 0 : align256(sizeof(float) * rows * b.col_v * b.dcol_slices);
     b.off_part = o; o += align256(sizeof(float) * rows * b.part_v);
     b.off_wcat = o; o += align256(sizeof(float) * rows * b.w_v);
     b.off_wd = o;   o += align256(sizeof(float) * rows * b.w_v);
