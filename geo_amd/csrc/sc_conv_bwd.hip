@@ -2604,7 +2604,7 @@ BwdLayout bwd_layout(const Geometry& g, int groups_per_round)
         split_tile_extents(g.c_in, m2 > 0x7fffffffLL ? 0x7fffffff : (int)m2, ti, tj);
         const long long tiles = (long long)((g.c_in + ti - 1) / ti) * ((m2 + tj - 1) / tj);
         b.dx_taps = !b.fused_k && g.mode == GEO_SC_ACC_Y && (2 * g.c_out) % kChunk == 0 &&
-                    rows == (size_t)b.G.n_groups && m2 < 0x7fffffffLL &&
+                    rows == (size_t)b.G.n_groups && m2 < 0x7fff0000LL &&
                     (long long)g.w_k * g.h_k * 2 * g.c_out < 0x7fffffffLL && tiles >= 2 * kBigWorkgroups;
     }
     size_t o = 0;
