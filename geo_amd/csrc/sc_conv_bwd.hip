@@ -2843,8 +2843,8 @@ int launch_conv_backward(const Geometry& g, int groups_per_round, const float* x
         if (!gx) continue;
         if (dx_taps) {
             // gx[n][ci][(p, c)] = sum_(u, v, j) wdx[(j, v, u)][ci] * E_v[(n, p + pad_w - u, c + pad_h - v)][j]: every
-            // kernel tap summed inside one GEMM (nine times the k of the product per tap, a ninth of its output,
-            // stored in the caller's layout); the operand wdx and the block of zeros come from k_bwd_prep
+            // kernel tap summed inside one GEMM (w_k h_k times the k of the product per tap, one output instead of one
+            // per tap, stored in the caller's layout); the operand wdx and the block of zeros come from k_bwd_prep
             float* zero = (float*)(ws + L.off_zero);
             const int k9 = g.w_k * g.h_k * J;
             const long long m2 = (long long)g.n * g.w_in * g.h_in;
